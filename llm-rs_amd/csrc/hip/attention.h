@@ -1,0 +1,18 @@
+// Causal attention of a step's query tokens over the paged cache.
+#pragma once
+#include "common.h"
+
+struct AttnArgs {
+    int n_tokens, n_heads, n_kv_heads, head_dim;
+    int page_size, table_width, num_pages;
+    int q_stride, out_stride;  // elements between tokens
+    int window;                // 0: all keys up to the query's position
+    float scale;
+};
+
+// The matrix-core kernels (attention_mfma.hip).  Return 1 when they took the
+// call, 0 when its shape is not theirs, -1 on error.
+int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, const bf16* k_cache, const bf16* v_cache,
+                              const int* block_table, const int* token_entry, const int* positions,
+                              const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
+                              size_t scratch_bytes, const AttnArgs& a);

@@ -1,0 +1,71 @@
+// Token embedding into the 32-bit residual stream, and RMSNorm out of it.
+#include "common.h"
+
+// out[t, :] = float(table[tokens[t], :])   (reference: embed_batch_*, shaders/ops.metal:878-915)
+template <class T>
+__global__ void embed_rows_kernel(float* __restrict__ out, const T* __restrict__ table,
+                                  const int* __restrict__ tokens, int D, int V) {
+    int t = blockIdx.x;
+    int row = tokens[t];
+    row = row < 0 ? 0 : (row >= V ? V - 1 : row);  // the host has checked ids; never read outside the table
+    const T* src = table + (size_t)row * D;
+    float* dst = out + (size_t)t * D;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = to_f32(src[d]);
+}
+
+// One block per row: ss = sum x^2 in 32-bit, inv = 1/sqrt(ss/D + eps),
+// y = (x * inv) * w, one rounding to the output type.  The weight multiplies
+// directly (no 1+w).  Reference: rms_norm_batch, shaders/ops.metal:970-1003.
+// The sum's order depends on D and the block size only, never on the row or batch.
+template <class T>
+__global__ void rmsnorm_rows_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                    const float* __restrict__ w, const int* __restrict__ rows, int D, float eps) {
+    __shared__ float partial[16];
+    int r = rows ? rows[blockIdx.x] : blockIdx.x;
+    const float* src = x + (size_t)r * D;
+    float ss = 0.0f;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float v = src[d];
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    if ((threadIdx.x & 63) == 0) partial[wave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+    for (int i = 0; i < nwaves; ++i) total += partial[i];
+    float inv = 1.0f / sqrtf(total / (float)D + eps);
+    T* dst = out + (size_t)blockIdx.x * D;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = from_f32<T>(src[d] * inv * w[d]);
+}
+
+extern "C" int llmrs_embed_rows(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens,
+                                int n_tokens, int D, int V) {
+    LLMRS_REQUIRE(n_tokens >= 0 && D > 0 && V > 0, "embed_rows: bad sizes T=%d D=%d V=%d", n_tokens, D, V);
+    if (n_tokens == 0) return 0;
+    if (dtype == LLMRS_F32)
+        embed_rows_kernel<float><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, tokens, D, V);
+    else if (dtype == LLMRS_BF16)
+        embed_rows_kernel<bf16><<<n_tokens, 256, 0, stream>>>(out, (const bf16*)table, tokens, D, V);
+    else
+        return llmrs_fail("embed_rows: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("embed_rows");
+    return 0;
+}
+
+// rows == nullptr: row i of x -> row i of out; else row rows[i] of x -> row i of out.
+extern "C" int llmrs_rmsnorm(hipStream_t stream, int dtype, void* out, const float* x, const float* weight,
+                             const int* rows, int n_rows, int D, float eps) {
+    LLMRS_REQUIRE(n_rows >= 0 && D > 0, "rmsnorm: bad sizes rows=%d D=%d", n_rows, D);
+    LLMRS_REQUIRE(eps > 0.0f, "rmsnorm: eps must be positive, got %g", eps);
+    if (n_rows == 0) return 0;
+    int threads = D >= 2048 ? 1024 : 256;
+    if (dtype == LLMRS_F32)
+        rmsnorm_rows_kernel<float><<<n_rows, threads, 0, stream>>>((float*)out, x, weight, rows, D, eps);
+    else if (dtype == LLMRS_BF16)
+        rmsnorm_rows_kernel<bf16><<<n_rows, threads, 0, stream>>>((bf16*)out, x, weight, rows, D, eps);
+    else
+        return llmrs_fail("rmsnorm: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}

@@ -1,0 +1,94 @@
+// The plain product: 64x64 tiles through LDS, 32-bit FMA, k in ascending order.
+// It is the whole 32-bit path (no matrix-core mode rounds its inputs) and the
+// bfloat16 fallback for shapes the MFMA kernels refuse.  The order of the sum for
+// an output depends on K only, so a row's result does not depend on M, on the
+// row's place in the batch or on its tile.
+// Reference: gemm_f32 accumulates in 32-bit the same way (shaders/ops.metal:1053-1079).
+#include "gemm.h"
+
+#define TILE 64
+#define TILE_K 16
+
+template <class T>
+__global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ A, int lda,
+                                                          const T* __restrict__ W, void* __restrict__ out, int ldc,
+                                                          int M, int N, int K, int epi) {
+    __shared__ float As[TILE_K][TILE + 4];
+    __shared__ float Ws[TILE_K][TILE + 4];
+    int tid = threadIdx.x;
+    int m0 = blockIdx.y * TILE, n0 = blockIdx.x * TILE;
+    int ty = tid / 16, tx = tid % 16;
+    int lrow = tid / 4, lk = (tid % 4) * 4;  // this thread stages 4 k-values of one row of each tile
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += TILE_K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int k = k0 + lk + i;
+            int am = m0 + lrow, wn = n0 + lrow;
+            As[lk + i][lrow] = (am < M && k < K) ? to_f32(A[(size_t)am * lda + k]) : 0.0f;
+            Ws[lk + i][lrow] = (wn < N && k < K) ? to_f32(W[(size_t)wn * K + k]) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TILE_K; ++kk) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+        if (epi == LLMRS_EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                int n = n0 + tx * 4 + j;
+                if (n + 1 < N) ((T*)out)[(size_t)m * ldc + n / 2] = from_f32<T>(silu_f32(acc[i][j]) * acc[i][j + 1]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int n = n0 + tx * 4 + j;
+                if (n < N) epilogue_store<T>(epi, out, ldc, m, n, acc[i][j]);
+            }
+        }
+    }
+}
+
+// A: [M, K] with row stride lda; W: [N, K] dense; out: row stride ldc (elements of
+// its own type; for SWIGLU the output has N/2 columns).
+extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
+                          int M, int N, int K, int epi, int allow_mfma) {
+    LLMRS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    LLMRS_REQUIRE(lda >= K, "gemm: row stride %d of A is shorter than K=%d", lda, K);
+    LLMRS_REQUIRE(epi >= 0 && epi <= 3, "gemm: unknown epilogue %d", epi);
+    if (epi == LLMRS_EPI_SWIGLU) {
+        LLMRS_REQUIRE(N % 2 == 0, "gemm: the gate/up epilogue needs an even N, got %d", N);
+        LLMRS_REQUIRE(ldc >= N / 2, "gemm: row stride %d of out is shorter than N/2=%d", ldc, N / 2);
+    } else {
+        LLMRS_REQUIRE(ldc >= N, "gemm: row stride %d of out is shorter than N=%d", ldc, N);
+    }
+    if (M == 0) return 0;
+    if (dtype == LLMRS_BF16 && allow_mfma) {
+        int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
+        if (took != 0) return took < 0 ? -1 : 0;
+    }
+    dim3 grid(ceil_div(N, TILE), ceil_div(M, TILE));
+    LLMRS_REQUIRE(grid.y <= 65535, "gemm: M=%d is too large for one launch", M);
+    if (dtype == LLMRS_F32)
+        gemm_simple_kernel<float><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, out, ldc, M, N, K, epi);
+    else if (dtype == LLMRS_BF16)
+        gemm_simple_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
+    else
+        return llmrs_fail("gemm: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("gemm");
+    return 0;
+}

@@ -1,0 +1,97 @@
+// Rotary position encoding of q and k, and the write of k and v into the paged
+// cache, in one pass over the projection's output.
+//
+// Rotation as the reference does it (rope_batch, shaders/ops.metal:1011-1042):
+// angle = float(pos) * freq_i, (a, b) <- (a cos - b sin, a sin + b cos), all in
+// 32-bit, one rounding on the way out.  freq_i comes from a table the host makes
+// once (so that scaling of the frequencies is the host's matter); the pair is
+// (i, i + rot/2) ("split half") or (2i, 2i+1) ("interleaved")
+// (src/tensor/mod.rs:133-139).  Features past rotary_dim pass unchanged.
+// The cache write replaces scatter_kv (shaders/ops.metal:841-853).
+#include "cache_layout.h"
+#include "common.h"
+
+struct RopeKvArgs {
+    int n_tokens, n_heads, n_kv_heads, head_dim;
+    int rotary_dim, interleaved;
+    int page_size, write_kv, num_pages;
+    int row_stride;  // elements between tokens in qkv
+};
+
+template <class T>
+__global__ void rope_kv_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                               const int* __restrict__ slot_map, const float* __restrict__ inv_freq,
+                               T* __restrict__ k_cache, T* __restrict__ v_cache, RopeKvArgs a) {
+    int half = a.head_dim / 2;
+    int pairs_per_token = (a.n_heads + 2 * a.n_kv_heads) * half;
+    int t = blockIdx.x;
+    int idx = blockIdx.y * blockDim.x + threadIdx.x;
+    if (idx >= pairs_per_token) return;
+    int head = idx / half, i = idx % half;
+    T* row = qkv + (size_t)t * a.row_stride + (size_t)head * a.head_dim;
+    bool is_q = head < a.n_heads;
+    bool is_k = !is_q && head < a.n_heads + a.n_kv_heads;
+    if (!is_q && !a.write_kv) return;
+    int da, db;  // the two features this thread owns
+    bool rotate = !(!is_q && !is_k) && i < a.rotary_dim / 2;
+    if (i < a.rotary_dim / 2) {
+        if (a.interleaved) { da = 2 * i; db = 2 * i + 1; }
+        else { da = i; db = i + a.rotary_dim / 2; }
+    } else {
+        da = a.rotary_dim + 2 * (i - a.rotary_dim / 2);
+        db = da + 1;
+    }
+    float xa = to_f32(row[da]), xb = to_f32(row[db]);
+    if (rotate) {
+        float angle = (float)positions[t] * inv_freq[i];
+        float s, c;
+        sincosf(angle, &s, &c);
+        float ya = xa * c - xb * s;
+        float yb = xa * s + xb * c;
+        xa = ya; xb = yb;
+    }
+    if (is_q) {
+        row[da] = from_f32<T>(xa);
+        row[db] = from_f32<T>(xb);
+        return;
+    }
+    int slot = slot_map[t];
+    if (slot < 0 || slot >= a.num_pages * a.page_size) return;  // never write outside the cache
+    int page = slot / a.page_size, off = slot % a.page_size;
+    if (is_k) {
+        int kvh = head - a.n_heads;
+        k_cache[k_cache_index(page, kvh, off, da, a.n_kv_heads, a.page_size, a.head_dim)] = from_f32<T>(xa);
+        k_cache[k_cache_index(page, kvh, off, db, a.n_kv_heads, a.page_size, a.head_dim)] = from_f32<T>(xb);
+    } else {
+        int kvh = head - a.n_heads - a.n_kv_heads;
+        v_cache[v_cache_index(page, kvh, off, da, a.n_kv_heads, a.page_size, a.head_dim)] = from_f32<T>(xa);
+        v_cache[v_cache_index(page, kvh, off, db, a.n_kv_heads, a.page_size, a.head_dim)] = from_f32<T>(xb);
+    }
+}
+
+// qkv: [n_tokens, row_stride], a row is q heads, then k heads, then v heads.
+// q is rotated in place; k is rotated and written to k_cache; v is copied to
+// v_cache.  Slots outside [0, num_pages * page_size) are skipped.
+extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int row_stride, const int* positions,
+                                   const int* slot_map, const float* inv_freq, int rotary_dim, int interleaved,
+                                   void* k_cache, void* v_cache, int n_tokens, int n_heads, int n_kv_heads,
+                                   int head_dim, int page_size, int num_pages, int write_kv) {
+    LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope_kv_write: bad sizes");
+    LLMRS_REQUIRE(head_dim % 2 == 0, "rope_kv_write: head_dim %d is odd", head_dim);
+    LLMRS_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+                  "rope_kv_write: rotary_dim %d does not fit head_dim %d", rotary_dim, head_dim);
+    LLMRS_REQUIRE(row_stride >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_kv_write: row stride %d too short", row_stride);
+    LLMRS_REQUIRE(page_size > 0, "rope_kv_write: page_size %d", page_size);
+    if (n_tokens == 0) return 0;
+    RopeKvArgs a{n_tokens, n_heads, n_kv_heads, head_dim, rotary_dim, interleaved, page_size, write_kv, num_pages, row_stride};
+    int pairs = (n_heads + 2 * n_kv_heads) * (head_dim / 2);
+    dim3 grid(n_tokens, ceil_div(pairs, 256));
+    if (dtype == LLMRS_F32)
+        rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, positions, slot_map, inv_freq, (float*)k_cache, (float*)v_cache, a);
+    else if (dtype == LLMRS_BF16)
+        rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
+    else
+        return llmrs_fail("rope_kv_write: unknown dtype %d", dtype);
+    LLMRS_LAUNCH_CHECK("rope_kv_write");
+    return 0;
+}

@@ -1,0 +1,167 @@
+#include "scheduler.h"
+
+#include <algorithm>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+
+namespace llmrs {
+
+Scheduler::Scheduler(CacheManager& cache, int token_budget, int max_chunk, int max_positions)
+    : cache_(cache), budget_(token_budget), max_chunk_(max_chunk > 0 ? max_chunk : token_budget),
+      max_positions_(max_positions), requests_(cache.max_requests()) {
+    if (token_budget <= 0) throw std::invalid_argument("token budget must be positive");
+}
+
+int Scheduler::add(const int32_t* prompt, int n_prompt, int max_new, const SamplingParams& sp,
+                   const int32_t* stop, int n_stop) {
+    if (n_prompt <= 0) throw std::invalid_argument("a request needs at least one prompt token");
+    if (max_new <= 0) throw std::invalid_argument("max_new_tokens must be positive");
+    int total = n_prompt + max_new;
+    if (total > max_positions_)
+        throw std::invalid_argument("request needs " + std::to_string(total) + " positions, the model has " +
+                                    std::to_string(max_positions_));
+    // The last step of a request alone in the pool: all it has computed plus one
+    // portion.  If even that exceeds a pool, no schedule can ever finish it.
+    for (int g = 0; g < cache_.num_groups(); ++g) {
+        int worst = 0;
+        if (cache_.group(g).window == 0) {
+            worst = cache_.pages_needed(g, 0, total - 1);
+        } else {
+            int chunk = std::min(max_chunk_, budget_);
+            for (int start = 0; start < total - 1; start += chunk)
+                worst = std::max(worst, cache_.pages_needed(g, start, std::min(chunk, total - 1 - start)));
+        }
+        if (worst > cache_.pages_total(g))
+            throw std::invalid_argument("request needs " + std::to_string(worst) + " pages of cache group " +
+                                        std::to_string(g) + ", the pool has " + std::to_string(cache_.pages_total(g)));
+    }
+    int slot = cache_.acquire_slot();
+    if (slot < 0) return -1;
+    Request& r = requests_[slot];
+    r = Request();
+    r.tokens.assign(prompt, prompt + n_prompt);
+    r.prompt_len = n_prompt;
+    r.max_new = max_new;
+    r.stop.assign(stop, stop + n_stop);
+    r.sampling = sp;
+    r.rng = Xorshift64(sp.seed);
+    r.phase = Phase::Waiting;
+    waiting_.push_back(slot);
+    return slot;
+}
+
+int Scheduler::portion(const Request& r, int budget) const {
+    int needed = (int)r.tokens.size() - r.computed;
+    return std::min({needed, budget, max_chunk_});
+}
+
+void Scheduler::preempt_last() {
+    int slot = running_.back();
+    running_.pop_back();
+    Request& r = requests_[slot];
+    cache_.release_pages(slot);
+    r.computed = 0;
+    r.phase = Phase::Waiting;
+    ++r.preemptions;
+    ++preemptions_;
+    waiting_.push_front(slot);
+}
+
+const std::vector<PlannedEntry>& Scheduler::plan() {
+    for (;;) {
+        plan_.clear();
+        int budget = budget_;
+        bool starved = false;
+        // 1. running requests, in admission order (scheduler.rs:42-54)
+        for (int slot : running_) {
+            if (budget == 0) break;
+            Request& r = requests_[slot];
+            int n = portion(r, budget);
+            if (n <= 0) continue;
+            if (!cache_.ensure(slot, r.computed, n)) {
+                starved = true;
+                continue;  // no pages now; it tries again in the next step
+            }
+            plan_.push_back({{slot, r.computed, n}, r.computed + n == (int)r.tokens.size()});
+            budget -= n;
+        }
+        // 2. waiting requests, first in first out (scheduler.rs:56-73)
+        while (budget > 0 && !waiting_.empty()) {
+            int slot = waiting_.front();
+            Request& r = requests_[slot];
+            int n = portion(r, budget);
+            if (!cache_.ensure(slot, r.computed, n)) {
+                starved = true;
+                break;  // head of the line waits, and so do those behind it
+            }
+            waiting_.pop_front();
+            r.phase = Phase::Running;
+            running_.push_back(slot);
+            plan_.push_back({{slot, r.computed, n}, r.computed + n == (int)r.tokens.size()});
+            budget -= n;
+        }
+        if (!plan_.empty() || !starved) return plan_;
+        // Nothing can advance and pages are the reason.  With nobody running, the
+        // head of the queue found an empty pool too small: add() rules that out.
+        if (running_.empty())
+            throw std::logic_error("a waiting request does not fit an empty cache pool");
+        preempt_last();
+    }
+}
+
+void Scheduler::plan_tokens(std::vector<int32_t>& tokens, std::vector<int32_t>& want_rows,
+                            std::vector<int32_t>& sampling_words) {
+    tokens.clear();
+    want_rows.clear();
+    sampling_words.clear();
+    for (const auto& p : plan_) {
+        Request& r = requests_[p.entry.slot];
+        tokens.insert(tokens.end(), r.tokens.begin() + p.entry.start, r.tokens.begin() + p.entry.start + p.entry.count);
+        if (!p.samples) continue;
+        want_rows.push_back((int32_t)tokens.size() - 1);
+        float u = r.sampling.temperature > 0.0f ? r.rng.next_f32() : 0.0f;
+        int32_t w[4];
+        std::memcpy(&w[0], &u, 4);
+        std::memcpy(&w[1], &r.sampling.temperature, 4);
+        w[2] = r.sampling.top_k;
+        std::memcpy(&w[3], &r.sampling.top_p, 4);
+        sampling_words.insert(sampling_words.end(), w, w + 4);
+    }
+}
+
+std::vector<int> Scheduler::commit(const int32_t* sampled, int n_sampled) {
+    std::vector<int> finished;
+    int i = 0;
+    for (const auto& p : plan_) {
+        Request& r = requests_[p.entry.slot];
+        r.computed += p.entry.count;
+        if (!p.samples) continue;  // a portion of a prompt: nothing to sample yet (engine.rs:209)
+        if (i >= n_sampled) throw std::invalid_argument("fewer sampled tokens than entries that sample");
+        int32_t token = sampled[i++];
+        if (std::find(r.stop.begin(), r.stop.end(), token) != r.stop.end()) {
+            r.finish = Finish::Stop;  // the stop token itself is not part of the output (engine.rs:214-216)
+        } else {
+            r.tokens.push_back(token);
+            if (r.generated() >= r.max_new) r.finish = Finish::Length;
+        }
+        if (r.finish != Finish::None) {
+            r.phase = Phase::Finished;
+            cache_.release_pages(p.entry.slot);
+            running_.erase(std::remove(running_.begin(), running_.end(), p.entry.slot), running_.end());
+            finished.push_back(p.entry.slot);
+        }
+    }
+    if (i != n_sampled) throw std::invalid_argument("more sampled tokens than entries that sample");
+    plan_.clear();
+    return finished;
+}
+
+void Scheduler::drop(int slot) {
+    Request& r = requests_[slot];
+    if (r.phase != Phase::Finished) throw std::logic_error("slot " + std::to_string(slot) + " holds no finished request");
+    r = Request();
+    cache_.release_slot(slot);
+}
+
+}  // namespace llmrs

@@ -1,0 +1,99 @@
+// Continuous batching above the step function: which requests run in the next
+// step and with how many tokens.
+//
+// As the reference's scheduler (src/serve/scheduler.rs:34-76): running requests
+// come first, in the order they were admitted, each with what it still has to
+// compute (one token when it decodes, the rest of its prompt otherwise), cut to
+// the step's token budget; then waiting requests are admitted first-in first-out
+// while budget is left; a request that cannot get its pages is skipped for the
+// step, and the first waiting request that does not fit stops admission.
+//
+// Added to that: a cap on one request's portion; finishing at exactly max_new
+// tokens without the reference's extra step (src/serve/engine.rs:214-229); and a
+// decision for the case the reference spins on (engine.rs:190): when no request
+// can advance because pages ran out, the request admitted last gives its pages
+// back and goes to the front of the waiting queue, to be computed again from its
+// prompt and what it has generated.  Its generator state stays, so its output
+// does not change.
+#pragma once
+#include <cstdint>
+#include <deque>
+#include <vector>
+
+#include "batch.h"
+#include "cache_manager.h"
+#include "sampler_rng.h"
+
+namespace llmrs {
+
+struct SamplingParams {
+    float temperature = 0.0f;  // 0: greedy
+    int top_k = 0;             // 0 or >= vocabulary: off
+    float top_p = 1.0f;        // >= 1: off
+    uint64_t seed = 42;
+};
+
+enum class Phase { Free, Waiting, Running, Finished };
+enum class Finish { None = 0, Stop = 1, Length = 2 };
+
+struct Request {
+    std::vector<int32_t> tokens;  // prompt, then what was generated
+    int prompt_len = 0;
+    int computed = 0;             // tokens whose keys and values are in the cache
+    int max_new = 0;
+    std::vector<int32_t> stop;
+    SamplingParams sampling;
+    Xorshift64 rng;
+    Phase phase = Phase::Free;
+    Finish finish = Finish::None;
+    int preemptions = 0;
+    int generated() const { return (int)tokens.size() - prompt_len; }
+};
+
+struct PlannedEntry {
+    BatchEntry entry;
+    bool samples;  // the portion ends at the request's last known token
+};
+
+class Scheduler {
+public:
+    Scheduler(CacheManager& cache, int token_budget, int max_chunk, int max_positions);
+
+    // Slot of the new request; -1 when no slot is free (ask again later).
+    // Throws when the request could never run: longer than the positions allow,
+    // or needing more pages at once than a pool has.
+    int add(const int32_t* prompt, int n_prompt, int max_new, const SamplingParams& sp,
+            const int32_t* stop, int n_stop);
+    bool idle() const { return running_.empty() && waiting_.empty(); }
+
+    // The next step's entries; empty when idle.
+    const std::vector<PlannedEntry>& plan();
+    const std::vector<PlannedEntry>& planned() const { return plan_; }
+    // Tokens, wanted rows (the last row of each entry that samples) and sampling
+    // words (a uniform drawn from each such request's generator) of the plan.
+    void plan_tokens(std::vector<int32_t>& tokens, std::vector<int32_t>& want_rows,
+                     std::vector<int32_t>& sampling_words);
+    // Takes the sampled token of each entry that samples, in plan order; returns
+    // the slots that finished (their pages are back; the slot stays until drop()).
+    std::vector<int> commit(const int32_t* sampled, int n_sampled);
+
+    const Request& request(int slot) const { return requests_[slot]; }
+    void drop(int slot);  // forget a finished request, free its slot
+    int num_running() const { return (int)running_.size(); }
+    int num_waiting() const { return (int)waiting_.size(); }
+    int64_t preemptions() const { return preemptions_; }
+
+private:
+    int portion(const Request& r, int budget) const;
+    void preempt_last();
+
+    CacheManager& cache_;
+    int budget_, max_chunk_, max_positions_;
+    std::vector<Request> requests_;  // by slot
+    std::vector<int> running_;       // admission order
+    std::deque<int> waiting_;
+    std::vector<PlannedEntry> plan_;
+    int64_t preemptions_ = 0;
+};
+
+}  // namespace llmrs

@@ -1,0 +1,186 @@
+"""The engine: configuration -> model -> cache -> step function -> scheduler ->
+sampler, and `generate()` above them.  Its loop is the reference's serving loop
+without the HTTP channel (src/serve/engine.rs:161-231): plan, flatten, run,
+sample, commit, free what finished."""
+from __future__ import annotations
+
+import sys
+import time
+from dataclasses import dataclass, field
+from typing import Dict, List, Mapping, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from ..config import load_config
+from ..sampling import Sampler, SamplingParams
+from ..weights import load_tensors, random_tensors
+from .model import Model
+from .step import StepEntry, StepRunner
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
+           "fp32": torch.float32, torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+@dataclass
+class GenerationStats:
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    steps: int = 0
+    seconds: float = 0.0
+    preemptions: int = 0
+    first_token_seconds: float = 0.0
+
+
+@dataclass
+class Finished:
+    tokens: List[int]
+    reason: str          # "stop" or "length"
+
+
+class Engine:
+    def __init__(self, config, tensors: Mapping[str, torch.Tensor], *, dtype="bfloat16", device="cuda",
+                 page_size: int = 16, num_pages=None, kv_memory_fraction: float = 0.8, max_requests: int = 256,
+                 max_batch_tokens: int = 2048, max_chunk: int = 0, max_seq_len: Optional[int] = None, log: bool = False):
+        if dtype not in _DTYPES:
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
+        self.config = config
+        self.dtype = _DTYPES[dtype]
+        self.device = torch.device(device)
+        self.log = log
+        spec = config.model_spec()
+        self.model = Model(spec, self.dtype, self.device)
+        self.model.load(tensors)
+        self.max_seq_len = min(max_seq_len or spec.max_positions, spec.max_positions)
+        needs = self.model.cache_needs()
+        if num_pages is None:
+            num_pages = self._pages_from_memory(needs, page_size, kv_memory_fraction, max_requests)
+        self.cache = CacheManager(needs, self.dtype, self.device, page_size, num_pages, max_requests,
+                                  token_budget=max_batch_tokens, max_chunk=max_chunk, max_positions=self.max_seq_len)
+        self.runner = StepRunner(self.model, self.cache, self.device)
+        self.sampler = Sampler(self.device)
+        self.max_batch_tokens = max_batch_tokens
+        self.last_stats = GenerationStats()
+        if log:
+            for g, grp in enumerate(self.cache.groups):
+                gb = grp.num_pages * page_size * grp.bytes_per_token() / 1e9
+                print(f"KV pool {g}: {grp.num_pages} pages x {page_size} tokens = {grp.num_pages * page_size} max tokens, {gb:.2f} GB",
+                      file=sys.stderr)
+
+    # -- construction ----------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, **kw) -> "Engine":
+        config = load_config(folder)
+        probe = Model(config.model_spec(), torch.bfloat16, "cpu")
+        want = {n: t.shape for n, t in probe.tensors().items()}
+        tensors = load_tensors(folder, want, device="cpu", log=kw.get("log", False))
+        return cls(config, tensors, **kw)
+
+    @classmethod
+    def from_random(cls, config, seed: int, **kw) -> "Engine":
+        """Random weights made where the engine lives, without a folder in between."""
+        tensors = random_model_tensors(config, seed, device=kw.get("device", "cuda"))
+        return cls(config, tensors, **kw)
+
+    def _pages_from_memory(self, needs, page_size, fraction, max_requests):
+        """Pages that fit `fraction` of the memory still free after the weights
+        (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
+        from ..cache.spec import PagedKV
+        groups: Dict[PagedKV, int] = {}
+        for need, cache_of in needs:
+            if isinstance(need, PagedKV) and cache_of is None:
+                groups[need] = groups.get(need, 0) + 1
+        if not groups:
+            return []
+        if self.device.type != "cuda":
+            raise ValueError("num_pages must be given when the engine is not on a GPU")
+        free, _ = torch.cuda.mem_get_info(self.device)
+        per_token = sum(2 * n * need.kv_heads * need.head_dim * self.dtype.itemsize for need, n in groups.items())
+        tokens = int(free * fraction) // per_token
+        tokens = min(tokens, max_requests * self.max_seq_len)
+        pages = max(tokens // page_size, 1)
+        return [pages] * len(groups)
+
+    # -- manual stepping (trace replay, tests) -----------------------------------
+    def open_request(self) -> int:
+        """A slot for a request that the caller steps by hand."""
+        return self.cache.core.acquire_slot()
+
+    def close_request(self, slot: int) -> None:
+        self.cache.core.release_slot(slot)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        return self.runner.run(entries)
+
+    # -- generation ----------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 256, temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 1.0, seed: Union[int, Sequence[int]] = 42,
+                 stop_token_ids: Sequence[int] = (), return_reasons: bool = False):
+        """Token ids generated for each prompt.  Every request has its own generator
+        started from `seed` (one for all, or one each), so a prompt's output does not
+        depend on what it was batched with."""
+        n = len(prompts)
+        seeds = [seed] * n if isinstance(seed, int) else list(seed)
+        if len(seeds) != n:
+            raise ValueError("one seed, or one for each prompt")
+        vocab = self.model.spec.vocab_size
+        for i, p in enumerate(prompts):
+            if len(p) == 0:
+                raise ValueError(f"prompt {i} is empty")
+            if min(p) < 0 or max(p) >= vocab:
+                raise ValueError(f"prompt {i}: token ids must be in [0, {vocab})")
+        params = [SamplingParams(temperature, top_k, top_p, s) for s in seeds]
+        results: List[Optional[Finished]] = [None] * n
+        if max_new_tokens <= 0:
+            results = [Finished([], "length") for _ in range(n)]
+            return [r.tokens for r in results] if not return_reasons else results
+        core = self.cache.core
+        pending = list(range(n))
+        slot_of: Dict[int, int] = {}
+        stats = GenerationStats(prompt_tokens=sum(len(p) for p in prompts))
+        all_greedy = temperature == 0.0
+        t0 = time.perf_counter()
+
+        def admit():
+            while pending:
+                i = pending[0]
+                slot = core.add_request(prompts[i], max_new_tokens, params[i].temperature, params[i].top_k,
+                                        params[i].top_p, params[i].seed, stop_token_ids)
+                if slot < 0:
+                    return
+                slot_of[slot] = i
+                pending.pop(0)
+
+        admit()
+        while not core.idle() or pending:
+            logits, n_want, plan = self.runner.run_planned()
+            if not plan:
+                raise RuntimeError("the scheduler planned nothing although requests are waiting")
+            sampled = []
+            if n_want:
+                sampled = self.sampler.sample(logits, self.runner.ctx.sampling, all_greedy).cpu().numpy()
+                if stats.first_token_seconds == 0.0:
+                    stats.first_token_seconds = time.perf_counter() - t0
+            stats.steps += 1
+            for slot in core.commit(sampled):
+                info = core.request_info(slot)
+                i = slot_of.pop(slot)
+                results[i] = Finished(core.request_output(slot), "stop" if info["finish"] == 1 else "length")
+                core.drop_request(slot)
+            admit()
+        if self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
+        stats.seconds = time.perf_counter() - t0
+        stats.generated_tokens = sum(len(r.tokens) for r in results)
+        stats.preemptions = core.preemptions()
+        self.last_stats = stats
+        return results if return_reasons else [r.tokens for r in results]
+
+
+def random_model_tensors(config, seed: int, dtype=torch.bfloat16, device="cpu") -> Dict[str, torch.Tensor]:
+    """The tensors a configuration's model needs, drawn from `seed`."""
+    probe = Model(config.model_spec(), torch.bfloat16, "cpu")
+    specs = probe.tensors()
+    return random_tensors({n: s.shape for n, s in specs.items()}, {n: s.kind for n, s in specs.items()},
+                          seed, dtype=dtype, device=device)

@@ -1,0 +1,91 @@
+"""A model as data: token table, blocks built from a `ModelSpec`, the order they
+run in, final norm and output matrix.  It knows no architecture; the typed
+configuration's `model_spec()` does (config/llama.py).  Reference counterpart:
+LlamaModel / run_layers (src/arch/llama.rs:24-43, :146-172)."""
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..kernels import EPI_STORE_F32, kernels
+from ..parts import TensorSpec, build_block, build_norm
+from ..weights import check_tensors
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        spec.validate()
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"the engine computes in float32 or bfloat16, not {dtype}")
+        self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
+        self.blocks = [build_block(layer, dtype) for layer in spec.layers]
+        self.final_norm = build_norm(spec.final_norm, dtype)
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+
+    # -- weights -------------------------------------------------------------
+    def tensors(self) -> Dict[str, TensorSpec]:
+        s = self.spec
+        out = {s.embedding_name: TensorSpec((s.vocab_size, s.hidden_size))}
+        if s.head_name is not None:
+            out[s.head_name] = TensorSpec((s.vocab_size, s.hidden_size))
+        for block in self.blocks:
+            for part in block.parts():
+                out.update(part.tensors())
+        out.update(self.final_norm.tensors())
+        return out
+
+    def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        """Takes every tensor `tensors()` names; anything missing, left over or
+        of another shape is reported in one error."""
+        want = {n: t.shape for n, t in self.tensors().items()}
+        check_tensors({n: tuple(t.shape) for n, t in tensors.items()}, want)
+        s = self.spec
+        self.embedding = tensors[s.embedding_name].to(device=self.device, dtype=self.dtype).contiguous()
+        # tied: the output matrix is the token table (src/arch/llama.rs:81)
+        self.head = self.embedding if s.head_name is None else \
+            tensors[s.head_name].to(device=self.device, dtype=self.dtype).contiguous()
+        for block in self.blocks:
+            for part in block.parts():
+                part.load(tensors, self.device)
+        self.final_norm.load(tensors, self.device)
+
+    def weight_bytes_per_step(self) -> int:
+        """Bytes of weights one step reads when it uses each once (the table's rows aside)."""
+        total = 0
+        seen = set()
+        for run in self.spec.schedule:
+            for part in self.blocks[run.layer].parts():
+                for v in vars(part).values():
+                    if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                        seen.add(v.data_ptr())
+                        total += v.numel() * v.element_size()
+        total += self.head.numel() * self.head.element_size() + self.final_norm.weight.numel() * 4
+        return total
+
+    # -- cache ---------------------------------------------------------------
+    def cache_needs(self) -> List[Tuple[object, Optional[int]]]:
+        return [(self.blocks[run.layer].mixer.cache_need(), run.cache_of) for run in self.spec.schedule]
+
+    # -- one step --------------------------------------------------------------
+    def forward(self, ctx, cache_views) -> Optional[torch.Tensor]:
+        """Runs the step's T tokens through the schedule; returns float32 logits
+        [n_want, vocab] at the wanted rows, or None when none is wanted."""
+        k = kernels()
+        T = ctx.n_tokens
+        h = ctx.workspace("model.h", (T, self.spec.hidden_size), torch.float32)
+        k.embed_rows(h, self.embedding, ctx.tokens)
+        for i, run in enumerate(self.spec.schedule):
+            ctx.run_index = i
+            self.blocks[run.layer].forward(ctx, h, cache_views[i])
+        if ctx.n_want == 0:
+            return None
+        # Norm only the wanted rows, then the output matrix: the reference norms all
+        # rows and gathers after (src/arch/llama.rs:135-139), which is the same numbers.
+        x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
+        self.final_norm.forward(ctx, h, x, ctx.want_rows)
+        logits = ctx.workspace("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
+        k.gemm(x, self.head, logits, EPI_STORE_F32)
+        return logits

@@ -1,0 +1,186 @@
+"""The step function: a batch of (request, its next tokens) in, logits at the
+wanted places out.  Prompt portions and single decoded tokens are the same
+thing here, entries of `count` tokens from position `start`, and all run as one
+batch from the cache that earlier steps left (src/model.rs:5-8 `forward`, with
+the batch of src/batch.rs:5-16 built as in src/serve/engine.rs:96-154).
+
+Host work per step: ask the core for pages, let it flatten the batch into one
+block of words in pinned memory, copy that block to the device once, launch.
+Activations live in a workspace that grows to the largest step seen and is then
+reused, so steady-state steps allocate nothing.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+
+
+class OutOfPages(RuntimeError):
+    pass
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    start: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()      # places among `tokens` whose logits are wanted
+
+
+class StepContext:
+    """What parts see of the running step.  Device arrays are int32."""
+
+    def __init__(self, runner: "StepRunner"):
+        self._runner = runner
+        self.n_tokens = 0
+        self.n_entries = 0
+        self.n_want = 0
+        self.run_index = -1
+        self.tokens = self.positions = self.token_entry = None
+        self.q_starts = self.seq_lens = self.slots = self.want_rows = self.sampling = None
+        self.slot_maps: List[torch.Tensor] = []
+        self.block_tables: List[torch.Tensor] = []
+        self.entries: List[Tuple[int, int, int]] = []   # host copy: (slot, start, count)
+        self.scratch: Optional[torch.Tensor] = None
+        self.device = runner.device
+
+    def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        return self._runner.workspace(name, shape, dtype)
+
+
+class StepRunner:
+    def __init__(self, model, cache: CacheManager, device, words_capacity: int = 1 << 16):
+        self.model, self.cache, self.device = model, cache, torch.device(device)
+        self._buffers: Dict[str, torch.Tensor] = {}
+        self._pinned = self.device.type == "cuda"
+        self._host = [self._new_host(words_capacity) for _ in range(2)]
+        self._events = [None, None]
+        self._turn = 0
+        self._dev_words = torch.zeros(words_capacity, dtype=torch.int32, device=self.device)
+        self.ctx = StepContext(self)
+        # partial results of split attention over long contexts
+        self.ctx.scratch = torch.empty(self.attention_scratch_floats(), dtype=torch.float32, device=self.device)
+
+    def attention_scratch_floats(self) -> int:
+        return 1 << 22
+
+    def _new_host(self, n: int) -> torch.Tensor:
+        return torch.zeros(n, dtype=torch.int32, pin_memory=self._pinned)
+
+    def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        nbytes = n * dtype.itemsize
+        buf = self._buffers.get(name)
+        if buf is None or buf.numel() < nbytes:
+            # grow with head room so that a slowly growing step does not reallocate each time
+            cap = max(nbytes, 256) if buf is None else max(nbytes, 2 * buf.numel())
+            buf = torch.empty(cap, dtype=torch.uint8, device=self.device)
+            self._buffers[name] = buf
+        return buf[:nbytes].view(dtype).view(*shape)
+
+    # -- staging -----------------------------------------------------------------
+    def _staging(self, words_needed: int) -> np.ndarray:
+        self._turn ^= 1
+        i = self._turn
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+            self._events[i] = None
+        if self._host[i].numel() < words_needed:
+            self._host[i] = self._new_host(max(words_needed, 2 * self._host[i].numel()))
+        return self._host[i].numpy()
+
+    def _upload(self, n_words: int) -> torch.Tensor:
+        i = self._turn
+        if self._dev_words.numel() < n_words:
+            self._dev_words = torch.zeros(max(n_words, 2 * self._dev_words.numel()), dtype=torch.int32, device=self.device)
+        dev = self._dev_words[:n_words]
+        dev.copy_(self._host[i][:n_words], non_blocking=True)
+        if self._pinned:
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[i] = ev
+        return dev
+
+    def _estimate_words(self, T: int, R: int, n_want: int, longest: int) -> int:
+        """Upper bound of the flattened batch's size; `longest` is the largest start + count.
+        A block table never has more entries than the positions ensured for it need."""
+        words = 4 + 3 * T + 3 * R + 1 + 5 * n_want
+        for grp in self.cache.groups:
+            words += T + R * max(1, -(-longest // grp.page_size))
+        return words + 16
+
+    def _bind(self, dev: torch.Tensor, off, T: int, R: int, n_want: int, entries) -> StepContext:
+        c = self.ctx
+        c.n_tokens, c.n_entries, c.n_want = T, R, n_want
+        c.entries = entries
+        c.tokens = dev[off.tokens:off.tokens + T]
+        c.positions = dev[off.positions:off.positions + T]
+        c.token_entry = dev[off.token_entry:off.token_entry + T]
+        c.q_starts = dev[off.q_starts:off.q_starts + R + 1]
+        c.seq_lens = dev[off.seq_lens:off.seq_lens + R]
+        c.slots = dev[off.slots:off.slots + R]
+        c.want_rows = dev[off.want_rows:off.want_rows + n_want]
+        c.sampling = dev[off.sampling:off.sampling + 4 * n_want].view(n_want, 4)
+        c.slot_maps = [dev[o:o + T] for o in off.slot_maps]
+        c.block_tables = [dev[o:o + R * w].view(R, w) for o, w in zip(off.tables, off.widths)]
+        return c
+
+    # -- the step ------------------------------------------------------------------
+    def run(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs the entries' tokens as one batch; returns float32 logits
+        [wanted, vocab] (a view into the workspace, valid until the next step), in
+        the order of the entries and of their `want`, or None."""
+        entries = [e for e in entries]
+        if not entries:
+            return None
+        core = self.cache.core
+        vocab = self.model.spec.vocab_size
+        slots, starts, counts, tokens, want_rows = [], [], [], [], []
+        for e in entries:
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"the entry of slot {e.slot} brings no tokens")
+            if e.start + n > self.model.spec.max_positions:
+                raise ValueError(f"slot {e.slot}: position {e.start + n - 1} is beyond the model's {self.model.spec.max_positions}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"slot {e.slot}: wanted place {w} is outside its {n} tokens")
+                want_rows.append(len(tokens) + w)
+            ids = np.asarray(e.tokens, dtype=np.int64)
+            if ids.min() < 0 or ids.max() >= vocab:
+                raise ValueError(f"slot {e.slot}: token ids must be in [0, {vocab}), got {int(ids.min())}..{int(ids.max())}")
+            if not core.ensure(e.slot, e.start, n):
+                raise OutOfPages(f"no cache pages left for slot {e.slot} at positions {e.start}..{e.start + n - 1}")
+            slots.append(e.slot); starts.append(e.start); counts.append(n); tokens.extend(ids.tolist())
+        T, R = len(tokens), len(entries)
+        words = self._staging(self._estimate_words(T, R, len(want_rows), max(a + b for a, b in zip(starts, counts))))
+        off = core.build_batch(slots, starts, counts, tokens, want_rows, words)
+        dev = self._upload(off.words)
+        ctx = self._bind(dev, off, T, R, len(want_rows), list(zip(slots, starts, counts)))
+        return self._execute(ctx)
+
+    def run_planned(self):
+        """Runs the step the scheduler planned; returns (logits or None, rows that sample)."""
+        core = self.cache.core
+        plan = core.plan()
+        if not plan:
+            return None, 0, plan
+        T = sum(p[2] for p in plan)
+        R = len(plan)
+        words = self._staging(self._estimate_words(T, R, R, max(p[1] + p[2] for p in plan)))
+        off, n_tokens, n_want = core.build_planned(words)
+        dev = self._upload(off.words)
+        ctx = self._bind(dev, off, n_tokens, R, n_want, [(p[0], p[1], p[2]) for p in plan])
+        return self._execute(ctx), n_want, plan
+
+    def _execute(self, ctx: StepContext) -> Optional[torch.Tensor]:
+        fresh = [slot for slot, start, _ in ctx.entries if start == 0]
+        self.cache.reset_state(fresh)
+        return self.model.forward(ctx, self.cache.views)

@@ -1,0 +1,156 @@
+"""The kernel interface: every device operation of the engine goes through the
+object `kernels()` returns.  It is the gfx950 library (csrc/hip) or nothing:
+when that library cannot be built or loaded, or there is no GPU, the first use
+raises.  `use_kernels()` lets a test put another object with the same methods in
+its place; the package itself never does.
+
+Op set of the reference's `Backend` trait (src/backend/mod.rs:15-89), fused:
+embed, rms_norm, matmul (+ residual add / SwiGLU epilogues for add/silu/mul),
+rope + scatter_kv, attention, gather (folded into rms_norm's row list), argmax.
+"""
+from __future__ import annotations
+
+import contextlib
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from typing import Optional
+
+import torch
+
+EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16, not {dtype}") from None
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+class HipKernels:
+    """Launches on the current torch stream of the tensors' device."""
+
+    def __init__(self):
+        from .csrc.build import load_hip
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU: the engine's kernels are gfx950 HIP kernels and there is no other path")
+        self.lib = lib = load_hip()
+        lib.llmrs_hip_error.restype = c_char_p
+        V, I, F = c_void_p, c_int, c_float
+        sigs = {
+            "llmrs_embed_rows": [V, I, V, V, V, I, I, I],
+            "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, I],
+            "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
+            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I],
+            "llmrs_argmax_rows": [V, V, I, I, I, V],
+        }
+        for name, args in sigs.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = I
+        buf = ctypes.create_string_buffer(64)
+        lib.llmrs_device_arch.argtypes = [c_char_p, I]
+        lib.llmrs_device_arch.restype = I
+        self.compute_units = lib.llmrs_device_arch(buf, 64)
+        self.arch = buf.value.decode()
+        if not self.arch.startswith("gfx950"):
+            raise KernelError(f"the kernel library is built for gfx950, the device is {self.arch!r}")
+        self.allow_mfma = True  # tests switch the matrix-core kernels off to compare paths
+
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise KernelError(self.lib.llmrs_hip_error().decode())
+
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    # out[t, :] = table[tokens[t], :] as float32
+    def embed_rows(self, out: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor) -> None:
+        assert out.dtype == torch.float32 and tokens.dtype == torch.int32 and table.is_contiguous() and out.is_contiguous()
+        assert out.shape[0] == tokens.shape[0] and out.shape[1] == table.shape[1]
+        self._check(self.lib.llmrs_embed_rows(self._stream(), _code(table.dtype), _p(out), _p(table), _p(tokens),
+                                              tokens.shape[0], table.shape[1], table.shape[0]))
+
+    # out[i, :] = rmsnorm(x[rows[i] or i, :]) * weight
+    def rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
+                rows: Optional[torch.Tensor] = None) -> None:
+        assert x.dtype == torch.float32 and weight.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous()
+        n = out.shape[0]
+        assert out.shape[1] == x.shape[1] == weight.shape[0]
+        assert (rows is None and n == x.shape[0]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
+        self._check(self.lib.llmrs_rmsnorm(self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(rows),
+                                           n, x.shape[1], eps))
+
+    # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
+    def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+        M, K = a.shape
+        N = w.shape[0]
+        assert w.shape[1] == K and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1 and a.dtype == w.dtype
+        want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
+        assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
+        self._check(self.lib.llmrs_gemm(self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
+                                        M, N, K, epilogue, int(self.allow_mfma)))
+
+    def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
+                      n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:
+        assert qkv.stride(1) == 1 and positions.dtype == torch.int32
+        assert rotary_dim == 0 or (inv_freq.dtype == torch.float32 and inv_freq.shape[0] == rotary_dim // 2)
+        if write_kv:
+            assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+            assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
+            assert slot_map.dtype == torch.int32 and slot_map.shape[0] == qkv.shape[0]
+        self._check(self.lib.llmrs_rope_kv_write(
+            self._stream(), _code(qkv.dtype), _p(qkv), qkv.stride(0), _p(positions), _p(slot_map), _p(inv_freq),
+            rotary_dim, int(interleaved), _p(k_cache), _p(v_cache), qkv.shape[0], n_heads, n_kv_heads, head_dim,
+            page_size, num_pages, int(write_kv)))
+
+    def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None) -> None:
+        assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
+        assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+        assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
+        T = q.shape[0]
+        assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
+        self._check(self.lib.llmrs_attention(
+            self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
+            _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
+            block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
+            _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(self.allow_mfma)))
+
+    def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor) -> None:
+        assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
+        self._check(self.lib.llmrs_argmax_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
+                                               logits.shape[1], _p(out)))
+
+
+_kernels = None
+
+
+def kernels():
+    global _kernels
+    if _kernels is None:
+        _kernels = HipKernels()
+    return _kernels
+
+
+@contextlib.contextmanager
+def use_kernels(obj):
+    """For tests: run the engine's host logic against a stand-in for the device."""
+    global _kernels
+    old, _kernels = _kernels, obj
+    try:
+        yield obj
+    finally:
+        _kernels = old

@@ -1,0 +1,89 @@
+"""Causal grouped-query attention over the paged cache.
+
+Parameters: hidden_size, num_heads, num_kv_heads, head_dim, window (None: every
+earlier key), position (a position-encoding spec or None), scale (None:
+1/sqrt(head_dim), shaders/ops.metal:670), kv_proj (False: the part has no k and
+v of its own and only reads a cache that another run wrote).
+
+One step (src/arch/llama.rs:153-163): q, k, v = x Wq^T, x Wk^T, x Wv^T in one
+product over the row-concatenated weight; rotate q and k and write k, v into
+their pages in one kernel; attention of every query token over its request's
+pages; h += o Wo^T with the sum fused into the product.  No biases.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..cache.spec import PagedKV
+from ..kernels import EPI_ACCUM_F32, EPI_STORE, kernels
+from .base import Mixer, TensorSpec, build_position, register_mixer
+
+
+class Attention(Mixer):
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.heads = int(p["num_heads"])
+        self.kv_heads = int(p["num_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.window = int(p.get("window") or 0)
+        self.kv_proj = bool(p.get("kv_proj", True))
+        scale = p.get("scale")
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.position = build_position(p.get("position"), dtype)
+        if self.heads % self.kv_heads:
+            raise ValueError(f"{self.heads} heads are no multiple of {self.kv_heads} kv heads")
+        self.q_size = self.heads * self.head_dim
+        self.kv_size = self.kv_heads * self.head_dim
+        self.w_qkv = None
+        self.w_o = None
+
+    def tensors(self):
+        t = {self.name("q_proj.weight"): TensorSpec((self.q_size, self.hidden)),
+             self.name("o_proj.weight"): TensorSpec((self.hidden, self.q_size))}
+        if self.kv_proj:
+            t[self.name("k_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
+            t[self.name("v_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
+        return t
+
+    def load(self, tensors, device):
+        names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.kv_proj else [])
+        self.w_qkv = torch.cat([tensors[self.name(n)].to(device=device, dtype=self.dtype) for n in names], dim=0).contiguous()
+        self.w_o = tensors[self.name("o_proj.weight")].to(device=device, dtype=self.dtype).contiguous()
+        if self.position is not None:
+            self.position.to(device)
+
+    def cache_need(self):
+        return PagedKV(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, ctx, x, h, cache):
+        k = kernels()
+        T = x.shape[0]
+        write = self.kv_proj and cache.writes
+        n_kv = self.kv_heads if self.kv_proj else 0
+        qkv = ctx.workspace("attn.qkv", (T, self.q_size + 2 * n_kv * self.head_dim), self.dtype)
+        k.gemm(x, self.w_qkv, qkv, EPI_STORE)
+        rotary = self.position.rotary() if self.position is not None else None
+        if rotary is None:
+            if self.position is not None:
+                q3 = qkv[:, :self.q_size].unflatten(1, (self.heads, self.head_dim))
+                k3 = qkv[:, self.q_size:self.q_size + self.kv_size].unflatten(1, (self.kv_heads, self.head_dim)) if n_kv else None
+                self.position.apply(ctx, q3, k3)
+            inv_freq, rotary_dim, interleaved = None, 0, False
+        else:
+            inv_freq, rotary_dim, interleaved = rotary
+        g = cache.group
+        if write or rotary_dim:
+            k.rope_kv_write(qkv, ctx.positions, ctx.slot_maps[g], inv_freq, rotary_dim, interleaved,
+                            cache.k, cache.v, self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
+        o = ctx.workspace("attn.out", (T, self.q_size), self.dtype)
+        k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
+                    ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
+                    cache.num_pages, self.window, self.scale, ctx.scratch)
+        k.gemm(o, self.w_o, h, EPI_ACCUM_F32)
+
+
+register_mixer("attention", Attention)

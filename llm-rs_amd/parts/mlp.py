@@ -1,0 +1,41 @@
+"""SwiGLU feed-forward(hidden_size, intermediate_size):
+h += (silu(x Wg^T) * (x Wu^T)) Wd^T, silu(v) = v / (1 + exp(-v))
+(src/arch/llama.rs:165-170, shaders/ops.metal:762-793).  The gate and up weights
+are interleaved row by row at load, so one product yields (gate_j, up_j) side by
+side and its epilogue writes silu(gate) * up, computed in 32-bit, once; the down
+product adds into the 32-bit residual stream.  No biases."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import EPI_ACCUM_F32, EPI_SWIGLU, kernels
+from .base import FeedForward, TensorSpec, register_feed_forward
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+        self.w_gate_up = None
+        self.w_down = None
+
+    def tensors(self):
+        return {self.name("gate_proj.weight"): TensorSpec((self.inter, self.hidden)),
+                self.name("up_proj.weight"): TensorSpec((self.inter, self.hidden)),
+                self.name("down_proj.weight"): TensorSpec((self.hidden, self.inter))}
+
+    def load(self, tensors, device):
+        gate = tensors[self.name("gate_proj.weight")].to(device=device, dtype=self.dtype)
+        up = tensors[self.name("up_proj.weight")].to(device=device, dtype=self.dtype)
+        self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
+        self.w_down = tensors[self.name("down_proj.weight")].to(device=device, dtype=self.dtype).contiguous()
+
+    def forward(self, ctx, x, h):
+        k = kernels()
+        act = ctx.workspace("mlp.act", (x.shape[0], self.inter), self.dtype)
+        k.gemm(x, self.w_gate_up, act, EPI_SWIGLU)
+        k.gemm(act, self.w_down, h, EPI_ACCUM_F32)
+
+
+register_feed_forward("swiglu", SwiGLU)

@@ -1,0 +1,31 @@
+"""RMSNorm(size, eps): y = x / sqrt(mean(x^2) + eps) * weight, computed in 32-bit,
+the weight multiplying directly.  Reference: rms_norm_batch
+(shaders/ops.metal:970-1003), used at src/arch/llama.rs:152,164,135."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import kernels
+from .base import Norm, TensorSpec, register_norm
+
+
+class RMSNorm(Norm):
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.size = int(spec.params["size"])
+        self.eps = float(spec.params["eps"])
+        self.weight = None
+
+    def tensors(self):
+        return {self.name("weight"): TensorSpec((self.size,), "norm")}
+
+    def load(self, tensors, device):
+        # The reference wants norm weights in 32-bit (ops.metal:972); whatever the
+        # file stores, the kernel multiplies by a float32 weight.
+        self.weight = tensors[self.name("weight")].to(device=device, dtype=torch.float32).contiguous()
+
+    def forward(self, ctx, h, out, rows=None):
+        kernels().rmsnorm(out, h, self.weight, self.eps, rows)
+
+
+register_norm("rmsnorm", RMSNorm)

@@ -1,0 +1,240 @@
+"""A plain, slow Llama decoder for the tests to compare the engine with.
+
+Whole sequences, no cache, no batching, one function for each part, written from
+the reference's formulas (each function cites them) in ordinary tensor
+operations.  It shares no code with the package: it reads config.json and
+model.safetensors itself.  Computation is in the dtype of `compute` (float64 by
+default) from the weights as stored.
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+import struct
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+_ST_DTYPES = {"F32": torch.float32, "BF16": torch.bfloat16, "F16": torch.float16, "F64": torch.float64}
+
+
+def read_model_folder(folder: str):
+    """(config dict, {name: tensor}) read directly from the files."""
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    tensors = {}
+    with open(os.path.join(folder, "model.safetensors"), "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        header = json.loads(f.read(n))
+        data = f.read()
+    for name, e in header.items():
+        if name == "__metadata__":
+            continue
+        lo, hi = e["data_offsets"]
+        t = torch.frombuffer(bytearray(data[lo:hi]), dtype=_ST_DTYPES[e["dtype"]]).reshape(e["shape"])
+        tensors[name] = t.clone()
+    return cfg, tensors
+
+
+# ---- parts -------------------------------------------------------------------
+
+def plain_embedding(table: torch.Tensor, tokens: Sequence[int]) -> torch.Tensor:
+    """x[t, :] = table[tok[t], :], no scaling (src/arch/llama.rs:150, shaders/ops.metal:878-902)."""
+    return table[torch.tensor(list(tokens), dtype=torch.long)]
+
+
+def plain_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    """ss = sum x^2; inv = rsqrt(ss / D + eps); y = x * inv * w; the weight
+    multiplies directly (shaders/ops.metal:980-1002)."""
+    ss = (x * x).sum(dim=-1, keepdim=True)
+    inv = 1.0 / torch.sqrt(ss / x.shape[-1] + eps)
+    return x * inv * w
+
+
+def plain_inv_freq(rotary_dim: int, theta: float, scaling: Optional[dict]) -> torch.Tensor:
+    """freq_i = 1 / theta^(2i/d) (shaders/ops.metal:1030).  The reference scales
+    nothing; "llama3" scaling follows the engine's own statement of it: by
+    wavelength 2 pi / freq against L = original_max_position_embeddings: shorter
+    than L/high kept, longer than L/low divided by factor, between blended linearly
+    in L/wavelength.  Rounded to float32, as the engine's table is."""
+    i = torch.arange(rotary_dim // 2, dtype=torch.float64)
+    freq = 1.0 / (theta ** (2.0 * i / rotary_dim))
+    if scaling is not None and scaling.get("rope_type", scaling.get("type")) == "llama3":
+        factor, low, high = scaling["factor"], scaling["low_freq_factor"], scaling["high_freq_factor"]
+        L = scaling["original_max_position_embeddings"]
+        wavelength = 2.0 * math.pi / freq
+        smooth = (L / wavelength - low) / (high - low)
+        blended = (1.0 - smooth) * freq / factor + smooth * freq
+        freq = torch.where(wavelength < L / high, freq, torch.where(wavelength > L / low, freq / factor, blended))
+    return freq.to(torch.float32)
+
+
+def plain_rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, layout: str = "split_half") -> torch.Tensor:
+    """x: [T, heads, head_dim].  angle = float(pos) * freq_i in 32-bit;
+    (a, b) <- (a cos - b sin, a sin + b cos) (shaders/ops.metal:1031-1041); the pair
+    is (i, i + d/2) for "split_half", (2i, 2i+1) for "interleaved"
+    (src/tensor/mod.rs:133-139).  Features past the rotary width are unchanged."""
+    rot = 2 * inv_freq.shape[0]
+    angle = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).to(x.dtype)   # [T, rot/2]
+    cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+    out = x.clone()
+    if layout == "split_half":
+        a, b = x[..., :rot // 2], x[..., rot // 2:rot]
+        out[..., :rot // 2] = a * cos - b * sin
+        out[..., rot // 2:rot] = a * sin + b * cos
+    elif layout == "interleaved":
+        a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+        out[..., 0:rot:2] = a * cos - b * sin
+        out[..., 1:rot:2] = a * sin + b * cos
+    else:
+        raise ValueError(layout)
+    return out
+
+
+def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
+                    window: int = 0, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q: [T, heads, d]; k, v: [T, kv_heads, d]; one sequence, causal.
+    Head h uses kv head h / (heads / kv_heads); s_j = (q . k_j) * rsqrt(d), the scale
+    after the dot; keys j <= the query's place (and > place - window if a window is
+    given); softmax over j; o = sum_j p_j v_j (shaders/ops.metal:658-757)."""
+    T, H, d = q.shape
+    KV = k.shape[1]
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    out = torch.zeros_like(q)
+    place = torch.arange(T) if positions is None else positions
+    for h in range(H):
+        g = h // (H // KV)
+        scores = (q[:, h, :] @ k[:, g, :].T) * scale                      # [T, T]
+        visible = place[None, :] <= place[:, None]
+        if window > 0:
+            visible &= place[None, :] > place[:, None] - window
+        scores = scores.masked_fill(~visible, float("-inf"))
+        out[:, h, :] = torch.softmax(scores, dim=-1) @ v[:, g, :]
+    return out
+
+
+def plain_silu(x: torch.Tensor) -> torch.Tensor:
+    """v / (1 + exp(-v)) (shaders/ops.metal:769)."""
+    return x / (1.0 + torch.exp(-x))
+
+
+def plain_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """(silu(x Wg^T) * (x Wu^T)) Wd^T (src/arch/llama.rs:165-169)."""
+    return (plain_silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+
+
+# ---- the model -----------------------------------------------------------------
+
+def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
+                  compute: torch.dtype = torch.float64, layout: str = "split_half") -> torch.Tensor:
+    """Logits [T, vocab] for one whole sequence from position 0.  Layer loop of
+    src/arch/llama.rs:150-171, final norm and output matrix of :135-139; tied
+    embeddings reuse the token table (:81)."""
+    W = {n: t.to(compute) for n, t in weights.items()}
+    H, D = cfg["num_attention_heads"], cfg["hidden_size"]
+    KV = cfg.get("num_key_value_heads") or H
+    d = cfg.get("head_dim") or D // H
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    inv_freq = plain_inv_freq(d, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
+    T = len(tokens)
+    pos = torch.arange(T)
+    x = plain_embedding(W["model.embed_tokens.weight"], tokens)
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        xn = plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps)
+        q = (xn @ W[p + "self_attn.q_proj.weight"].T).view(T, H, d)
+        k = (xn @ W[p + "self_attn.k_proj.weight"].T).view(T, KV, d)
+        v = (xn @ W[p + "self_attn.v_proj.weight"].T).view(T, KV, d)
+        q, k = plain_rope(q, pos, inv_freq, layout), plain_rope(k, pos, inv_freq, layout)
+        o = plain_attention(q, k, v).reshape(T, H * d)
+        x = x + o @ W[p + "self_attn.o_proj.weight"].T
+        xn = plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps)
+        x = x + plain_swiglu(xn, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+    xn = plain_rmsnorm(x, W["model.norm.weight"], eps)
+    head = W["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else W["lm_head.weight"]
+    return xn @ head.T
+
+
+# ---- sampling ------------------------------------------------------------------
+
+class PlainXorshift:
+    """xorshift64 with shifts 13, 7, 17; seed 0 stands for 0xDEADBEEFCAFE; a float is
+    the top 24 bits over 2^24 (src/sampler/mod.rs:7-24)."""
+
+    def __init__(self, seed: int):
+        self.state = 0xDEADBEEFCAFE if seed == 0 else seed
+
+    def next_u64(self) -> int:
+        x = self.state
+        x ^= (x << 13) & 0xFFFFFFFFFFFFFFFF
+        x ^= x >> 7
+        x ^= (x << 17) & 0xFFFFFFFFFFFFFFFF
+        self.state = x
+        return x
+
+    def next_f32(self) -> float:
+        return (self.next_u64() >> 40) / float(1 << 24)
+
+
+def plain_argmax(logits: torch.Tensor) -> int:
+    """Greedy; of equal logits the lowest index (the engine's rule; the reference
+    leaves ties open, shaders/ops.metal:803-835 vs src/sampler/mod.rs:65-68)."""
+    best = logits.max()
+    return int((logits == best).nonzero()[0])
+
+
+def plain_probabilities(logits: torch.Tensor, temperature: float, top_k: int, top_p: float) -> torch.Tensor:
+    """The distribution the reference samples from (src/sampler/mod.rs:84-141), in
+    float64: logits / T; all but the top_k largest dropped; softmax; the smallest
+    prefix of the descending order whose mass reaches top_p kept and renormalised.
+    Ties at a cut are broken towards the lower index (the reference's unstable
+    sorts leave them open)."""
+    z = logits.to(torch.float64) * (1.0 / temperature)
+    V = z.shape[0]
+    order = sorted(range(V), key=lambda i: (-float(z[i]), i))
+    keep = torch.ones(V, dtype=torch.bool)
+    if 0 < top_k < V:
+        keep[:] = False
+        keep[order[:top_k]] = True
+    z = z.masked_fill(~keep, float("-inf"))
+    p = torch.softmax(z, dim=0)
+    if top_p < 1.0:
+        total, cut = 0.0, V
+        for n, i in enumerate(order):
+            total += float(p[i])
+            if total >= top_p:
+                cut = n + 1
+                break
+        drop = order[cut:]
+        p[drop] = 0.0
+        p = p / p.sum()
+    return p
+
+
+def plain_sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, rng: PlainXorshift) -> int:
+    """One draw: the first index whose cumulative probability exceeds the uniform,
+    walking in index order (src/sampler/mod.rs:143-154)."""
+    if temperature == 0.0:
+        return plain_argmax(logits)
+    p = plain_probabilities(logits, temperature, top_k, top_p)
+    r = rng.next_f32()
+    cum = torch.cumsum(p, dim=0)
+    hit = (cum > r).nonzero()
+    return int(hit[0]) if len(hit) else int(p.nonzero()[-1])
+
+
+def plain_generate(cfg: dict, weights: Dict[str, torch.Tensor], prompt: Sequence[int], max_new: int,
+                   temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: int = 42,
+                   stop: Sequence[int] = (), compute: torch.dtype = torch.float64) -> List[int]:
+    """The whole sequence is run again for every new token."""
+    rng = PlainXorshift(seed)
+    tokens, out = list(prompt), []
+    for _ in range(max_new):
+        logits = plain_forward(cfg, weights, tokens, compute)[-1]
+        tok = plain_sample(logits.to(torch.float32), temperature, top_k, top_p, rng)
+        if tok in stop:
+            break
+        out.append(tok)
+        tokens.append(tok)
+    return out
