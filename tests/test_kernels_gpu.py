@@ -1,0 +1,282 @@
+"""Each kernel alone against the plain reference of its part, at sizes other than
+the tiny models': widths and vocabularies that are no power of two, head sizes in
+steps of 16, any number of heads and groups."""
+import math
+
+import pytest
+import torch
+
+from llm_rs_amd.kernels import EPI_ACCUM_F32, EPI_STORE, EPI_STORE_F32, EPI_SWIGLU, kernels
+from plain_llama import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope, plain_silu
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def out_tol(ref, dtype, floor):
+    """Allowed error per element: half an ulp of the output type and then some, or a floor
+    for sums that cancel (tests/ops.rs:142-145 uses |e|/64 and a floor for bfloat16 output)."""
+    rel = 1.0 / 64 if dtype == torch.bfloat16 else 1e-5
+    return ref.abs() * rel + floor
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_rows(dtype):
+    table = rnd((1000, 200), dtype, 0)
+    tokens = torch.tensor([0, 999, 17, 17, 500], dtype=torch.int32, device=DEV)
+    out = torch.empty((5, 200), dtype=torch.float32, device=DEV)
+    kernels().embed_rows(out, table, tokens)
+    assert torch.equal(out, table[tokens.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,eps", [(200, 1e-5), (4104, 1e-6), (64, 1e-2)])
+def test_rmsnorm(dtype, D, eps):
+    x = rnd((9, D), torch.float32, 1, 3.0)
+    w = rnd((D,), torch.float32, 2) * 0.1 + 1
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)
+    for r in (None, rows):
+        n = 9 if r is None else 4
+        out = torch.empty((n, D), dtype=dtype, device=DEV)
+        kernels().rmsnorm(out, x, w, eps, r)
+        src = x if r is None else x[r.long()]
+        ref = plain_rmsnorm(src.double().cpu(), w.double().cpu(), eps)
+        err = (out.double().cpu() - ref).abs()
+        assert (err <= out_tol(ref, dtype, 1e-6)).all(), float(err.max())
+
+
+GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256, 128), (65, 130, 1024),
+               (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("epi", [EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU])
+def test_gemm(dtype, M, N, K, epi):
+    pad = 24
+    a_full = rnd((M, K + pad), dtype, 3)
+    a = a_full[:, :K]                       # rows with a stride, as q inside qkv has
+    w = rnd((N, K), dtype, 4, 0.1)
+    acc = a.double().cpu() @ w.double().cpu().T
+    floor = 2e-6 * math.sqrt(K) if dtype == torch.float32 else 1e-5 * math.sqrt(K)
+    if epi == EPI_STORE:
+        out = torch.zeros((M, N), dtype=dtype, device=DEV)
+        ref, odt = acc, dtype
+    elif epi == EPI_STORE_F32:
+        out = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+        ref, odt = acc, torch.float32
+    elif epi == EPI_ACCUM_F32:
+        out = rnd((M, N), torch.float32, 5)
+        ref, odt = out.double().cpu() + acc, torch.float32
+    else:
+        out = torch.zeros((M, N // 2), dtype=dtype, device=DEV)
+        ref, odt = plain_silu(acc[:, 0::2]) * acc[:, 1::2], dtype
+    kernels().gemm(a, w, out, epi)
+    err = (out.double().cpu() - ref).abs()
+    tol = out_tol(ref, odt, floor)
+    assert (err <= tol).all(), f"max err {float(err.max())} at {int(err.argmax())}, tol there {float(tol.flatten()[err.argmax()])}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_rows_do_not_depend_on_batch(dtype):
+    """Row t of the result depends on row t of the input only: the same row alone, in a
+    small batch and in a large one agrees to rounding of the output."""
+    K, N = 320, 200
+    a = rnd((150, K), dtype, 6)
+    w = rnd((N, K), dtype, 7, 0.1)
+    outs = []
+    for rows in ([7], list(range(4, 12)), list(range(150))):
+        sub = a[rows].contiguous()
+        out = torch.zeros((len(rows), N), dtype=torch.float32, device=DEV)
+        kernels().gemm(sub, w, out, EPI_STORE_F32)
+        outs.append(out[rows.index(7)].cpu())
+    assert (outs[0] - outs[1]).abs().max() <= 2e-5 and (outs[0] - outs[2]).abs().max() <= 2e-5
+
+
+def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, scaling=None):
+    T, num_pages = 11, 9
+    S = (n_heads + 2 * n_kv) * hd + 8
+    qkv = rnd((T, S), dtype, 8)
+    before = qkv.clone()
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 5, 6, 7, 300, 301], dtype=torch.int32, device=DEV)
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(9))[:T].to(torch.int32).to(DEV)
+    inv_freq = plain_inv_freq(rot, theta, scaling).to(DEV)
+    kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=dtype, device=DEV)
+    vc = torch.zeros((num_pages, n_kv, hd, page_size), dtype=dtype, device=DEV)
+    kernels().rope_kv_write(qkv, positions, slots, inv_freq, rot, layout == "interleaved", kc, vc,
+                            n_heads, n_kv, hd, page_size, num_pages, True)
+    b = before.double().cpu()
+    q = b[:, :n_heads * hd].view(T, n_heads, hd)
+    k = b[:, n_heads * hd:(n_heads + n_kv) * hd].view(T, n_kv, hd)
+    v = b[:, (n_heads + n_kv) * hd:(n_heads + 2 * n_kv) * hd].view(T, n_kv, hd)
+    qr = plain_rope(q, positions.cpu(), inv_freq.cpu(), layout)
+    kr = plain_rope(k, positions.cpu(), inv_freq.cpu(), layout)
+    floor = 1e-6 if dtype == torch.float32 else 1e-3
+    got_q = qkv[:, :n_heads * hd].double().cpu().view(T, n_heads, hd)
+    assert ((got_q - qr).abs() <= out_tol(qr, dtype, floor)).all()
+    assert torch.equal(qkv[:, (n_heads + 2 * n_kv) * hd:], before[:, (n_heads + 2 * n_kv) * hd:]), "padding touched"
+    page, off = (slots // page_size).long().cpu(), (slots % page_size).long().cpu()
+    got_k = kc.double().cpu()[page, :, off, :]
+    got_v = vc.double().cpu()[page, :, :, off]
+    assert ((got_k - kr).abs() <= out_tol(kr, dtype, floor)).all()
+    assert torch.equal(got_v, v), "values are copied unchanged"
+    written = torch.zeros(num_pages * page_size, dtype=torch.bool)
+    written[slots.long().cpu()] = True
+    kflat = kc.cpu().permute(0, 2, 1, 3).reshape(num_pages * page_size, -1)
+    assert (kflat[~written] == 0).all(), "a slot that no token maps to was written"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,rot,layout,page_size", [
+    (4, 2, 16, 16, "split_half", 4), (3, 1, 32, 32, "split_half", 16), (5, 5, 48, 48, "interleaved", 16),
+    (6, 2, 80, 32, "split_half", 8), (2, 1, 128, 128, "interleaved", 16), (8, 2, 64, 0, "split_half", 16)])
+def test_rope_kv_write(dtype, n_heads, n_kv, hd, rot, layout, page_size):
+    _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size)
+
+
+def test_rope_kv_write_llama3_scaling():
+    _rope_case(torch.float32, 4, 2, 64, 64, "split_half", 16, theta=500000.0,
+               scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                            original_max_position_embeddings=64))
+
+
+class PagedCase:
+    """Sequences with keys and values scattered over shuffled pages."""
+
+    def __init__(self, dtype, lens, n_heads, n_kv, hd, page_size, seed=0, extra_pages=3):
+        self.dtype, self.lens, self.n_heads, self.n_kv, self.hd, self.ps = dtype, lens, n_heads, n_kv, hd, page_size
+        g = torch.Generator().manual_seed(seed)
+        pages_per = [-(-n // page_size) for n in lens]
+        self.num_pages = sum(pages_per) + extra_pages
+        self.k = [torch.randn((n, n_kv, hd), generator=g).to(dtype) for n in lens]
+        self.v = [torch.randn((n, n_kv, hd), generator=g).to(dtype) for n in lens]
+        perm = torch.randperm(self.num_pages, generator=g).tolist()
+        self.width = max(pages_per)
+        self.tables = torch.zeros((len(lens), self.width), dtype=torch.int32)
+        self.kc = torch.zeros((self.num_pages, n_kv, page_size, hd), dtype=dtype)
+        self.vc = torch.zeros((self.num_pages, n_kv, hd, page_size), dtype=dtype)
+        at = 0
+        for r, n in enumerate(lens):
+            for i in range(pages_per[r]):
+                page = perm[at]; at += 1
+                self.tables[r, i] = page
+                lo, hi = i * page_size, min((i + 1) * page_size, n)
+                self.kc[page, :, :hi - lo, :] = self.k[r][lo:hi].permute(1, 0, 2)
+                self.vc[page, :, :, :hi - lo] = self.v[r][lo:hi].permute(1, 2, 0)
+
+    def run(self, q_list, q_pos_list, window=0, scale=None):
+        """q_list[r]: [n_r, heads, hd] queries of request r at positions q_pos_list[r]."""
+        scale = 1.0 / math.sqrt(self.hd) if scale is None else scale
+        q = torch.cat(q_list).reshape(-1, self.n_heads * self.hd).to(DEV)
+        T = q.shape[0]
+        entry = torch.cat([torch.full((len(p),), r, dtype=torch.int32) for r, p in enumerate(q_pos_list)]).to(DEV)
+        pos = torch.cat([torch.tensor(p, dtype=torch.int32) for p in q_pos_list]).to(DEV)
+        counts = [len(p) for p in q_pos_list]
+        q_starts = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
+        seq_lens = torch.tensor([max(p) + 1 for p in q_pos_list], dtype=torch.int32, device=DEV)
+        out = torch.zeros((T, self.n_heads * self.hd), dtype=self.dtype, device=DEV)
+        scratch = torch.empty(1 << 22, dtype=torch.float32, device=DEV)
+        kernels().attention(q, out, self.kc.to(DEV), self.vc.to(DEV), self.tables.to(DEV), entry, pos, q_starts, seq_lens,
+                            self.n_heads, self.n_kv, self.hd, self.ps, self.num_pages, window, scale, scratch)
+        return out.cpu().view(T, self.n_heads, self.hd)
+
+    def reference(self, r, q, positions, window=0, scale=None):
+        """Plain attention of request r's queries, each over keys 0..its position."""
+        outs = []
+        for i, p in enumerate(positions):
+            n = p + 1
+            qq = torch.zeros((n, self.n_heads, self.hd), dtype=torch.float64)
+            qq[-1] = q[i].double()
+            o = plain_attention(qq, self.k[r][:n].double(), self.v[r][:n].double(), scale, window)
+            outs.append(o[-1])
+        return torch.stack(outs)
+
+
+ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 16), (8, 8, 64, 16), (8, 2, 128, 16), (6, 3, 48, 8), (5, 1, 80, 16),
+               (32, 8, 128, 16), (2, 2, 256, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps", ATTN_SHAPES)
+def test_attention_mixed_batch(dtype, n_heads, n_kv, hd, ps):
+    """A prompt portion, a whole prompt, and two decoding requests in one call."""
+    lens = [70, 37, 131, 16]
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=hd)
+    g = torch.Generator().manual_seed(1)
+    q_pos = [list(range(50, 70)), list(range(0, 37)), [130], [15]]
+    qs = [torch.randn((len(p), n_heads, hd), generator=g).to(dtype) for p in q_pos]
+    got = case.run(qs, q_pos)
+    at = 0
+    floor = 2e-6 if dtype == torch.float32 else 4e-3
+    for r, p in enumerate(q_pos):
+        ref = case.reference(r, qs[r], p)
+        err = (got[at:at + len(p)].double() - ref).abs()
+        assert (err <= out_tol(ref, dtype, floor)).all(), f"request {r}: max err {float(err.max())}"
+        at += len(p)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,ps,n", [(64, 16, 700), (128, 16, 1500), (32, 4, 300)])
+def test_attention_finds_a_far_key(dtype, hd, ps, n):
+    """Random keys hide a key that is skipped or read from the wrong page: here one
+    early key matches the query so strongly that the output must be its value."""
+    n_heads, n_kv = 4, 2
+    case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=3)
+    for far in (0, ps - 1, ps, n // 2 + 1, n - 2):
+        q = torch.zeros((1, n_heads, hd))
+        q[0, :, :] = case.k[0][far, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
+        got = case.run([q.to(dtype)], [[n - 1]])
+        want = case.v[0][far].float().repeat_interleave(n_heads // n_kv, dim=0)
+        ref = case.reference(0, q.to(dtype), [n - 1])
+        assert (ref[0].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
+        tol = 1e-4 if dtype == torch.float32 else 2e-2
+        assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64])
+def test_attention_window_edge(dtype, window):
+    """The key just outside the window must not be seen, the one just inside must."""
+    n_heads, n_kv, hd, ps, n = 2, 1, 32, 16, 90
+    case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=4)
+    p = n - 1
+    for key, visible in ((p - window, False), (p - window + 1, True)):
+        if key < 0:
+            continue
+        q = torch.zeros((1, n_heads, hd))
+        q[0] = case.k[0][key, 0].float() * 8.0
+        got = case.run([q.to(dtype)], [[p]], window=window)
+        ref = case.reference(0, q.to(dtype), [p], window=window)
+        tol = 1e-4 if dtype == torch.float32 else 2e-2
+        assert (got[0].float() - ref[0].float()).abs().max() <= tol
+        near = (got[0, 0].float() - case.v[0][key, 0].float()).abs().max() < 0.1
+        assert bool(near) == visible, f"window {window}: key {key} should {'' if visible else 'not '}be visible"
+
+
+def test_attention_pages_may_move():
+    """The same keys on other pages give the same result (bitwise: same order of sums)."""
+    a = PagedCase(torch.float32, [100], 4, 2, 32, 16, seed=5, extra_pages=1)
+    b = PagedCase(torch.float32, [100], 4, 2, 32, 16, seed=5, extra_pages=9)
+    assert not torch.equal(a.tables, b.tables[:, :a.tables.shape[1]])
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn((3, 4, 32), generator=g)
+    assert torch.equal(a.run([q], [[97, 98, 99]]), b.run([q], [[97, 98, 99]]))
+
+
+def test_argmax_rows():
+    V = 1003
+    logits = rnd((6, V + 5), torch.float32, 11)[:, :V]
+    logits[1, 77] = 50.0
+    logits[2, [5, 900]] = 60.0          # a tie: the lower index wins
+    logits[3, V - 1] = 70.0
+    logits[4] = -3.0                    # all equal
+    out = torch.zeros(6, dtype=torch.int32, device=DEV)
+    kernels().argmax_rows(logits, out)
+    want = [int(logits[0].argmax()), 77, 5, V - 1, 0, int(logits[5].argmax())]
+    assert out.tolist() == want
