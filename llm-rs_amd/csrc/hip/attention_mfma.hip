@@ -1,3 +1,287 @@
+// Paged causal attention on the matrix cores: bfloat16, pages of 16 slots,
+// head sizes that are multiples of 32, up to 32 query heads per kv head.
+//
+// A wave owns a tile of 32 "query columns": the heads of one kv group for as many
+// consecutive tokens of a request as fit (8 tokens x 4 heads for a 4:1 group; one
+// token's heads when decoding).  It walks the request's keys 32 at a time:
+//
+//   S^T[key, col] = sum_d K[key, d] Q[col, d]      v_mfma_f32_32x32x16_bf16, A = K rows
+//   online softmax down each column: a column is one lane pair, so the running
+//   maximum and sum need one exchange with lane ^ 32 and no LDS
+//   O^T[d, col]  += sum_key V^T[d, key] P^T[key, col]    A = V^T rows, B = P^T
+//
+// The accumulator of the first product is already the B operand of the second,
+// if row r of the K operand holds key (r with bits 2 and 3 swapped): then lane
+// half h holds, in registers 8s..8s+7, the probabilities of keys 16s + 8h + 0..7,
+// which are the 8 consecutive slots of page s that the V^T operand reads with one
+// 16-byte load (values lie [head_dim][slot] in a page).  No transpose, no LDS.
+//
+// Requests that bring one token (decoding) are split over waves by key range
+// (ATTN_CHUNK keys, aligned to absolute positions, so the split depends on the
+// request's length only) and merged in ascending order by a second kernel.
+//
+// Math as in the reference's paged_attention (shaders/ops.metal:636-758): scale
+// after the dot, mask = loop bound, max/exp/sums in 32-bit.  Probabilities are
+// rounded to bfloat16 for the second product; their sum is not.
 #include "attention.h"
-int llmrs_attention_bf16_mfma(hipStream_t, const bf16*, bf16*, const bf16*, const bf16*, const int*, const int*,
-                              const int*, const int*, const int*, int, float*, size_t, const AttnArgs&) { return 0; }
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define ATTN_CHUNK 128
+
+extern "C" int llmrs_attention_chunk() { return ATTN_CHUNK; }
+
+struct TileState {
+    float m, l;
+};
+
+// One wave: keys [t_begin, t_end) (t_begin a multiple of 32) against its 32 columns.
+// pos / lo: this lane's column may see keys lo..pos (pos < 0: nothing).
+template <int HD>
+__device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16 (&O)[HD / 32], float& m, float& l,
+                                             const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                             const int* __restrict__ table, int table_width, int num_pages,
+                                             int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale) {
+    int lane = threadIdx.x & 63;
+    int r = lane & 31, h = lane >> 5;
+    int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
+    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+        int lp = t0 >> 4;
+        int p0 = table[min(lp, table_width - 1)];
+        int p1 = (t0 + 16 < t_end) ? table[min(lp + 1, table_width - 1)] : p0;
+        p0 = min(max(p0, 0), num_pages - 1);
+        p1 = min(max(p1, 0), num_pages - 1);
+        const bf16* kp = kc + (((size_t)(kk < 16 ? p0 : p1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8;
+        f32x16 S;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < HD / 16; ++ks) {
+            bf16x8 kf = *(const bf16x8*)(kp + ks * 16);
+            S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
+        }
+        // values of both pages: issued here so that their latency hides behind the softmax
+        bf16x8 vf[HD / 32][2];
+        const bf16* vp0 = vc + (((size_t)p0 * n_kv + kvh) * HD + r) * 16 + h * 8;
+        const bf16* vp1 = vc + (((size_t)p1 * n_kv + kvh) * HD + r) * 16 + h * 8;
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+            vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
+            vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
+            float s = S[i] * scale;
+            s = (key > pos || key < lo) ? -INFINITY : s;
+            S[i] = s;
+            mx = fmaxf(mx, s);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float m_new = fmaxf(m, mx);
+        float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        float alpha = expf(m - m_safe);
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            S[i] = expf(S[i] - m_safe);
+            sum += S[i];
+        }
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * alpha + sum;
+        m = m_new;
+        bf16x8 pf[2];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pf[0][i] = (bf16)S[i];
+            pf[1][i] = (bf16)S[8 + i];
+        }
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pf[0], O[dt], 0, 0, 0);
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pf[1], O[dt], 0, 0, 0);
+        }
+    }
+}
+
+// Feature that register i of O^T tile dt holds in lane half h.
+__device__ __forceinline__ int o_feature(int dt, int i, int h) { return dt * 32 + 8 * (i >> 2) + 4 * h + (i & 3); }
+
+// ---- entries with several tokens (and, when nothing is split, all entries) --
+template <int HD>
+__global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
+                                                         const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                                         const int* __restrict__ block_table,
+                                                         const int* __restrict__ positions,
+                                                         const int* __restrict__ q_starts, int n_entries,
+                                                         AttnArgs a, int G, int tpt, int skip_single) {
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int c = lane & 31, h = lane >> 5;
+    int task = blockIdx.x * 4 + wave;
+    int kvh = (task >> 2) % a.n_kv_heads;
+    int tile = (task / (4 * a.n_kv_heads)) * 4 + (task & 3);
+    int e = 0, rem = tile;
+    for (; e < n_entries; ++e) {
+        int cnt = q_starts[e + 1] - q_starts[e];
+        int nt = (cnt == 1 && skip_single) ? 0 : (cnt + tpt - 1) / tpt;
+        if (rem < nt) break;
+        rem -= nt;
+    }
+    if (e == n_entries) return;
+    int tok0 = q_starts[e] + rem * tpt;
+    int ntok = min(tpt, q_starts[e + 1] - tok0);
+    int tq = c / G, hg = c - tq * G;
+    bool cvalid = tq < ntok;
+    int token = tok0 + min(tq, ntok - 1);
+    int head = kvh * G + hg;
+    int pos = cvalid ? positions[token] : -1;
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int last = positions[tok0 + ntok - 1], first = positions[tok0];
+    int t_end = last + 1;
+    int t_begin = ((a.window > 0 && first + 1 > a.window) ? first + 1 - a.window : 0) & ~31;
+
+    bf16x8 qf[HD / 16];
+    const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+    f32x16 O[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
+                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo, a.scale);
+    if (!cvalid) return;
+    float inv = 1.0f / l;
+    bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            bf16x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv);
+            *(bf16x4*)(op + o_feature(dt, i4 * 4, h)) = v;
+        }
+}
+
+// ---- entries with one token: a wave for each (entry, kv head, chunk of keys) --
+// partial: [(entry * n_heads + head) * max_chunks + chunk][HD + 2] = m, l, O (not yet divided)
+template <int HD>
+__global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
+                                                        const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                                        const int* __restrict__ block_table,
+                                                        const int* __restrict__ positions,
+                                                        const int* __restrict__ q_starts, AttnArgs a, int G,
+                                                        int max_chunks) {
+    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z;
+    if (q_starts[e + 1] - q_starts[e] != 1) return;
+    int token = q_starts[e];
+    int pos_t = positions[token];
+    int lo_t = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
+    int first_chunk = lo_t / ATTN_CHUNK;
+    int n_chunks = pos_t / ATTN_CHUNK - first_chunk + 1;
+    if (ch >= n_chunks) return;
+    int t_begin = (first_chunk + ch) * ATTN_CHUNK;
+    int t_end = min(t_begin + ATTN_CHUNK, pos_t + 1);
+    int lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
+    bool cvalid = c < G;
+    int head = kvh * G + min(c, G - 1);
+    int pos = cvalid ? pos_t : -1;
+
+    bf16x8 qf[HD / 16];
+    const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+    f32x16 O[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
+                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale);
+    if (!cvalid) return;
+    float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
+    if (h == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) pp[2 + o_feature(dt, i, h)] = O[dt][i];
+}
+
+__global__ void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
+                                  const int* __restrict__ positions, const int* __restrict__ q_starts, AttnArgs a,
+                                  int max_chunks) {
+    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim;
+    if (q_starts[e + 1] - q_starts[e] != 1) return;
+    int token = q_starts[e];
+    int pos = positions[token];
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int n_chunks = pos / ATTN_CHUNK - lo / ATTN_CHUNK + 1;
+    const float* pp = partial + (size_t)(e * a.n_heads + head) * max_chunks * (hd + 2);
+    float M = -INFINITY;
+    for (int ch = 0; ch < n_chunks; ++ch) M = fmaxf(M, pp[(size_t)ch * (hd + 2)]);
+    float L = 0.0f;
+    for (int ch = 0; ch < n_chunks; ++ch) L += pp[(size_t)ch * (hd + 2) + 1] * expf(pp[(size_t)ch * (hd + 2)] - M);
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float o = 0.0f;
+        for (int ch = 0; ch < n_chunks; ++ch)   // ascending chunks: a fixed order
+            o += pp[(size_t)ch * (hd + 2) + 2 + d] * expf(pp[(size_t)ch * (hd + 2)] - M);
+        out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / L);
+    }
+}
+
+template <int HD>
+static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
+                  const int* positions, const int* q_starts, int n_entries, float* scratch, size_t scratch_bytes,
+                  int max_seq_len, const AttnArgs& a) {
+    int G = a.n_heads / a.n_kv_heads;
+    int tpt = 32 / G;
+    int max_chunks = max_seq_len > 0 ? (max_seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK : 0;
+    size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
+    // Split the single-token entries when the caller gave room for their partial results.
+    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= 65535;
+    int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
+    if (!only_single) {
+        int tiles = a.n_tokens / tpt + n_entries;
+        int blocks = ((tiles + 3) / 4) * a.n_kv_heads;
+        attn_tiles_kernel<HD><<<blocks, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts, n_entries, a, G, tpt, split);
+    }
+    if (split) {
+        dim3 grid(n_entries, a.n_kv_heads, max_chunks);
+        attn_split_kernel<HD><<<grid, 64, 0, stream>>>(q, scratch, kc, vc, table, positions, q_starts, a, G, max_chunks);
+        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, positions, q_starts, a, max_chunks);
+    }
+    return 1;
+}
+
+int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, const bf16* k_cache, const bf16* v_cache,
+                              const int* block_table, const int* token_entry, const int* positions,
+                              const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
+                              size_t scratch_bytes, int max_seq_len, const AttnArgs& a) {
+    (void)token_entry; (void)seq_lens;
+    int G = a.n_heads / a.n_kv_heads;
+    if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
+    if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
+    if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;
+    int rc;
+    switch (a.head_dim) {
+#define CASE(HD) case HD: rc = launch<HD>(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, n_entries, scratch, scratch_bytes, max_seq_len, a); break;
+        CASE(32) CASE(64) CASE(96) CASE(128) CASE(192) CASE(256)
+#undef CASE
+        default: return 0;
+    }
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        llmrs_fail("attention (mfma): launch failed: %s", hipGetErrorString(err));
+        return -1;
+    }
+    return rc;
+}

@@ -46,7 +46,7 @@ class StepContext:
         self.slot_maps: List[torch.Tensor] = []
         self.block_tables: List[torch.Tensor] = []
         self.entries: List[Tuple[int, int, int]] = []   # host copy: (slot, start, count)
-        self.scratch: Optional[torch.Tensor] = None
+        self.max_seq_len = 0                            # largest start + count among the entries
         self.device = runner.device
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
@@ -63,11 +63,6 @@ class StepRunner:
         self._turn = 0
         self._dev_words = torch.zeros(words_capacity, dtype=torch.int32, device=self.device)
         self.ctx = StepContext(self)
-        # partial results of split attention over long contexts
-        self.ctx.scratch = torch.empty(self.attention_scratch_floats(), dtype=torch.float32, device=self.device)
-
-    def attention_scratch_floats(self) -> int:
-        return 1 << 22
 
     def _new_host(self, n: int) -> torch.Tensor:
         return torch.zeros(n, dtype=torch.int32, pin_memory=self._pinned)
@@ -120,6 +115,7 @@ class StepRunner:
         c = self.ctx
         c.n_tokens, c.n_entries, c.n_want = T, R, n_want
         c.entries = entries
+        c.max_seq_len = max(start + count for _, start, count in entries)
         c.tokens = dev[off.tokens:off.tokens + T]
         c.positions = dev[off.positions:off.positions + T]
         c.token_entry = dev[off.token_entry:off.token_entry + T]

@@ -52,8 +52,9 @@ class HipKernels:
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
             "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
-            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I],
+            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I],
             "llmrs_argmax_rows": [V, V, I, I, I, V],
+            "llmrs_sample_rows": [V, V, I, I, I, V, V],
         }
         for name, args in sigs.items():
             fn = getattr(lib, name)
@@ -67,6 +68,12 @@ class HipKernels:
         if not self.arch.startswith("gfx950"):
             raise KernelError(f"the kernel library is built for gfx950, the device is {self.arch!r}")
         self.allow_mfma = True  # tests switch the matrix-core kernels off to compare paths
+        lib.llmrs_attention_chunk.restype = I
+        self.attention_chunk = lib.llmrs_attention_chunk()
+
+    def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int) -> int:
+        """Room the split of single-token entries needs for its partial results."""
+        return n_entries * n_heads * (-(-max_seq_len // self.attention_chunk)) * (head_dim + 2)
 
     def _check(self, rc: int) -> None:
         if rc != 0:
@@ -117,7 +124,7 @@ class HipKernels:
             page_size, num_pages, int(write_kv)))
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None) -> None:
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0) -> None:
         assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
@@ -127,12 +134,20 @@ class HipKernels:
             self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
             _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
             block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
-            _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(self.allow_mfma)))
+            _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
+            int(self.allow_mfma)))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor) -> None:
         assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
         self._check(self.lib.llmrs_argmax_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
                                                logits.shape[1], _p(out)))
+
+    # words[i] = uniform (float bits), temperature (float bits), top_k, top_p (float bits) of row i
+    def sample_rows(self, logits: torch.Tensor, words: torch.Tensor, out: torch.Tensor) -> None:
+        assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
+        assert words.dtype == torch.int32 and words.is_contiguous() and words.shape == (logits.shape[0], 4)
+        self._check(self.lib.llmrs_sample_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
+                                               logits.shape[1], _p(words), _p(out)))
 
 
 _kernels = None

@@ -80,9 +80,12 @@ class Attention(Mixer):
             k.rope_kv_write(qkv, ctx.positions, ctx.slot_maps[g], inv_freq, rotary_dim, interleaved,
                             cache.k, cache.v, self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
         o = ctx.workspace("attn.out", (T, self.q_size), self.dtype)
+        # room for the partial results of single-token entries, which the kernel splits by key range
+        need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len)
+        scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
-                    cache.num_pages, self.window, self.scale, ctx.scratch)
+                    cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32)
 
 

@@ -15,6 +15,9 @@ EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 class EmulatedKernels:
     allow_mfma = False
 
+    def attention_scratch_floats(self, n_entries, n_heads, head_dim, max_seq_len):
+        return 0
+
     def embed_rows(self, out, table, tokens):
         out.copy_(table[tokens.long()].float())
 
@@ -66,7 +69,7 @@ class EmulatedKernels:
             vc[page[t], :, :, off[t]] = heads[t, n_rot:, :]
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None):
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0):
         T = q.shape[0]
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
         vc = v_cache.view(num_pages, n_kv_heads, head_dim, page_size).float()

@@ -183,7 +183,8 @@ class PagedCase:
         out = torch.zeros((T, self.n_heads * self.hd), dtype=self.dtype, device=DEV)
         scratch = torch.empty(1 << 22, dtype=torch.float32, device=DEV)
         kernels().attention(q, out, self.kc.to(DEV), self.vc.to(DEV), self.tables.to(DEV), entry, pos, q_starts, seq_lens,
-                            self.n_heads, self.n_kv, self.hd, self.ps, self.num_pages, window, scale, scratch)
+                            self.n_heads, self.n_kv, self.hd, self.ps, self.num_pages, window, scale, scratch,
+                            max(max(p) + 1 for p in q_pos_list))
         return out.cpu().view(T, self.n_heads, self.hd)
 
     def reference(self, r, q, positions, window=0, scale=None):
@@ -280,3 +281,73 @@ def test_argmax_rows():
     kernels().argmax_rows(logits, out)
     want = [int(logits[0].argmax()), 77, 5, V - 1, 0, int(logits[5].argmax())]
     assert out.tolist() == want
+
+
+def _words(rows):
+    """[(uniform, temperature, top_k, top_p)] -> the int32 words the sampler reads."""
+    w = torch.zeros((len(rows), 4), dtype=torch.int32)
+    for i, (u, t, k, p) in enumerate(rows):
+        f = torch.tensor([u, t, p], dtype=torch.float32).view(torch.int32)
+        w[i, 0], w[i, 1], w[i, 2], w[i, 3] = f[0], f[1], k, f[2]
+    return w.to(DEV)
+
+
+@pytest.mark.parametrize("V", [1003, 5000])
+def test_sample_rows_against_plain(V):
+    """The token must be the one whose interval of the plain implementation's cumulative
+    distribution (float64) holds the uniform; a uniform within 1e-5 of an interval's edge
+    may fall to either side, since the kernel sums in 32-bit."""
+    from plain_llama import plain_probabilities
+    g = torch.Generator().manual_seed(V)
+    settings = [(0.8, 0, 1.0), (0.7, 40, 0.9), (1.3, 5, 1.0), (0.5, 0, 0.8), (1.0, 3000, 0.95), (2.0, 1, 1.0),
+                (0.9, 40, 0.3), (1.0, 0, 0.999)]
+    rows, logit_rows = [], []
+    for (t, k, p) in settings:
+        for _ in range(6):
+            rows.append((float(torch.rand(1, generator=g)), t, k, p))
+            logit_rows.append(torch.randn(V, generator=g) * 3.0)
+    rows.append((0.3, 0.0, 0, 1.0))                     # a greedy row among the others
+    logit_rows.append(torch.randn(V, generator=g))
+    logits = torch.stack(logit_rows).to(DEV)
+    out = torch.zeros(len(rows), dtype=torch.int32, device=DEV)
+    kernels().sample_rows(logits, _words(rows), out)
+    out = out.tolist()
+    for i, (u, t, k, p) in enumerate(rows):
+        if t == 0.0:
+            assert out[i] == int(logit_rows[i].argmax())
+            continue
+        prob = plain_probabilities(logit_rows[i], t, k, p)
+        cum = torch.cumsum(prob, 0)
+        tok = out[i]
+        assert prob[tok] > 0, f"row {i}: token {tok} is outside the kept set (T={t} k={k} p={p})"
+        lo = float(cum[tok] - prob[tok])
+        assert lo - 1e-5 <= u < float(cum[tok]) + 1e-5, f"row {i}: u={u} not in [{lo}, {float(cum[tok])}) of token {tok}"
+
+
+def test_sample_rows_ties_and_edges():
+    V = 300
+    logits = torch.full((4, V), -2.0)
+    logits[0, [10, 20, 30]] = 5.0          # three equal maxima, top_k 2: the two lowest indices stay
+    logits[1, [10, 20, 30]] = 5.0          # top_p cut through equal values
+    logits[2, 7] = 9.0                     # u close to 1 still lands on a kept token
+    logits[3, :] = 0.0                     # uniform distribution, top_k 1 -> index 0
+    rows = [(0.99, 1.0, 2, 1.0), (0.6, 1.0, 0, 0.5), (0.999999, 1.0, 5, 0.9), (0.5, 1.0, 1, 1.0)]
+    out = torch.zeros(4, dtype=torch.int32, device=DEV)
+    kernels().sample_rows(logits.to(DEV), _words(rows), out)
+    out = out.tolist()
+    assert out[0] == 20 and out[1] == 20 and out[3] == 0
+    assert out[2] == 7
+
+
+def test_sample_rows_frequencies():
+    """Many draws from one row: observed frequencies match the softmax."""
+    V, n = 50, 4000
+    g = torch.Generator().manual_seed(1)
+    row = torch.randn(V, generator=g) * 2
+    us = torch.rand(n, generator=g)
+    rows = [(float(u), 1.0, 0, 1.0) for u in us]
+    out = torch.zeros(n, dtype=torch.int32, device=DEV)
+    kernels().sample_rows(row.repeat(n, 1).to(DEV), _words(rows), out)
+    freq = torch.bincount(out.cpu().long(), minlength=V).double() / n
+    p = torch.softmax(row.double(), 0)
+    assert (freq - p).abs().max() < 4 * (p * (1 - p) / n).sqrt().max() + 1e-3
