@@ -46,6 +46,7 @@ def _lib():
             "llmrs_request_info": [c_void_p, c_int, c_void_p],
             "llmrs_request_output": [c_void_p, c_int, c_void_p, c_int],
             "llmrs_request_drop": [c_void_p, c_int],
+            "llmrs_request_abort": [c_void_p, c_int],
         }.items():
             fn = getattr(lib, name)
             fn.argtypes = args
@@ -206,6 +207,10 @@ class HostCore:
 
     def drop_request(self, slot: int) -> None:
         self._check(self._lib.llmrs_request_drop(self._h, slot))
+
+    def abort_request(self, slot: int) -> None:
+        """Ends a request wherever it stands; its pages and its slot go back."""
+        self._check(self._lib.llmrs_request_abort(self._h, slot))
 
 
 def xorshift64_stream(seed: int, n: int) -> List[int]:

@@ -214,6 +214,7 @@ int llmrs_request_output(void* h, int slot, int32_t* out, int cap) {
     });
 }
 
+int llmrs_request_abort(void* h, int slot) { auto c = (Core*)h; return guarded(c, [&] { c->scheduler->abort(slot); return 0; }); }
 int llmrs_request_drop(void* h, int slot) { auto c = (Core*)h; return guarded(c, [&] { c->scheduler->drop(slot); return 0; }); }
 
 // The reference's generator, for callers that sample outside the scheduler.

@@ -157,7 +157,19 @@ std::vector<int> Scheduler::commit(const int32_t* sampled, int n_sampled) {
     return finished;
 }
 
+void Scheduler::abort(int slot) {
+    if (slot < 0 || slot >= (int)requests_.size() || requests_[slot].phase == Phase::Free)
+        throw std::logic_error("slot " + std::to_string(slot) + " holds no request");
+    running_.erase(std::remove(running_.begin(), running_.end(), slot), running_.end());
+    waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), slot), waiting_.end());
+    plan_.erase(std::remove_if(plan_.begin(), plan_.end(), [&](const PlannedEntry& p) { return p.entry.slot == slot; }),
+                plan_.end());
+    requests_[slot] = Request();
+    cache_.release_slot(slot);
+}
+
 void Scheduler::drop(int slot) {
+    if (slot < 0 || slot >= (int)requests_.size()) throw std::logic_error("no such slot");
     Request& r = requests_[slot];
     if (r.phase != Phase::Finished) throw std::logic_error("slot " + std::to_string(slot) + " holds no finished request");
     r = Request();

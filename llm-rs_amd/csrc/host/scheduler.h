@@ -79,6 +79,7 @@ public:
 
     const Request& request(int slot) const { return requests_[slot]; }
     void drop(int slot);  // forget a finished request, free its slot
+    void abort(int slot); // end a request wherever it stands: pages and slot go back
     int num_running() const { return (int)running_.size(); }
     int num_waiting() const { return (int)waiting_.size(); }
     int64_t preemptions() const { return preemptions_; }

@@ -49,6 +49,9 @@ class Engine:
         self.dtype = _DTYPES[dtype]
         self.device = torch.device(device)
         self.log = log
+        if self.device.type == "cuda":
+            from ..kernels import kernels
+            kernels()    # no GPU or no kernel library: fail here, with that message, before any weight moves
         spec = config.model_spec()
         self.model = Model(spec, self.dtype, self.device)
         self.model.load(tensors)
@@ -152,23 +155,28 @@ class Engine:
                 slot_of[slot] = i
                 pending.pop(0)
 
-        admit()
-        while not core.idle() or pending:
-            logits, n_want, plan = self.runner.run_planned()
-            if not plan:
-                raise RuntimeError("the scheduler planned nothing although requests are waiting")
-            sampled = []
-            if n_want:
-                sampled = self.sampler.sample(logits, self.runner.ctx.sampling, all_greedy).cpu().numpy()
-                if stats.first_token_seconds == 0.0:
-                    stats.first_token_seconds = time.perf_counter() - t0
-            stats.steps += 1
-            for slot in core.commit(sampled):
-                info = core.request_info(slot)
-                i = slot_of.pop(slot)
-                results[i] = Finished(core.request_output(slot), "stop" if info["finish"] == 1 else "length")
-                core.drop_request(slot)
+        try:
             admit()
+            while not core.idle() or pending:
+                logits, n_want, plan = self.runner.run_planned()
+                if not plan:
+                    raise RuntimeError("the scheduler planned nothing although requests are waiting")
+                sampled = []
+                if n_want:
+                    sampled = self.sampler.sample(logits, self.runner.ctx.sampling, all_greedy).cpu().numpy()
+                    if stats.first_token_seconds == 0.0:
+                        stats.first_token_seconds = time.perf_counter() - t0
+                stats.steps += 1
+                for slot in core.commit(sampled):
+                    info = core.request_info(slot)
+                    i = slot_of.pop(slot)
+                    results[i] = Finished(core.request_output(slot), "stop" if info["finish"] == 1 else "length")
+                    core.drop_request(slot)
+                admit()
+        except BaseException:
+            for slot in list(slot_of):      # leave the engine as it was found
+                core.abort_request(slot)
+            raise
         if self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         stats.seconds = time.perf_counter() - t0

@@ -127,8 +127,9 @@ def plain_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_do
 # ---- the model -----------------------------------------------------------------
 
 def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
-                  compute: torch.dtype = torch.float64, layout: str = "split_half") -> torch.Tensor:
-    """Logits [T, vocab] for one whole sequence from position 0.  Layer loop of
+                  compute: torch.dtype = torch.float64, layout: str = "split_half",
+                  position_offset: int = 0) -> torch.Tensor:
+    """Logits [T, vocab] for one whole sequence from position 0 (or `position_offset`).  Layer loop of
     src/arch/llama.rs:150-171, final norm and output matrix of :135-139; tied
     embeddings reuse the token table (:81)."""
     W = {n: t.to(compute) for n, t in weights.items()}
@@ -138,7 +139,7 @@ def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[
     eps = cfg.get("rms_norm_eps", 1e-5)
     inv_freq = plain_inv_freq(d, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
     T = len(tokens)
-    pos = torch.arange(T)
+    pos = torch.arange(T) + position_offset
     x = plain_embedding(W["model.embed_tokens.weight"], tokens)
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."

@@ -1,0 +1,157 @@
+"""Generation through the Python entry point: greedy against the plain
+implementation, long decoding, the first tokens of a sequence, batching that
+does not change outputs, seeds that reproduce, a pool so small that requests are
+preempted and computed again."""
+import pytest
+import torch
+
+from llm_rs_amd import Engine, StepEntry
+from plain_llama import plain_forward, plain_generate, read_model_folder
+from replay_cases import random_tokens
+from replay_checks import TOLERANCE
+from tiny_configs import CONFIGS, PAGE_SIZE, make_folder
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    d = tmp_path_factory.mktemp("models")
+    return {w: make_folder(d, w, seed=7) for w in "AB"}
+
+
+def engine(folder, which, dtype, **kw):
+    kw.setdefault("num_pages", 256)
+    kw.setdefault("max_requests", 16)
+    return Engine.from_folder(folder, dtype=dtype, page_size=PAGE_SIZE[which], **kw)
+
+
+def check_greedy_path(cfg, weights, prompt, out, dtype):
+    """Every generated token is the plain implementation's choice given the same
+    prefix, or (bfloat16) so close to it that rounding decides."""
+    logits = plain_forward(cfg, weights, prompt + out)
+    scale = max(float(logits.abs().max()), 1.0)
+    for i, tok in enumerate(out):
+        row = logits[len(prompt) - 1 + i]
+        gap = float(row.max() - row[tok])
+        assert gap <= 2 * TOLERANCE[dtype] * scale, f"token {i}: engine chose {tok}, plain prefers {int(row.argmax())} by {gap}"
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_matches_plain_float32(folders, which):
+    cfg, weights = read_model_folder(folders[which])
+    eng = engine(folders[which], which, "float32")
+    lengths = {"A": [5, 17, 33], "B": [1, 7, 64]}[which]
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=n) for n in lengths]
+    got = eng.generate(prompts, max_new_tokens=16)
+    for p, out in zip(prompts, got):
+        assert len(out) == 16
+        check_greedy_path(cfg, weights, p, out, "float32")
+    want = [plain_generate(cfg, weights, p, 16) for p in prompts[:2]]
+    assert got[:2] == want
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_greedy_bfloat16(folders, which):
+    cfg, weights = read_model_folder(folders[which])
+    eng = engine(folders[which], which, "bfloat16")
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=100 + n) for n in (3, 20, 41)]
+    for p, out in zip(prompts, eng.generate(prompts, max_new_tokens=24)):
+        check_greedy_path(cfg, weights, p, out, "bfloat16")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """A short prompt and then hundreds of tokens one by one, to the model's last position."""
+    which = "B"
+    cfg, weights = read_model_folder(folders[which])
+    toks = random_tokens(cfg["vocab_size"], cfg["max_position_embeddings"], seed=1)
+    ref = plain_forward(cfg, weights, toks)
+    eng = engine(folders[which], which, dtype)
+    s = eng.open_request()
+    rows = [eng.step([StepEntry(s, 0, toks[:9], list(range(9)))]).clone()]
+    for i in range(9, len(toks)):
+        rows.append(eng.step([StepEntry(s, i, [toks[i]], [0])]).clone())
+    eng.close_request(s)
+    got = torch.cat(rows).double().cpu()
+    err = (got - ref).abs().max(dim=1).values / max(float(ref.abs().max()), 1.0)
+    bad = (err > TOLERANCE[dtype]).nonzero()
+    assert len(bad) == 0, f"first wrong position {int(bad[0])}: {float(err[int(bad[0])])}"
+    with pytest.raises(ValueError, match="beyond the model"):
+        s = eng.open_request()
+        eng.step([StepEntry(s, 0, toks + [1], [])])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(folders, dtype):
+    """Positions 0, 1, 2: one-token prompts, alone and side by side."""
+    which = "A"
+    cfg, weights = read_model_folder(folders[which])
+    eng = engine(folders[which], which, dtype)
+    seqs = [random_tokens(cfg["vocab_size"], 3, seed=s) for s in range(4)]
+    slots = [eng.open_request() for _ in seqs]
+    scale_tol = TOLERANCE[dtype]
+    for pos in range(3):
+        out = eng.step([StepEntry(s, pos, [seq[pos]], [0]) for s, seq in zip(slots, seqs)]).double().cpu()
+        for i, seq in enumerate(seqs):
+            ref = plain_forward(cfg, weights, seq[:pos + 1])[-1]
+            assert float((out[i] - ref).abs().max()) <= scale_tol * max(float(ref.abs().max()), 1.0), (pos, i)
+
+
+def test_batching_and_seeds_do_not_change_outputs(folders):
+    which = "B"
+    cfg, _ = read_model_folder(folders[which])
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=50 + n) for n in (1, 7, 64, 130, 300)]
+    kw = dict(max_new_tokens=24, temperature=0.8, top_k=40, top_p=0.9, seed=42)
+    together = engine(folders[which], which, "float32", max_chunk=32).generate(prompts, **kw)
+    alone_eng = engine(folders[which], which, "float32")
+    alone = [alone_eng.generate([p], **kw)[0] for p in prompts]
+    assert together == alone, "a request's tokens do not depend on what it is batched with or how its prompt was cut"
+    assert together == engine(folders[which], which, "float32", max_chunk=32).generate(prompts, **kw), "same seed, same tokens"
+    other = alone_eng.generate(prompts, **{**kw, "seed": 43})
+    assert other != together, "another seed draws other tokens"
+    per_request = alone_eng.generate(prompts[:2], **{**kw, "seed": [42, 43]})
+    assert per_request[0] == together[0] and per_request[1] == other[1]
+
+
+def test_sampled_tokens_follow_the_plain_sampler(folders):
+    """Temperature sampling end to end in float32: the same tokens as the plain
+    implementation drawing from the same generator."""
+    which = "A"
+    cfg, weights = read_model_folder(folders[which])
+    eng = engine(folders[which], which, "float32")
+    prompt = random_tokens(cfg["vocab_size"], 6, seed=3)
+    got = eng.generate([prompt], max_new_tokens=12, temperature=0.8, seed=7)[0]
+    assert got == plain_generate(cfg, weights, prompt, 12, temperature=0.8, seed=7)
+    got = eng.generate([prompt], max_new_tokens=12, temperature=1.1, top_k=5, top_p=0.7, seed=0)[0]
+    assert got == plain_generate(cfg, weights, prompt, 12, temperature=1.1, top_k=5, top_p=0.7, seed=0)
+
+
+def test_stop_tokens_and_reasons(folders):
+    which = "B"
+    cfg, weights = read_model_folder(folders[which])
+    eng = engine(folders[which], which, "float32")
+    prompt = random_tokens(cfg["vocab_size"], 7, seed=9)
+    free = eng.generate([prompt], max_new_tokens=10)[0]
+    res = eng.generate([prompt], max_new_tokens=10, stop_token_ids=[free[4]], return_reasons=True)[0]
+    first = free.index(free[4])
+    assert res.tokens == free[:first] and res.reason == "stop", "the stop token ends the output and is not part of it"
+    assert eng.generate([prompt], max_new_tokens=3, return_reasons=True)[0].reason == "length"
+    assert eng.generate([prompt], max_new_tokens=0) == [[]]
+
+
+def test_small_pool_preempts_and_recomputes(folders):
+    """So few pages that running requests cannot all grow: some are evicted, wait, and are
+    computed again; every output equals the run with plenty of pages."""
+    which = "B"
+    cfg, _ = read_model_folder(folders[which])
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=70 + n) for n in (30, 45, 20, 60, 10, 33)]
+    kw = dict(max_new_tokens=40, temperature=0.7, seed=5)
+    roomy = engine(folders[which], which, "float32").generate(prompts, **kw)
+    tight = engine(folders[which], which, "float32", num_pages=14, max_chunk=16)      # 224 token slots for ~480 tokens of need
+    assert tight.generate(prompts, **kw) == roomy
+    assert tight.last_stats.preemptions > 0, "the case must make the scheduler evict"
+    core = tight.cache.core
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
+    with pytest.raises(Exception, match="pages"):
+        tight.generate([random_tokens(cfg["vocab_size"], 200, seed=1)], max_new_tokens=100)

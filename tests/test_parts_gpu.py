@@ -1,0 +1,298 @@
+"""Each part alone against the plain function of its formula, and the generality
+of how parts are put together: a sliding-window attention, a schedule that runs
+a layer twice and lets a run read another run's cache, and a toy mixer with
+state of its own that is defined and registered here, in the test, and built and
+stepped without a change to the package."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from llm_rs_amd import (Engine, FixedState, LayerSpec, ModelSpec, PartSpec, RunSpec, StepEntry, StepRunner,
+                        register_architecture)
+from llm_rs_amd.cache import CacheManager, PagedKV
+from llm_rs_amd.parts import (Mixer, TensorSpec, build_block, build_feed_forward, build_mixer, build_norm,
+                              build_position, register_mixer)
+from plain_llama import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope, plain_swiglu
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.float32: 2e-5, torch.bfloat16: 1.5e-2}
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+class Harness:
+    """Runs `fn(ctx, cache_views)` as a step's model, over a real cache manager and step function."""
+
+    def __init__(self, needs, dtype, page_size=16, num_pages=64):
+        self.cache = CacheManager(needs, dtype, DEV, page_size, num_pages, max_requests=8)
+        self.stub = SimpleNamespace(spec=SimpleNamespace(vocab_size=1 << 30, max_positions=1 << 20), forward=None)
+        self.runner = StepRunner(self.stub, self.cache, DEV)
+
+    def run(self, entries, fn):
+        self.stub.forward = fn
+        return self.runner.run(entries)
+
+
+def close(got, ref, dtype):
+    scale = max(float(ref.abs().max()), 1.0)
+    return float((got.double().cpu() - ref).abs().max()) <= TOL[dtype] * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(dtype):
+    norm = build_norm(PartSpec("rmsnorm", "n", {"size": 72, "eps": 1e-3}), dtype)
+    assert norm.tensors() == {"n.weight": TensorSpec((72,), "norm")}
+    w = rnd((72,), 0) * 0.1 + 1
+    norm.load({"n.weight": w.bfloat16()}, DEV)
+    assert norm.weight.dtype == torch.float32
+    h = rnd((5, 72), 1, 2.0).to(DEV)
+    out = torch.empty((5, 72), dtype=dtype, device=DEV)
+    norm.forward(None, h, out)
+    assert close(out, plain_rmsnorm(h.double().cpu(), w.bfloat16().double(), 1e-3), dtype)
+
+
+def test_rotary_part_makes_the_table():
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=64)
+    rope = build_position({"kind": "rope", "head_dim": 48, "rotary_dim": 32, "theta": 500000.0, "layout": "interleaved", "scaling": sc}, torch.float32)
+    table, rotary_dim, interleaved = rope.rotary()
+    assert rotary_dim == 32 and interleaved and torch.equal(table, plain_inv_freq(32, 500000.0, sc))
+    assert build_position(None, torch.float32) is None
+    with pytest.raises(KeyError, match="unknown position encoding"):
+        build_position({"kind": "alibi"}, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part(dtype):
+    ffn = build_feed_forward(PartSpec("swiglu", "f", {"hidden_size": 40, "intermediate_size": 88}), dtype)
+    ws = {"f.gate_proj.weight": rnd((88, 40), 2, 0.2).bfloat16(), "f.up_proj.weight": rnd((88, 40), 3, 0.2).bfloat16(),
+          "f.down_proj.weight": rnd((40, 88), 4, 0.2).bfloat16()}
+    assert {n: t.shape for n, t in ffn.tensors().items()} == {n: tuple(t.shape) for n, t in ws.items()}
+    ffn.load(ws, DEV)
+    x = rnd((7, 40), 5).to(dtype)
+    h0 = rnd((7, 40), 6)
+    hz = Harness([], dtype)
+    out = {}
+
+    def fn(ctx, views):
+        h = h0.to(DEV).clone()
+        ffn.forward(ctx, x.to(DEV), h)
+        out["h"] = h
+    s = hz.cache.core.acquire_slot()
+    hz.run([StepEntry(s, 0, [0] * 7, [])], fn)
+    ref = h0.double() + plain_swiglu(x.double(), *(ws[k].double() for k in ("f.gate_proj.weight", "f.up_proj.weight", "f.down_proj.weight")))
+    assert close(out["h"], ref, dtype)
+
+
+def attention_reference(ws, prefix, x, heads, kv, hd, rope, window, scale=None):
+    T = x.shape[0]
+    q = (x @ ws[f"{prefix}.q_proj.weight"].double().T).view(T, heads, hd)
+    k = (x @ ws[f"{prefix}.k_proj.weight"].double().T).view(T, kv, hd)
+    v = (x @ ws[f"{prefix}.v_proj.weight"].double().T).view(T, kv, hd)
+    if rope is not None:
+        inv = plain_inv_freq(rope["rotary_dim"], rope["theta"], rope.get("scaling"))
+        pos = torch.arange(T)
+        q, k = plain_rope(q, pos, inv, rope["layout"]), plain_rope(k, pos, inv, rope["layout"])
+    o = plain_attention(q, k, v, scale, window).reshape(T, heads * hd)
+    return o @ ws[f"{prefix}.o_proj.weight"].double().T
+
+
+ATTN_CASES = [
+    dict(hidden=40, heads=4, kv=2, hd=16, window=None, rotary=16, layout="split_half", ps=4),
+    dict(hidden=72, heads=6, kv=2, hd=32, window=None, rotary=32, layout="split_half", ps=16),
+    dict(hidden=64, heads=4, kv=4, hd=32, window=9, rotary=16, layout="interleaved", ps=16),      # a window, part of the head rotated
+    dict(hidden=48, heads=2, kv=1, hd=64, window=20, rotary=0, layout="split_half", ps=16),        # no position encoding at all
+    dict(hidden=56, heads=3, kv=3, hd=48, window=None, rotary=48, layout="split_half", ps=8),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_attention_part(dtype, case):
+    c = SimpleNamespace(**case)
+    rope = None if c.rotary == 0 else {"kind": "rope", "head_dim": c.hd, "rotary_dim": c.rotary, "theta": 10000.0, "layout": c.layout}
+    att = build_mixer(PartSpec("attention", "a", {"hidden_size": c.hidden, "num_heads": c.heads, "num_kv_heads": c.kv,
+                                                  "head_dim": c.hd, "window": c.window, "position": rope}), dtype)
+    assert att.cache_need() == PagedKV(c.kv, c.hd, c.window or 0)
+    ws = {n: rnd(s.shape, i, 0.15).bfloat16() for i, (n, s) in enumerate(att.tensors().items())}
+    att.load(ws, DEV)
+    T = 45
+    x = rnd((T, c.hidden), 9).to(dtype)
+    ref = attention_reference(ws, "a", x.double(), c.heads, c.kv, c.hd, rope, c.window or 0)
+    hz = Harness([(att.cache_need(), None)], dtype, page_size=c.ps)
+    s = hz.cache.core.acquire_slot()
+    got, pos = [], 0
+    for n in (7, 2, 16, 1, 1, 11, 1, 6):           # portions and single tokens from the same cache
+        def fn(ctx, views, lo=pos, n=n):
+            h = torch.zeros((n, c.hidden), dtype=torch.float32, device=DEV)
+            att.forward(ctx, x[lo:lo + n].to(DEV), h, views[0])
+            got.append(h)
+        hz.run([StepEntry(s, pos, [0] * n, [])], fn)
+        pos += n
+    assert close(torch.cat(got), ref, dtype)
+    if c.window:
+        assert hz.cache.core.pages_held(s) < -(-T // c.ps) or c.window + c.ps >= T, "pages behind the window go back to the pool"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_alone(dtype):
+    H, F = 48, 80
+    layer = LayerSpec("prenorm",
+                      PartSpec("attention", "b.att", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 1, "head_dim": 32, "window": None,
+                                                      "position": {"kind": "rope", "head_dim": 32, "rotary_dim": 32, "theta": 1e4, "layout": "split_half"}}),
+                      PartSpec("swiglu", "b.mlp", {"hidden_size": H, "intermediate_size": F}),
+                      PartSpec("rmsnorm", "b.n1", {"size": H, "eps": 1e-5}), PartSpec("rmsnorm", "b.n2", {"size": H, "eps": 1e-6}))
+    block = build_block(layer, dtype)
+    ws = {}
+    for i, part in enumerate(block.parts()):
+        for n, s in part.tensors().items():
+            ws[n] = ((rnd(s.shape, 20 + len(ws)) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, 20 + len(ws), 0.15)).bfloat16()
+        part.load(ws, DEV)
+    T = 19
+    h0 = rnd((T, H), 3)
+    x = h0.double()
+    xn = plain_rmsnorm(x, ws["b.n1.weight"].double(), 1e-5)
+    x = x + attention_reference(ws, "b.att", xn, 3, 1, 32, layer.mixer.params["position"], 0)
+    xn = plain_rmsnorm(x, ws["b.n2.weight"].double(), 1e-6)
+    ref = x + plain_swiglu(xn, ws["b.mlp.gate_proj.weight"].double(), ws["b.mlp.up_proj.weight"].double(), ws["b.mlp.down_proj.weight"].double())
+    hz = Harness([(block.mixer.cache_need(), None)], dtype)
+    s = hz.cache.core.acquire_slot()
+    out = {}
+
+    def fn(ctx, views):
+        h = h0.to(DEV).clone()
+        block.forward(ctx, h, views[0])
+        out["h"] = h
+    hz.run([StepEntry(s, 0, [0] * T, [])], fn)
+    assert close(out["h"], ref, dtype)
+
+
+# ---- a toy mixer with state of its own, defined here -------------------------------------------
+
+class DecayMixer(Mixer):
+    """s_t = decay * s_{t-1} + x_t per request; y_t = s_t W^T.  Its state is one vector per
+    request, kept in the request's slot; it needs no pages."""
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.hidden, self.decay = spec.params["hidden_size"], spec.params["decay"]
+        self.w = None
+
+    def tensors(self):
+        return {self.name("w"): TensorSpec((self.hidden, self.hidden))}
+
+    def load(self, tensors, device):
+        self.w = tensors[self.name("w")].to(device=device, dtype=torch.float32)
+
+    def cache_need(self):
+        return FixedState((self.hidden,), torch.float32)
+
+    def forward(self, ctx, x, h, cache):
+        at = 0
+        for slot, start, count in ctx.entries:       # the step's host-side view: (slot, start, count)
+            s = cache.state[slot]
+            for t in range(at, at + count):
+                s.mul_(self.decay).add_(x[t].float())
+                h[t] += s @ self.w.T
+            at += count
+
+
+class ToyConfig:
+    """Four runs over three layers: decay mixer, attention, the decay layer again (with a state
+    of its own for that run), and attention that reads the cache the first attention run wrote."""
+
+    def __init__(self, d):
+        self.d = d
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        H, V = self.d["hidden_size"], self.d["vocab_size"]
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": H, "eps": 1e-5})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": H, "intermediate_size": 2 * H})
+        rope = {"kind": "rope", "head_dim": 32, "rotary_dim": 32, "theta": 1e4, "layout": "split_half"}
+        att = lambda p, kvp: PartSpec("attention", p, {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 32,
+                                                       "window": None, "position": rope, "kv_proj": kvp})
+        layers = [LayerSpec("prenorm", PartSpec("test_decay", "l0.mix", {"hidden_size": H, "decay": 0.9}), ffn("l0.mlp"), norm("l0.n1"), norm("l0.n2")),
+                  LayerSpec("prenorm", att("l1.att", True), ffn("l1.mlp"), norm("l1.n1"), norm("l1.n2")),
+                  LayerSpec("prenorm", att("l2.att", False), ffn("l2.mlp"), norm("l2.n1"), norm("l2.n2"))]
+        return ModelSpec(H, V, 256, layers, [RunSpec(0), RunSpec(1), RunSpec(0), RunSpec(2, cache_of=1)],
+                         norm("final"), "embed", None)
+
+
+def toy_reference(ws, tokens, H):
+    x = ws["embed"].double()[torch.tensor(tokens)]
+    T = len(tokens)
+    rope = {"rotary_dim": 32, "theta": 1e4, "layout": "split_half"}
+    inv = plain_inv_freq(32, 1e4, None)
+    pos = torch.arange(T)
+    shared = {}
+
+    def mlp(x, p):
+        xn = plain_rmsnorm(x, ws[f"{p}.n2.weight"].double(), 1e-5)
+        return x + plain_swiglu(xn, ws[f"{p}.mlp.gate_proj.weight"].double(), ws[f"{p}.mlp.up_proj.weight"].double(), ws[f"{p}.mlp.down_proj.weight"].double())
+
+    def decay(x):
+        xn = plain_rmsnorm(x, ws["l0.n1.weight"].double(), 1e-5)
+        s, ys = torch.zeros(H, dtype=torch.float64), []
+        for t in range(T):
+            s = 0.9 * s + xn[t]
+            ys.append(s @ ws["l0.mix.w"].double().T)
+        return mlp(x + torch.stack(ys), "l0")
+
+    x = decay(x)
+    xn = plain_rmsnorm(x, ws["l1.n1.weight"].double(), 1e-5)
+    q = plain_rope((xn @ ws["l1.att.q_proj.weight"].double().T).view(T, 2, 32), pos, inv)
+    shared["k"] = plain_rope((xn @ ws["l1.att.k_proj.weight"].double().T).view(T, 1, 32), pos, inv)
+    shared["v"] = (xn @ ws["l1.att.v_proj.weight"].double().T).view(T, 1, 32)
+    x = mlp(x + plain_attention(q, shared["k"], shared["v"]).reshape(T, 64) @ ws["l1.att.o_proj.weight"].double().T, "l1")
+    x = decay(x)                                     # the same layer, run again, with a fresh state
+    xn = plain_rmsnorm(x, ws["l2.n1.weight"].double(), 1e-5)
+    q = plain_rope((xn @ ws["l2.att.q_proj.weight"].double().T).view(T, 2, 32), pos, inv)
+    x = mlp(x + plain_attention(q, shared["k"], shared["v"]).reshape(T, 64) @ ws["l2.att.o_proj.weight"].double().T, "l2")
+    return plain_rmsnorm(x, ws["final.weight"].double(), 1e-5) @ ws["embed"].double().T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_a_stateful_mixer(dtype):
+    register_mixer("test_decay", DecayMixer)
+    register_architecture("TestToyForCausalLM", ToyConfig)
+    H, V = 40, 90
+    cfg = ToyConfig({"architectures": ["TestToyForCausalLM"], "hidden_size": H, "vocab_size": V})
+    from llm_rs_amd.engine import Model
+    names = Model(cfg.model_spec(), torch.float32, "cpu").tensors()
+    assert "l2.att.k_proj.weight" not in names and "l1.att.k_proj.weight" in names
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.2)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    eng = Engine(cfg, ws, dtype=dtype, page_size=16, num_pages=32, max_requests=4)
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].n_layers == 1, "two attention runs share one cache layer"
+    assert len(eng.cache.state_tensors) == 2, "each run of the decay layer has a state of its own"
+    seqs = {0: torch.randint(0, V, (50,), generator=torch.Generator().manual_seed(1)).tolist(),
+            1: torch.randint(0, V, (23,), generator=torch.Generator().manual_seed(2)).tolist()}
+    refs = {i: toy_reference(ws, t, H) for i, t in seqs.items()}
+    tol = 3e-5 if dtype == "float32" else 2e-2
+    # whole, then in portions side by side with the other request, then the slots are used again
+    for cuts in ([50], [9, 2, 20, 1, 1, 17]):
+        slots = {i: eng.open_request() for i in seqs}
+        pos, rows = {0: 0, 1: 0}, {0: [], 1: []}
+        for n in cuts:
+            entries = []
+            for i in seqs:
+                m = min(n, len(seqs[i]) - pos[i])
+                if m > 0:
+                    entries.append((i, StepEntry(slots[i], pos[i], seqs[i][pos[i]:pos[i] + m], list(range(m)))))
+            out = eng.step([e for _, e in entries]).double().cpu()
+            at = 0
+            for i, e in entries:
+                rows[i].append(out[at:at + len(e.tokens)]); at += len(e.tokens); pos[i] += len(e.tokens)
+        for i in seqs:
+            got = torch.cat(rows[i])
+            ref = refs[i][:got.shape[0]]
+            assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), (cuts, i)
+            eng.close_request(slots[i])
+    assert eng.generate([seqs[1][:5]], max_new_tokens=4)[0] == eng.generate([seqs[1][:5]], max_new_tokens=4)[0]
