@@ -43,6 +43,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
+    ap.add_argument("--only", default="", choices=["", "prefill", "decode"], help="for profiling: time one phase only")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -89,7 +90,7 @@ def main() -> int:
 
     toks = prompt(args.prefill_tokens)
     prefill_once()
-    prefill_s = timed(prefill_once, 3)
+    prefill_s = timed(prefill_once, 3 if args.only != "decode" else 1)
     spec = engine.model.spec
     D, F, V, L = config.hidden_size, config.intermediate_size, vocab, config.num_hidden_layers
     Hq, Hkv = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
@@ -127,6 +128,9 @@ def main() -> int:
             engine.close_request(s)
         return sec
 
+    if args.only == "prefill":
+        print(json.dumps({"prefill_ms": round(prefill_s * 1e3, 3), "tokens": T}))
+        return 0
     step_s = decode_run(args.batch, args.steps, args.warmup)
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
     point_values = {}
