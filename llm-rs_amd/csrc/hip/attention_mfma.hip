@@ -216,10 +216,15 @@ __global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__
         for (int i = 0; i < 16; ++i) pp[2 + o_feature(dt, i, h)] = O[dt][i];
 }
 
-__global__ void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
-                                  const int* __restrict__ positions, const int* __restrict__ q_starts, AttnArgs a,
-                                  int max_chunks) {
-    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim;
+#define MERGE_MAX_CHUNKS 1024
+
+// One wave for each (entry, head): lanes share out the chunks for the common maximum and
+// the sum, then the features.  Chunks are added in ascending order.
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
+                                                        const int* __restrict__ positions,
+                                                        const int* __restrict__ q_starts, AttnArgs a, int max_chunks) {
+    __shared__ float weight[MERGE_MAX_CHUNKS];
+    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim, lane = threadIdx.x;
     if (q_starts[e + 1] - q_starts[e] != 1) return;
     int token = q_starts[e];
     int pos = positions[token];
@@ -227,14 +232,21 @@ __global__ void attn_merge_kernel(const float* __restrict__ partial, bf16* __res
     int n_chunks = pos / ATTN_CHUNK - lo / ATTN_CHUNK + 1;
     const float* pp = partial + (size_t)(e * a.n_heads + head) * max_chunks * (hd + 2);
     float M = -INFINITY;
-    for (int ch = 0; ch < n_chunks; ++ch) M = fmaxf(M, pp[(size_t)ch * (hd + 2)]);
+    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * (hd + 2)]);
+    M = wave_max(M);
     float L = 0.0f;
-    for (int ch = 0; ch < n_chunks; ++ch) L += pp[(size_t)ch * (hd + 2) + 1] * expf(pp[(size_t)ch * (hd + 2)] - M);
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    for (int ch = lane; ch < n_chunks; ch += 64) {
+        float w = expf(pp[(size_t)ch * (hd + 2)] - M);
+        weight[ch] = w;
+        L += pp[(size_t)ch * (hd + 2) + 1] * w;
+    }
+    L = wave_sum(L);
+    __syncthreads();
+    float inv = 1.0f / L;
+    for (int d = lane; d < hd; d += 64) {
         float o = 0.0f;
-        for (int ch = 0; ch < n_chunks; ++ch)   // ascending chunks: a fixed order
-            o += pp[(size_t)ch * (hd + 2) + 2 + d] * expf(pp[(size_t)ch * (hd + 2)] - M);
-        out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / L);
+        for (int ch = 0; ch < n_chunks; ++ch) o = fmaf(pp[(size_t)ch * (hd + 2) + 2 + d], weight[ch], o);
+        out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o * inv);
     }
 }
 
@@ -247,7 +259,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     int max_chunks = max_seq_len > 0 ? (max_seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK : 0;
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.
-    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= 65535;
+    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS;
     int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
     if (!only_single) {
         int tiles = a.n_tokens / tpt + n_entries;

@@ -1,12 +1,12 @@
 // bfloat16 products on the matrix cores, 32-bit accumulation.
 //
 // Two kernels, chosen by M (the number of tokens in the step):
-//   M <= 32  "skinny": decoding.  Every weight is read once, straight from
-//            memory into MFMA operands; a block owns 16 output features and its
-//            waves split K, so a layer's product has enough waves in flight to
+//   M <= 64  "skinny": decoding.  Every weight is read once, straight from
+//            memory into MFMA operands; a block owns 16 to 64 output features and
+//            its waves split K, so a layer's product has enough loads in flight to
 //            keep HBM busy.  v_mfma_f32_16x16x32_bf16, weights as the A operand.
-//   M  > 32  "tiled": prompts.  128x128 (or 64x128) tiles of the output, K in
-//            steps of 64 through double-buffered LDS, v_mfma_f32_32x32x16_bf16.
+//   M  > 64  "tiled": prompts.  128x128 tiles of the output, K in steps of 64
+//            through double-buffered LDS, v_mfma_f32_32x32x16_bf16.
 // Both need K % 8 == 0 and 16-byte aligned rows (16-byte loads); otherwise the
 // caller falls back to the plain kernel.
 //
@@ -30,71 +30,101 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // ---------------------------------------------------------------------------
 // skinny: C^T[n, m] = sum_k W[n, k] X[m, k]
-//   A operand = W rows: lane l holds row n0 + l%16, 8 consecutive k
-//   B operand = X rows: lane l holds token l%16 (+16 per tile), the same 8 k
-//   C: lane l holds token l%16 and features n0 + 4*(l/16) + r, r = 0..3
+//   A operand = W rows: lane l holds row n0 + l%16 (+16 per feature tile), 8 consecutive k
+//   B operand = X rows: lane l holds token l%16 (+16 per token tile), the same 8 k
+//   C: lane l holds token l%16 and features 4*(l/16) + r, r = 0..3
 // A lane's 8 k-values of one MFMA may be any 8, as long as both operands take
-// the same; each lane group takes 16 consecutive k (two MFMAs), so that a wave
-// reads 128 contiguous bytes of each of its 16 weight rows at a time.
+// the same; of a block of 64 k, lane group g takes [8g, 8g+8) for one MFMA and
+// [32+8g, 32+8g+8) for the next, so that each load instruction reads 64
+// contiguous bytes of every row and the two together one 128-byte line.
+// A block owns NT*16 features and MT*16 tokens; its NW waves take the 64-wide
+// k-blocks in turn (wave w: w, w+NW, ...), U of them per round with all loads of
+// a round issued before its first MFMA, and add their sums in wave order.
 // ---------------------------------------------------------------------------
-template <int MT, int NW>
+template <int MT, int NT, int NW, int U>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
                                                               int ldc, int M, int N, int K, int epi) {
-    __shared__ float red[NW][MT][4][64];
+    extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
+    float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int row = lane & 15, g = lane >> 4;
-    int n0 = blockIdx.x * 16;
-    const bf16* wp = W + (size_t)min(n0 + row, N - 1) * K;
+    int n0 = blockIdx.x * (NT * 16);
+    const bf16* wp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wp[nt] = W + (size_t)min(n0 + nt * 16 + row, N - 1) * K;
     const bf16* xp[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) xp[mt] = A + (size_t)min(mt * 16 + row, M - 1) * lda;
-    f32x4 acc[MT];
+    f32x4 acc[MT][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     int full = K / 64;             // blocks of 64 k that need no bounds
     int kb = wave;
-#pragma unroll 4
-    for (; kb < full; kb += NW) {
-        int k = kb * 64 + g * 16;
-        bf16x8 w0 = load8(wp + k), w1 = load8(wp + k + 8);
+    for (; kb + (U - 1) * NW < full; kb += U * NW) {
+        bf16x8 w[U][NT][2], x[U][MT][2];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 x0 = load8(xp[mt] + k), x1 = load8(xp[mt] + k + 8);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[mt], 0, 0, 0);
+        for (int u = 0; u < U; ++u) {
+            int k = (kb + u * NW) * 64 + g * 8;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) { w[u][nt][0] = load8(wp[nt] + k); w[u][nt][1] = load8(wp[nt] + k + 32); }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) { x[u][mt][0] = load8(xp[mt] + k); x[u][mt][1] = load8(xp[mt] + k + 32); }
         }
+        __builtin_amdgcn_sched_barrier(0);   // keep the round's loads together, ahead of its MFMAs
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][nt][0], x[u][mt][0], acc[mt][nt], 0, 0, 0);
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][nt][1], x[u][mt][1], acc[mt][nt], 0, 0, 0);
+                }
     }
-    if (kb == full && (K & 63)) {  // the wave whose turn it is takes the partial block
-        int k = kb * 64 + g * 16;
-        bool v0 = k < K, v1 = k + 8 < K;
-        bf16x8 w0 = v0 ? load8(wp + k) : zero8(), w1 = v1 ? load8(wp + k + 8) : zero8();
+    for (; kb <= full; kb += NW) {   // what is left of this wave's turns, and the partial block if it is its turn
+        if (kb == full && !(K & 63)) break;
+        int k = kb * 64 + g * 8;
+        bool v0 = k < K, v1 = k + 32 < K;
+        bf16x8 w0[NT], w1[NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            w0[nt] = v0 ? load8(wp[nt] + k) : zero8();
+            w1[nt] = v1 ? load8(wp[nt] + k + 32) : zero8();
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 x0 = load8(xp[mt] + (v0 ? k : 0)), x1 = load8(xp[mt] + (v1 ? k + 8 : 0));
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0, x0, acc[mt], 0, 0, 0);
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1, x1, acc[mt], 0, 0, 0);
+            bf16x8 x0 = load8(xp[mt] + (v0 ? k : 0)), x1 = load8(xp[mt] + (v1 ? k + 32 : 0));
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w0[nt], x0, acc[mt][nt], 0, 0, 0);
+                acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x1, acc[mt][nt], 0, 0, 0);
+            }
         }
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) red[wave][mt][r][lane] = acc[mt][r];
-    __syncthreads();
-    if (wave != 0) return;
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
+            for (int r = 0; r < 4; ++r) red[(((wave * MT + mt) * NT + nt) * 4 + r) * 64 + lane] = acc[mt][nt][r];
+    __syncthreads();
+    // the (mt, nt) tiles are shared out over the waves; each is summed over the waves in order
+    for (int tile = wave; tile < MT * NT; tile += NW) {
+        int mt = tile / NT, nt = tile % NT;
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             float s = 0.0f;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) s += red[w][mt][r][lane];  // waves in order: a fixed sum
+            for (int w = 0; w < NW; ++w) s += red[(((w * MT + mt) * NT + nt) * 4 + r) * 64 + lane];
             v[r] = s;
         }
         int m = mt * 16 + row;
-        int n = n0 + 4 * g;
+        int n = n0 + nt * 16 + 4 * g;
         if (m >= M) continue;
         if (epi == LLMRS_EPI_SWIGLU) {
 #pragma unroll
@@ -106,6 +136,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                 if (n + r < N) epilogue_store<bf16>(epi, out, ldc, m, n + r, v[r]);
         }
     }
+}
+
+template <int MT, int NT, int NW, int U>
+static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
+                          int M, int N, int K, int epi) {
+    size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NT, NW, U>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        configured = true;
+    }
+    gemm_skinny_kernel<MT, NT, NW, U><<<ceil_div(N, NT * 16), NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
 }
 
 // ---------------------------------------------------------------------------
@@ -230,20 +273,31 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                          int M, int N, int K, int epi) {
     if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return 0;
     int rc = 0;
-    if (M <= 32) {
-        // Waves per block from the weight's shape alone, so that a row's sum has one
-        // order whatever the batch: 8 waves when K is long enough to share out.
-        bool eight = K >= 2048;
-        dim3 grid(ceil_div(N, 16));
+    if (M <= 64) {
+        // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
+        // waves in turn and their sums are added in wave order, so for a given weight an
+        // output's sum has one order whatever M, MT, NT and U are.
+        // Features per block (NT*16) grow with N and M: a block reads its tokens' rows
+        // again for every 16*NT features, which costs L2 bandwidth once M is large, but
+        // a weight with few rows needs small blocks to have enough of them.
+        // (Measured on MI355X at the 8B shapes; see profiles/.)
+        bool wide = N >= 16384;
+        bool eight = !wide && K >= 2048;
+#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi)
         if (M <= 16) {
-            if (eight) gemm_skinny_kernel<1, 8><<<grid, 512, 0, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
-            else gemm_skinny_kernel<1, 4><<<grid, 256, 0, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+            if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else SKINNY(1, 4, 4, 2); }
+            else if (eight) SKINNY(1, 1, 8, 4);
+            else SKINNY(1, 1, 4, 4);
+        } else if (M <= 32) {
+            if (wide) SKINNY(2, 4, 4, 2);
+            else if (N > 4096) { if (eight) SKINNY(2, 2, 8, 2); else SKINNY(2, 2, 4, 2); }
+            else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {
-            if (eight) gemm_skinny_kernel<2, 8><<<grid, 512, 0, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
-            else gemm_skinny_kernel<2, 4><<<grid, 256, 0, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+            if (wide) SKINNY(4, 4, 4, 2);
+            else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
+            else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
         }
-    } else if (M <= 64) {
-        rc = launch_tiled<64, 128>(stream, A, lda, W, out, ldc, M, N, K, epi);
+#undef SKINNY
     } else {
         rc = launch_tiled<128, 128>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }

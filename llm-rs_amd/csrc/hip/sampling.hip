@@ -9,16 +9,32 @@ __device__ __forceinline__ void argmax_merge(float& v, int& i, float ov, int oi)
     if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
 }
 
+// Stage 1: block (row, part) scans its part of the row; stage 2 (part count 1, or
+// the second launch over the partial results) picks among the parts.
+#define ARGMAX_PARTS 32
+
 __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restrict__ logits, int ld, int V,
-                                                           int* __restrict__ out) {
+                                                           const float* __restrict__ part_val,
+                                                           const int* __restrict__ part_idx,
+                                                           float* __restrict__ out_val, int* __restrict__ out_idx) {
     __shared__ float sv[16];
     __shared__ int si[16];
-    const float* row = logits + (size_t)blockIdx.x * ld;
+    int row = blockIdx.x, parts = gridDim.y, part = blockIdx.y;
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        float v = row[i];
-        if (v > best || idx == 0x7fffffff) { best = v; idx = i; }
+    if (part_val == nullptr) {
+        const float* src = logits + (size_t)row * ld;
+        int per = (V + parts - 1) / parts;
+        int lo = part * per, hi = min(lo + per, V);
+        for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            float v = src[i];
+            if (v > best || idx == 0x7fffffff) { best = v; idx = i; }
+        }
+    } else {   // V is the number of partial results of this row
+        for (int i = threadIdx.x; i < V; i += blockDim.x) {
+            int pi = part_idx[row * V + i];
+            if (pi != 0x7fffffff) argmax_merge(best, idx, part_val[row * V + i], pi);
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -31,14 +47,25 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const float* __restri
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < (int)(blockDim.x >> 6); ++w) argmax_merge(best, idx, sv[w], si[w]);
-        out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+        if (out_val) { out_val[row * parts + part] = best; out_idx[row * parts + part] = idx; }
+        else out_idx[row] = idx == 0x7fffffff ? 0 : idx;
     }
 }
 
-extern "C" int llmrs_argmax_rows(hipStream_t stream, const float* logits, int ld, int n_rows, int V, int* out) {
+// scratch: room for n_rows * 32 (float, int) pairs, or null: then one block scans a whole row.
+extern "C" int llmrs_argmax_rows(hipStream_t stream, const float* logits, int ld, int n_rows, int V, int* out,
+                                 void* scratch, size_t scratch_bytes) {
     LLMRS_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax_rows: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
     if (n_rows == 0) return 0;
-    argmax_rows_kernel<<<n_rows, 1024, 0, stream>>>(logits, ld, V, out);
+    size_t need = (size_t)n_rows * ARGMAX_PARTS * 8;
+    if (V >= 8192 && scratch != nullptr && scratch_bytes >= need) {
+        float* pv = (float*)scratch;
+        int* pi = (int*)(pv + (size_t)n_rows * ARGMAX_PARTS);
+        argmax_rows_kernel<<<dim3(n_rows, ARGMAX_PARTS), 1024, 0, stream>>>(logits, ld, V, nullptr, nullptr, pv, pi);
+        argmax_rows_kernel<<<dim3(n_rows, 1), 64, 0, stream>>>(nullptr, 0, ARGMAX_PARTS, pv, pi, nullptr, out);
+    } else {
+        argmax_rows_kernel<<<dim3(n_rows, 1), 1024, 0, stream>>>(logits, ld, V, nullptr, nullptr, nullptr, out);
+    }
     LLMRS_LAUNCH_CHECK("argmax_rows");
     return 0;
 }

@@ -65,6 +65,10 @@ class Model:
         total += self.head.numel() * self.head.element_size() + self.final_norm.weight.numel() * 4
         return total
 
+    def graph_safe(self) -> bool:
+        """Whether a step of this model may be recorded into a HIP graph (every part says so)."""
+        return all(part.graph_safe for block in self.blocks for part in block.parts()) and self.final_norm.graph_safe
+
     # -- cache ---------------------------------------------------------------
     def cache_needs(self) -> List[Tuple[object, Optional[int]]]:
         return [(self.blocks[run.layer].mixer.cache_need(), run.cache_of) for run in self.spec.schedule]

@@ -8,11 +8,21 @@ Host work per step: ask the core for pages, let it flatten the batch into one
 block of words in pinned memory, copy that block to the device once, launch.
 Activations live in a workspace that grows to the largest step seen and is then
 reused, so steady-state steps allocate nothing.
+
+Steps in which every entry brings one token (decoding) are launch-bound: a few
+hundred small kernels.  Such a step is recorded once into a HIP graph, keyed by
+its batch size and block-table width, and replayed afterwards: the flattened
+batch has the same layout for the same key, every kernel reads positions, tables
+and counts from that block on the device, and nothing in the graph depends on
+host values.  Grids that depend on the context length are recorded for the
+width's capacity and leave early.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
+
+import os
 
 import numpy as np
 import torch
@@ -63,6 +73,13 @@ class StepRunner:
         self._turn = 0
         self._dev_words = torch.zeros(words_capacity, dtype=torch.int32, device=self.device)
         self.ctx = StepContext(self)
+        # HIP graphs of decode steps: key -> (graph, logits); a key is recorded the second time it is seen
+        self.use_graphs = (self._pinned and os.environ.get("LLMRS_GRAPHS", "1") != "0" and not cache.state_tensors
+                           and bool(getattr(model, "graph_safe", lambda: False)()))
+        self.max_graph_batch = 512
+        self._graphs: Dict[tuple, tuple] = {}
+        self._seen: Dict[tuple, int] = {}
+        self.graph_replays = 0
 
     def _new_host(self, n: int) -> torch.Tensor:
         return torch.zeros(n, dtype=torch.int32, pin_memory=self._pinned)
@@ -78,6 +95,8 @@ class StepRunner:
             cap = max(nbytes, 256) if buf is None else max(nbytes, 2 * buf.numel())
             buf = torch.empty(cap, dtype=torch.uint8, device=self.device)
             self._buffers[name] = buf
+            self._graphs.clear()        # recorded graphs hold the old addresses
+            self._seen.clear()
         return buf[:nbytes].view(dtype).view(*shape)
 
     # -- staging -----------------------------------------------------------------
@@ -95,6 +114,8 @@ class StepRunner:
         i = self._turn
         if self._dev_words.numel() < n_words:
             self._dev_words = torch.zeros(max(n_words, 2 * self._dev_words.numel()), dtype=torch.int32, device=self.device)
+            self._graphs.clear()
+            self._seen.clear()
         dev = self._dev_words[:n_words]
         dev.copy_(self._host[i][:n_words], non_blocking=True)
         if self._pinned:
@@ -103,13 +124,27 @@ class StepRunner:
             self._events[i] = ev
         return dev
 
-    def _estimate_words(self, T: int, R: int, n_want: int, longest: int) -> int:
+    def _estimate_words(self, T: int, R: int, n_want: int, longest: int, widths=None) -> int:
         """Upper bound of the flattened batch's size; `longest` is the largest start + count.
         A block table never has more entries than the positions ensured for it need."""
         words = 4 + 3 * T + 3 * R + 1 + 5 * n_want
-        for grp in self.cache.groups:
-            words += T + R * max(1, -(-longest // grp.page_size))
+        for g, grp in enumerate(self.cache.groups):
+            words += T + R * (widths[g] if widths else max(1, -(-longest // grp.page_size)))
         return words + 16
+
+    def _graph_widths(self, counts, longest: int):
+        """Block-table widths to record a decode step with, or None when the step is not one
+        that is recorded: every entry brings one token, and the batch is not huge."""
+        if not self.use_graphs or len(counts) > self.max_graph_batch or any(c != 1 for c in counts):
+            return None
+        widths = []
+        for grp in self.cache.groups:
+            need = max(1, -(-longest // grp.page_size))
+            cap = 64
+            while cap < need:
+                cap *= 2
+            widths.append(cap)
+        return widths
 
     def _bind(self, dev: torch.Tensor, off, T: int, R: int, n_want: int, entries) -> StepContext:
         c = self.ctx
@@ -156,11 +191,13 @@ class StepRunner:
                 raise OutOfPages(f"no cache pages left for slot {e.slot} at positions {e.start}..{e.start + n - 1}")
             slots.append(e.slot); starts.append(e.start); counts.append(n); tokens.extend(ids.tolist())
         T, R = len(tokens), len(entries)
-        words = self._staging(self._estimate_words(T, R, len(want_rows), max(a + b for a, b in zip(starts, counts))))
-        off = core.build_batch(slots, starts, counts, tokens, want_rows, words)
+        longest = max(a + b for a, b in zip(starts, counts))
+        widths = self._graph_widths(counts, longest)
+        words = self._staging(self._estimate_words(T, R, len(want_rows), longest, widths))
+        off = core.build_batch(slots, starts, counts, tokens, want_rows, words, fixed_widths=widths)
         dev = self._upload(off.words)
         ctx = self._bind(dev, off, T, R, len(want_rows), list(zip(slots, starts, counts)))
-        return self._execute(ctx)
+        return self._execute(ctx, widths)
 
     def run_planned(self):
         """Runs the step the scheduler planned; returns (logits or None, rows that sample)."""
@@ -170,13 +207,37 @@ class StepRunner:
             return None, 0, plan
         T = sum(p[2] for p in plan)
         R = len(plan)
-        words = self._staging(self._estimate_words(T, R, R, max(p[1] + p[2] for p in plan)))
-        off, n_tokens, n_want = core.build_planned(words)
+        longest = max(p[1] + p[2] for p in plan)
+        widths = self._graph_widths([p[2] for p in plan], longest)
+        words = self._staging(self._estimate_words(T, R, R, longest, widths))
+        off, n_tokens, n_want = core.build_planned(words, fixed_widths=widths)
         dev = self._upload(off.words)
         ctx = self._bind(dev, off, n_tokens, R, n_want, [(p[0], p[1], p[2]) for p in plan])
-        return self._execute(ctx), n_want, plan
+        return self._execute(ctx, widths), n_want, plan
 
-    def _execute(self, ctx: StepContext) -> Optional[torch.Tensor]:
+    def _execute(self, ctx: StepContext, graph_widths=None) -> Optional[torch.Tensor]:
         fresh = [slot for slot, start, _ in ctx.entries if start == 0]
         self.cache.reset_state(fresh)
-        return self.model.forward(ctx, self.cache.views)
+        if graph_widths is None:
+            return self.model.forward(ctx, self.cache.views)
+        # A decode step.  Everything the kernels take from the host must be the same for
+        # every step of this key: sizes, addresses, and the bound on the context length.
+        ctx.max_seq_len = min(w * g.page_size for w, g in zip(graph_widths, self.cache.groups)) if graph_widths else ctx.max_seq_len
+        key = (ctx.n_tokens, ctx.n_want, tuple(graph_widths), self._dev_words.data_ptr())
+        hit = self._graphs.get(key)
+        if hit is not None:
+            hit[0].replay()
+            self.graph_replays += 1
+            return hit[1]
+        self._seen[key] = self._seen.get(key, 0) + 1
+        if self._seen[key] < 2:
+            return self.model.forward(ctx, self.cache.views)     # first time: run it, and let the workspace grow
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(ctx, self.cache.views)
+        if key not in self._seen:       # the workspace grew while recording: those addresses are gone
+            return self.model.forward(ctx, self.cache.views)
+        self._graphs[key] = (graph, logits)
+        graph.replay()                  # recording does not run the kernels
+        self.graph_replays += 1
+        return logits

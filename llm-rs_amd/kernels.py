@@ -53,7 +53,7 @@ class HipKernels:
             "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I],
-            "llmrs_argmax_rows": [V, V, I, I, I, V],
+            "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
         }
         for name, args in sigs.items():
@@ -137,10 +137,12 @@ class HipKernels:
             _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
             int(self.allow_mfma)))
 
-    def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor) -> None:
+    def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
+        """`scratch`: 256 bytes per row let several blocks share a long row."""
         assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
         self._check(self.lib.llmrs_argmax_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
-                                               logits.shape[1], _p(out)))
+                                               logits.shape[1], _p(out), _p(scratch),
+                                               0 if scratch is None else scratch.numel() * scratch.element_size()))
 
     # words[i] = uniform (float bits), temperature (float bits), top_k, top_p (float bits) of row i
     def sample_rows(self, logits: torch.Tensor, words: torch.Tensor, out: torch.Tensor) -> None:

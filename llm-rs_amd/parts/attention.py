@@ -22,6 +22,8 @@ from .base import Mixer, TensorSpec, build_position, register_mixer
 
 
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
         p = spec.params
@@ -34,6 +36,8 @@ class Attention(Mixer):
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         self.position = build_position(p.get("position"), dtype)
+        if self.position is not None and self.position.rotary() is None:
+            self.graph_safe = False      # its apply() is free to do anything
         if self.heads % self.kv_heads:
             raise ValueError(f"{self.heads} heads are no multiple of {self.kv_heads} kv heads")
         self.q_size = self.heads * self.head_dim

@@ -28,6 +28,12 @@ class TensorSpec(NamedTuple):
 
 
 class Part:
+    # True when `forward` only launches kernels whose arguments do not change between steps of
+    # the same shape (everything step-specific is read from device memory): such a part may be
+    # recorded into a HIP graph.  A part that looks at host values of the step, allocates, or
+    # copies between host and device must leave this False; the model is then never recorded.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         self.spec = spec
         self.prefix = spec.prefix

@@ -13,6 +13,8 @@ from .base import FeedForward, TensorSpec, register_feed_forward
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
         self.hidden = int(spec.params["hidden_size"])

@@ -10,6 +10,8 @@ from .base import Norm, TensorSpec, register_norm
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, dtype):
         super().__init__(spec, dtype)
         self.size = int(spec.params["size"])

@@ -18,15 +18,17 @@ class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
         self._out = torch.zeros(1024, dtype=torch.int32, device=self.device)
+        self._scratch = torch.zeros(1024 * 64, dtype=torch.int32, device=self.device)   # 256 bytes per row
 
     def sample(self, logits: torch.Tensor, sampling_words: torch.Tensor, all_greedy: bool) -> torch.Tensor:
         """int32 [rows] on the device."""
         n = logits.shape[0]
         if self._out.numel() < n:
             self._out = torch.zeros(2 * n, dtype=torch.int32, device=self.device)
+            self._scratch = torch.zeros(2 * n * 64, dtype=torch.int32, device=self.device)
         out = self._out[:n]
         if all_greedy:
-            kernels().argmax_rows(logits, out)
+            kernels().argmax_rows(logits, out, self._scratch)
         else:
             kernels().sample_rows(logits, sampling_words, out)
         return out

@@ -89,7 +89,7 @@ class EmulatedKernels:
                 p = torch.softmax(s, dim=0)
                 out[t, h * head_dim:(h + 1) * head_dim] = (p @ vals[:, g, :]).to(out.dtype)
 
-    def argmax_rows(self, logits, out):
+    def argmax_rows(self, logits, out, scratch=None):
         for i in range(logits.shape[0]):
             best = logits[i].max()
             out[i] = int((logits[i] == best).nonzero()[0])

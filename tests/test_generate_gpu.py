@@ -155,3 +155,36 @@ def test_small_pool_preempts_and_recomputes(folders):
     assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
     with pytest.raises(Exception, match="pages"):
         tight.generate([random_tokens(cfg["vocab_size"], 200, seed=1)], max_new_tokens=100)
+
+
+@pytest.mark.parametrize("which,dtype", [("B", "bfloat16"), ("A", "float32")])
+def test_recorded_decode_steps_equal_eager_ones(folders, which, dtype):
+    """Decode steps are recorded into a HIP graph and replayed.  Every replay is compared
+    with the same step run eagerly by a second engine, with eager prompt steps, new
+    requests and synchronisations between the replays."""
+    cfg, _ = read_model_folder(folders[which])
+    recorded, eager = engine(folders[which], which, dtype), engine(folders[which], which, dtype)
+    eager.runner.use_graphs = False
+    assert recorded.runner.use_graphs
+    seqs = [random_tokens(cfg["vocab_size"], 90, seed=200 + i) for i in range(3)]
+
+    def both(make_entries):
+        a = recorded.step(make_entries(slots_r)).clone()
+        b = eager.step(make_entries(slots_e)).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(a, b)
+
+    slots_r = [recorded.open_request() for _ in seqs]
+    slots_e = [eager.open_request() for _ in seqs]
+    both(lambda sl: [StepEntry(sl[i], 0, seqs[i][:20 + i], [19 + i]) for i in range(3)])
+    pos = [20, 21, 22]
+    for step in range(40):
+        both(lambda sl: [StepEntry(sl[i], pos[i], [seqs[i][pos[i]]], [0]) for i in range(3)])
+        pos = [p + 1 for p in pos]
+        if step == 15:       # a prompt portion for one request between the replays: an eager step in both engines
+            both(lambda sl: [StepEntry(sl[0], pos[0], seqs[0][pos[0]:pos[0] + 9], [8])])
+            pos[0] += 9
+        if step == 25:       # another batch size: another graph
+            both(lambda sl: [StepEntry(sl[i], pos[i], [seqs[i][pos[i]]], [0]) for i in range(2)])
+            pos[0] += 1; pos[1] += 1
+    assert recorded.runner.graph_replays >= 30 and eager.runner.graph_replays == 0

@@ -283,6 +283,19 @@ def test_argmax_rows():
     assert out.tolist() == want
 
 
+def test_argmax_rows_long_rows_in_parts():
+    V = 128256
+    logits = rnd((5, V), torch.float32, 12)
+    logits[1, [4007, 4008, 100000]] = 50.0      # a tie across the parts of the row
+    logits[2, V - 1] = 60.0
+    logits[3] = 1.5
+    scratch = torch.zeros(5 * 64, dtype=torch.int32, device=DEV)
+    for s in (scratch, None):
+        out = torch.zeros(5, dtype=torch.int32, device=DEV)
+        kernels().argmax_rows(logits, out, s)
+        assert out.tolist() == [int(logits[0].argmax()), 4007, V - 1, 0, int(logits[4].argmax())]
+
+
 def _words(rows):
     """[(uniform, temperature, top_k, top_p)] -> the int32 words the sampler reads."""
     w = torch.zeros((len(rows), 4), dtype=torch.int32)
