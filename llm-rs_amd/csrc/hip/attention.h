@@ -15,4 +15,4 @@ struct AttnArgs {
 int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, const bf16* k_cache, const bf16* v_cache,
                               const int* block_table, const int* token_entry, const int* positions,
                               const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
-                              size_t scratch_bytes, int max_seq_len, const AttnArgs& a);
+                              size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a);

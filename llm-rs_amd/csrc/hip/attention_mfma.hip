@@ -253,13 +253,13 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
                   const int* positions, const int* q_starts, int n_entries, float* scratch, size_t scratch_bytes,
-                  int max_seq_len, const AttnArgs& a) {
+                  int max_seq_len, int n_single, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
     int tpt = 32 / G;
     int max_chunks = max_seq_len > 0 ? (max_seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK : 0;
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.
-    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS;
+    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
     int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
     if (!only_single) {
         int tiles = a.n_tokens / tpt + n_entries;
@@ -277,7 +277,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
 int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, const bf16* k_cache, const bf16* v_cache,
                               const int* block_table, const int* token_entry, const int* positions,
                               const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
-                              size_t scratch_bytes, int max_seq_len, const AttnArgs& a) {
+                              size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a) {
     (void)token_entry; (void)seq_lens;
     int G = a.n_heads / a.n_kv_heads;
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
@@ -285,7 +285,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;
     int rc;
     switch (a.head_dim) {
-#define CASE(HD) case HD: rc = launch<HD>(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, n_entries, scratch, scratch_bytes, max_seq_len, a); break;
+#define CASE(HD) case HD: rc = launch<HD>(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, n_entries, scratch, scratch_bytes, max_seq_len, n_single, a); break;
         CASE(32) CASE(64) CASE(96) CASE(128) CASE(192) CASE(256)
 #undef CASE
         default: return 0;

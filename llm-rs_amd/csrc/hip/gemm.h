@@ -20,5 +20,6 @@ __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int 
 
 // The 16-byte-load kernels on MFMA (gemm_mfma.hip).  Return 1 when they took the
 // product, 0 when its shape or alignment is not theirs, -1 on error.
+// workspace: device memory for the partial sums of products that split K over blocks (may be null).
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                         int M, int N, int K, int epi);
+                         int M, int N, int K, int epi, void* workspace, size_t workspace_bytes);

@@ -16,9 +16,19 @@
 // :1090-1143); unlike gemm_bf16 (:1107) the accumulator is 32-bit.
 #include "gemm.h"
 
+#include <type_traits>
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *(const bf16x8*)p; }
 __device__ __forceinline__ bf16x8 zero8() {
@@ -40,11 +50,18 @@ __device__ __forceinline__ bf16x8 zero8() {
 // A block owns NT*16 features and MT*16 tokens; its NW waves take the 64-wide
 // k-blocks in turn (wave w: w, w+NW, ...), U of them per round with all loads of
 // a round issued before its first MFMA, and add their sums in wave order.
+// With gridDim.y > 1 the k-blocks are shared out over that many blocks as well
+// (contiguous ranges): each writes its 32-bit partial sums to `partial`
+// [gridDim.y][M][N] and gemm_splitk_finish_kernel adds them in order and applies
+// the epilogue.  That is for weights with few rows and many tokens (33..64),
+// where blocks of 64 features are needed to keep the tokens' rows from being
+// read too often, and would otherwise be too few to fill the device.
 // ---------------------------------------------------------------------------
 template <int MT, int NT, int NW, int U>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
-                                                              int ldc, int M, int N, int K, int epi) {
+                                                              int ldc, int M, int N, int K, int epi,
+                                                              float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
     float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -63,8 +80,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     int full = K / 64;             // blocks of 64 k that need no bounds
-    int kb = wave;
-    for (; kb + (U - 1) * NW < full; kb += U * NW) {
+    int nkb = (K + 63) / 64;
+    int per = (nkb + gridDim.y - 1) / gridDim.y;
+    int kb_hi = min(nkb, (int)(blockIdx.y + 1) * per);     // this block's k-blocks: [blockIdx.y * per, kb_hi)
+    int full_hi = min(full, kb_hi);
+    int kb = blockIdx.y * per + wave;
+    for (; kb + (U - 1) * NW < full_hi; kb += U * NW) {
         bf16x8 w[U][NT][2], x[U][MT][2];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -85,8 +106,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][nt][1], x[u][mt][1], acc[mt][nt], 0, 0, 0);
                 }
     }
-    for (; kb <= full; kb += NW) {   // what is left of this wave's turns, and the partial block if it is its turn
-        if (kb == full && !(K & 63)) break;
+    for (; kb < kb_hi; kb += NW) {   // what is left of this wave's turns, and the partial block if it is its turn
         int k = kb * 64 + g * 8;
         bool v0 = k < K, v1 = k + 32 < K;
         bf16x8 w0[NT], w1[NT];
@@ -126,7 +146,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         int m = mt * 16 + row;
         int n = n0 + nt * 16 + 4 * g;
         if (m >= M) continue;
-        if (epi == LLMRS_EPI_SWIGLU) {
+        if (partial != nullptr) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) partial[((size_t)blockIdx.y * M + m) * N + n + r] = v[r];
+        } else if (epi == LLMRS_EPI_SWIGLU) {
 #pragma unroll
             for (int r = 0; r < 4; r += 2)
                 if (n + r + 1 < N) ((bf16*)out)[(size_t)m * ldc + (n + r) / 2] = (bf16)(silu_f32(v[r]) * v[r + 1]);
@@ -138,9 +162,32 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     }
 }
 
+// Adds the partial sums of a split product in order and applies the epilogue.
+// One thread for two adjacent features (a gate/up pair when the epilogue is SwiGLU).
+__global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int splits, void* __restrict__ out,
+                                          int ldc, int M, int N, int epi) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t pairs = (size_t)M * ((N + 1) / 2);
+    if (idx >= pairs) return;
+    int m = (int)(idx / ((N + 1) / 2)), n = 2 * (int)(idx % ((N + 1) / 2));
+    float v0 = 0.0f, v1 = 0.0f;
+    bool has1 = n + 1 < N;
+    for (int s = 0; s < splits; ++s) {
+        const float* p = partial + ((size_t)s * M + m) * N + n;
+        v0 += p[0];
+        if (has1) v1 += p[1];
+    }
+    if (epi == LLMRS_EPI_SWIGLU) {
+        if (has1) ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v0) * v1);
+    } else {
+        epilogue_store<bf16>(epi, out, ldc, m, n, v0);
+        if (has1) epilogue_store<bf16>(epi, out, ldc, m, n + 1, v1);
+    }
+}
+
 template <int MT, int NT, int NW, int U>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                          int M, int N, int K, int epi) {
+                          int M, int N, int K, int epi, int splits = 1, float* partial = nullptr) {
     size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
     static bool configured = false;
     if (!configured) {
@@ -148,7 +195,13 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         configured = true;
     }
-    gemm_skinny_kernel<MT, NT, NW, U><<<ceil_div(N, NT * 16), NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    dim3 grid(ceil_div(N, NT * 16), splits);
+    gemm_skinny_kernel<MT, NT, NW, U><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
+                                                                          splits > 1 ? partial : nullptr);
+    if (splits > 1) {
+        size_t pairs = (size_t)M * ((N + 1) / 2);
+        gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -157,44 +210,50 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
 //   C: lane l holds feature l%32 and tokens 8*(r/4) + 4*(l/32) + r%4, r = 0..15,
 //   so a store instruction writes 32 consecutive features of a token.
 // ---------------------------------------------------------------------------
-#define BK 64
-#define LDT (BK + 8)   // padded LDS row: 144 bytes, so 16 lanes' 16-byte reads hit distinct banks
-
-template <int BM, int BN>
+// BM x BN output tile per block of four waves (2 x 2); K in steps of BKT through
+// two LDS buffers.  The global loads of the next P tiles are in flight, in
+// registers, while this one is multiplied (one tile's product is far shorter than
+// a trip to memory); the oldest of them is written to the other LDS buffer
+// before the step's one barrier.
+// LDS rows are padded by 16 bytes so that 16 lanes' 16-byte reads hit distinct banks.
+template <int BM, int BN, int BKT, int P>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ A, int lda,
                                                          const bf16* __restrict__ W, void* __restrict__ out,
                                                          int ldc, int M, int N, int K, int epi) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     bf16* smem = (bf16*)smem_raw;
+    constexpr int LDT = BKT + 8;
     constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
-    constexpr int A_IT = BM / 32, W_IT = BN / 32, BUF = (BM + BN) * LDT;
+    constexpr int TPR = BKT / 8;              // threads that stage one row (16 bytes each)
+    constexpr int RPP = 256 / TPR;            // rows staged per pass
+    constexpr int A_IT = BM / RPP, W_IT = BN / RPP, BUF = (BM + BN) * LDT;
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int wm = wave >> 1, wn = wave & 1;
     int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-    int srow = tid >> 3, schunk = (tid & 7) * 8;   // staging: 8 threads per 128-byte row
-    bf16x8 ra[A_IT], rw[W_IT];
+    int srow = tid / TPR, schunk = (tid % TPR) * 8;
+    bf16x8 ra[P][A_IT], rw[P][W_IT];     // ring of tiles in flight: slot t % P holds tile t
 
-    auto load_tile = [&](int kt) {
-        int k = kt * BK + schunk;
+    auto load_tile = [&](int kt, int slot) {
+        int k = kt * BKT + schunk;
         bool in = k < K;
 #pragma unroll
         for (int i = 0; i < A_IT; ++i) {
-            int gm = min(m0 + srow + 32 * i, M - 1);
-            ra[i] = in ? load8(A + (size_t)gm * lda + k) : zero8();
+            int gm = min(m0 + srow + RPP * i, M - 1);
+            ra[slot][i] = in ? load8(A + (size_t)gm * lda + k) : zero8();
         }
 #pragma unroll
         for (int i = 0; i < W_IT; ++i) {
-            int gn = min(n0 + srow + 32 * i, N - 1);
-            rw[i] = in ? load8(W + (size_t)gn * K + k) : zero8();
+            int gn = min(n0 + srow + RPP * i, N - 1);
+            rw[slot][i] = in ? load8(W + (size_t)gn * K + k) : zero8();
         }
     };
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int buf, int slot) {
         bf16* as = smem + buf * BUF;
         bf16* ws = as + BM * LDT;
 #pragma unroll
-        for (int i = 0; i < A_IT; ++i) *(bf16x8*)(as + (srow + 32 * i) * LDT + schunk) = ra[i];
+        for (int i = 0; i < A_IT; ++i) *(bf16x8*)(as + (srow + RPP * i) * LDT + schunk) = ra[slot][i];
 #pragma unroll
-        for (int i = 0; i < W_IT; ++i) *(bf16x8*)(ws + (srow + 32 * i) * LDT + schunk) = rw[i];
+        for (int i = 0; i < W_IT; ++i) *(bf16x8*)(ws + (srow + RPP * i) * LDT + schunk) = rw[slot][i];
     };
 
     f32x16 acc[FM][FN];
@@ -205,72 +264,81 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    int nk = (K + BK - 1) / BK;
-    load_tile(0);
-    store_tile(0);
+    int nk = (K + BKT - 1) / BKT;
+    load_tile(0, 0);
+    store_tile(0, 0);
+#pragma unroll
+    for (int p = 1; p <= P - 1; ++p)
+        if (p < nk) load_tile(p, p % P);
     __syncthreads();
     int frow = lane & 31, fk = (lane >> 5) * 8;
-    for (int kt = 0; kt < nk; ++kt) {
-        int cur = kt & 1;
-        if (kt + 1 < nk) load_tile(kt + 1);
-        const bf16* as = smem + cur * BUF + (wm * TM + frow) * LDT + fk;
-        const bf16* ws = smem + cur * BUF + BM * LDT + (wn * TN + frow) * LDT + fk;
+    for (int kt0 = 0; kt0 < nk; kt0 += P) {
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 a[FM], b[FN];
+        for (int p = 0; p < P; ++p) {            // unrolled so that ring slots are compile-time
+            int kt = kt0 + p;
+            if (kt >= nk) break;
+            int cur = kt & 1;
+            // tile kt's slot (p) is free: tile kt went to LDS in the step before
+            if (kt + P < nk) load_tile(kt + P, p);
+            const bf16* as = smem + cur * BUF + (wm * TM + frow) * LDT + fk;
+            const bf16* ws = smem + cur * BUF + BM * LDT + (wn * TN + frow) * LDT + fk;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) a[i] = *(const bf16x8*)(as + i * 32 * LDT + ks * 16);
+            for (int ks = 0; ks < BKT / 16; ++ks) {
+                bf16x8 a[FM], b[FN];
 #pragma unroll
-            for (int j = 0; j < FN; ++j) b[j] = *(const bf16x8*)(ws + j * 32 * LDT + ks * 16);
+                for (int i = 0; i < FM; ++i) a[i] = *(const bf16x8*)(as + i * 32 * LDT + ks * 16);
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+                for (int j = 0; j < FN; ++j) b[j] = *(const bf16x8*)(ws + j * 32 * LDT + ks * 16);
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+            }
+            if (kt + 1 < nk) store_tile(cur ^ 1, (p + 1) % P);
+            __syncthreads();
         }
-        if (kt + 1 < nk) store_tile(cur ^ 1);
-        __syncthreads();
     }
 
+    // The accumulators must be indexed by constants or they end up in scratch memory:
+    // the tiles are walked by a compile-time loop.
+    static_for<0, FM * FN>([&](auto idx) {
+        constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
+        int n = n0 + wn * TN + j * 32 + (lane & 31);
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            int n = n0 + wn * TN + j * 32 + (lane & 31);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                float v = acc[i][j][r];
-                if (epi == LLMRS_EPI_SWIGLU) {
-                    float other = __shfl_xor(v, 1, 64);   // even lane: gate here, up next door
-                    if (!(lane & 1) && m < M && n + 1 < N)
-                        ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v) * other);
-                } else if (m < M && n < N) {
-                    epilogue_store<bf16>(epi, out, ldc, m, n, v);
-                }
+        for (int r = 0; r < 16; ++r) {
+            int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            float v = acc[i][j][r];
+            if (epi == LLMRS_EPI_SWIGLU) {
+                float other = __shfl_xor(v, 1, 64);   // even lane: gate here, up next door
+                if (!(lane & 1) && m < M && n + 1 < N)
+                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v) * other);
+            } else if (m < M && n < N) {
+                epilogue_store<bf16>(epi, out, ldc, m, n, v);
             }
         }
+    });
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int BKT, int P>
 static int launch_tiled(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                         int M, int N, int K, int epi) {
     static bool configured = false;
-    size_t bytes = 2 * (BM + BN) * LDT * sizeof(bf16);
+    size_t bytes = 2 * (BM + BN) * (BKT + 8) * sizeof(bf16);
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BKT, P>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
         configured = true;
     }
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
-    gemm_tiled_kernel<BM, BN><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    gemm_tiled_kernel<BM, BN, BKT, P><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
     return 0;
 }
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                         int M, int N, int K, int epi) {
+                         int M, int N, int K, int epi, void* workspace, size_t workspace_bytes) {
     if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return 0;
     int rc = 0;
     if (M <= 64) {
@@ -293,13 +361,23 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             else if (N > 4096) { if (eight) SKINNY(2, 2, 8, 2); else SKINNY(2, 2, 4, 2); }
             else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {
-            if (wide) SKINNY(4, 4, 4, 2);
+            // 64 x 64 outputs per block; when that leaves no more than 64 blocks, K is split
+            // over blocks too, if the caller gave room for the partial sums (measured: it
+            // pays for N = 4096, K = 14336, and no longer for N = 6144).
+            int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64);
+            int splits = 1;
+            while (blocks <= 64 && blocks * splits < 512 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
+            if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+                launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
+            } else if (wide) SKINNY(4, 4, 4, 2);
             else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
             else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
         }
 #undef SKINNY
     } else {
-        rc = launch_tiled<128, 128>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        // 128 x 128 x 64 with one tile of loads in flight measured best of the tile shapes
+        // tried here (larger tiles need a path without bounds checks to pay off).
+        rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
     if (rc != 0) return -1;
     hipError_t e = hipGetLastError();

@@ -64,9 +64,10 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 }
 
 // A: [M, K] with row stride lda; W: [N, K] dense; out: row stride ldc (elements of
-// its own type; for SWIGLU the output has N/2 columns).
+// its own type; for SWIGLU the output has N/2 columns).  workspace: optional device
+// memory (16 * 64 * N * 4 bytes is always enough) for products that split K over blocks.
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
-                          int M, int N, int K, int epi, int allow_mfma) {
+                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma) {
     LLMRS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     LLMRS_REQUIRE(lda >= K, "gemm: row stride %d of A is shorter than K=%d", lda, K);
     LLMRS_REQUIRE(epi >= 0 && epi <= 3, "gemm: unknown epilogue %d", epi);
@@ -78,7 +79,8 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
     }
     if (M == 0) return 0;
     if (dtype == LLMRS_BF16 && allow_mfma) {
-        int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
+        int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi, workspace,
+                                        workspace_bytes);
         if (took != 0) return took < 0 ? -1 : 0;
     }
     dim3 grid(ceil_div(N, TILE), ceil_div(M, TILE));

@@ -91,5 +91,5 @@ class Model:
         x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
         self.final_norm.forward(ctx, h, x, ctx.want_rows)
         logits = ctx.workspace("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
-        k.gemm(x, self.head, logits, EPI_STORE_F32)
+        k.gemm(x, self.head, logits, EPI_STORE_F32, ctx.gemm_workspace(x, self.head))
         return logits

@@ -57,10 +57,17 @@ class StepContext:
         self.block_tables: List[torch.Tensor] = []
         self.entries: List[Tuple[int, int, int]] = []   # host copy: (slot, start, count)
         self.max_seq_len = 0                            # largest start + count among the entries
+        self.n_single = 0                               # entries that bring one token
         self.device = runner.device
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)
+
+    def gemm_workspace(self, a: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
+        """Room for the partial sums of a @ w.T, when the kernel would split K over blocks."""
+        from ..kernels import kernels
+        n = kernels().gemm_workspace_floats(a.shape[0], w.shape[0], w.shape[1])
+        return self.workspace("gemm.partial", (n,), torch.float32) if n else None
 
 
 class StepRunner:
@@ -151,6 +158,7 @@ class StepRunner:
         c.n_tokens, c.n_entries, c.n_want = T, R, n_want
         c.entries = entries
         c.max_seq_len = max(start + count for _, start, count in entries)
+        c.n_single = sum(1 for _, _, count in entries if count == 1)
         c.tokens = dev[off.tokens:off.tokens + T]
         c.positions = dev[off.positions:off.positions + T]
         c.token_entry = dev[off.token_entry:off.token_entry + T]

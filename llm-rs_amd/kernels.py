@@ -50,9 +50,9 @@ class HipKernels:
         sigs = {
             "llmrs_embed_rows": [V, I, V, V, V, I, I, I],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
-            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, I],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
-            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I],
+            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
         }
@@ -70,6 +70,16 @@ class HipKernels:
         self.allow_mfma = True  # tests switch the matrix-core kernels off to compare paths
         lib.llmrs_attention_chunk.restype = I
         self.attention_chunk = lib.llmrs_attention_chunk()
+
+    @staticmethod
+    def gemm_workspace_floats(M: int, N: int, K: int) -> int:
+        """Room that lets a product with 33..64 tokens split K over blocks (the kernel's own rule)."""
+        if not 32 < M <= 64:
+            return 0
+        blocks, nkb, splits = -(-N // 64), -(-K // 64), 1
+        while blocks <= 64 and blocks * splits < 512 and splits < 16 and nkb // (splits * 2) >= 8:
+            splits *= 2
+        return splits * M * N if splits > 1 else 0
 
     def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int) -> int:
         """Room the split of single-token entries needs for its partial results."""
@@ -101,14 +111,17 @@ class HipKernels:
                                            n, x.shape[1], eps))
 
     # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
-    def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE) -> None:
+    def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
+             workspace: Optional[torch.Tensor] = None) -> None:
         M, K = a.shape
         N = w.shape[0]
         assert w.shape[1] == K and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1 and a.dtype == w.dtype
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
         assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
         self._check(self.lib.llmrs_gemm(self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
-                                        M, N, K, epilogue, int(self.allow_mfma)))
+                                        M, N, K, epilogue, _p(workspace),
+                                        0 if workspace is None else workspace.numel() * workspace.element_size(),
+                                        int(self.allow_mfma)))
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:
@@ -124,7 +137,7 @@ class HipKernels:
             page_size, num_pages, int(write_kv)))
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0) -> None:
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1) -> None:
         assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
@@ -135,7 +148,7 @@ class HipKernels:
             _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
             block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
             _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-            int(self.allow_mfma)))
+            int(n_single), int(self.allow_mfma)))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
         """`scratch`: 256 bytes per row let several blocks share a long row."""

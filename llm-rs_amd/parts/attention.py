@@ -69,7 +69,7 @@ class Attention(Mixer):
         write = self.kv_proj and cache.writes
         n_kv = self.kv_heads if self.kv_proj else 0
         qkv = ctx.workspace("attn.qkv", (T, self.q_size + 2 * n_kv * self.head_dim), self.dtype)
-        k.gemm(x, self.w_qkv, qkv, EPI_STORE)
+        k.gemm(x, self.w_qkv, qkv, EPI_STORE, ctx.gemm_workspace(x, self.w_qkv))
         rotary = self.position.rotary() if self.position is not None else None
         if rotary is None:
             if self.position is not None:
@@ -85,12 +85,12 @@ class Attention(Mixer):
                             cache.k, cache.v, self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
         o = ctx.workspace("attn.out", (T, self.q_size), self.dtype)
         # room for the partial results of single-token entries, which the kernel splits by key range
-        need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len)
+        need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len) if ctx.n_single else 0
         scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
-                    cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len)
-        k.gemm(o, self.w_o, h, EPI_ACCUM_F32)
+                    cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single)
+        k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
 
 
 register_mixer("attention", Attention)

@@ -36,8 +36,8 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, x, h):
         k = kernels()
         act = ctx.workspace("mlp.act", (x.shape[0], self.inter), self.dtype)
-        k.gemm(x, self.w_gate_up, act, EPI_SWIGLU)
-        k.gemm(act, self.w_down, h, EPI_ACCUM_F32)
+        k.gemm(x, self.w_gate_up, act, EPI_SWIGLU, ctx.gemm_workspace(x, self.w_gate_up))
+        k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
 
 
 register_feed_forward("swiglu", SwiGLU)

@@ -27,7 +27,11 @@ class EmulatedKernels:
         inv = 1.0 / torch.sqrt(ss / src.shape[-1] + eps)
         out.copy_((src * inv * weight).to(out.dtype))
 
-    def gemm(self, a, w, out, epilogue=EPI_STORE):
+    @staticmethod
+    def gemm_workspace_floats(M, N, K):
+        return 0
+
+    def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None):
         acc = a.float() @ w.float().T
         if epilogue == EPI_STORE:
             out.copy_(acc.to(out.dtype))
@@ -69,7 +73,7 @@ class EmulatedKernels:
             vc[page[t], :, :, off[t]] = heads[t, n_rot:, :]
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0):
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1):
         T = q.shape[0]
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
         vc = v_cache.view(num_pages, n_kv_heads, head_dim, page_size).float()
