@@ -14,11 +14,13 @@
 // kernel, never on M, the row's place in the batch or the tile it falls in.
 // Replaces the reference's matvec_bf16_simd / gemm_bf16 (shaders/ops.metal:52-159,
 // :1090-1143); unlike gemm_bf16 (:1107) the accumulator is 32-bit.
+#include "cache_layout.h"
 #include "gemm.h"
 
 #include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -61,7 +63,7 @@ template <int MT, int NT, int NW, int U>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
                                                               int ldc, int M, int N, int K, int epi,
-                                                              float* __restrict__ partial) {
+                                                              float* __restrict__ partial, QkvEpilogue qe) {
     extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
     float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -154,6 +156,43 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
             for (int r = 0; r < 4; r += 2)
                 if (n + r + 1 < N) ((bf16*)out)[(size_t)m * ldc + (n + r) / 2] = (bf16)(silu_f32(v[r]) * v[r + 1]);
+        } else if (epi == LLMRS_EPI_QKV) {
+            // four consecutive features of one head: two rotation pairs (2i, 2i+1); the
+            // rotation is applied to the 32-bit sums, which are rounded once
+            if (n >= N) continue;
+            int hd = qe.head_dim, head = n / hd, d = n % hd;
+            bool is_q = head < qe.n_heads, is_k = !is_q && head < qe.n_heads + qe.n_kv_heads;
+            if (is_q || is_k) {
+                float pos = (float)qe.positions[m];
+#pragma unroll
+                for (int r = 0; r < 4; r += 2)
+                    if (d + r < qe.rotary_dim) {
+                        float sn, cs;
+                        sincosf(pos * qe.inv_freq[(d + r) >> 1], &sn, &cs);
+                        float a = v[r], b = v[r + 1];
+                        v[r] = a * cs - b * sn;
+                        v[r + 1] = a * sn + b * cs;
+                    }
+            }
+            bf16x4 o4;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o4[r] = (bf16)v[r];
+            if (is_q) {
+                *(bf16x4*)((bf16*)out + (size_t)m * ldc + n) = o4;
+            } else if (qe.write_kv) {
+                int slot = qe.slot_map[m];
+                if (slot < 0 || slot >= qe.num_pages * qe.page_size) continue;   // never write outside the cache
+                int page = slot / qe.page_size, off = slot % qe.page_size;
+                if (is_k) {
+                    int kvh = head - qe.n_heads;
+                    *(bf16x4*)(qe.k_cache + k_cache_index(page, kvh, off, d, qe.n_kv_heads, qe.page_size, hd)) = o4;
+                } else {
+                    int kvh = head - qe.n_heads - qe.n_kv_heads;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        qe.v_cache[v_cache_index(page, kvh, off, d + r, qe.n_kv_heads, qe.page_size, hd)] = o4[r];
+                }
+            }
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -187,7 +226,8 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
 
 template <int MT, int NT, int NW, int U>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                          int M, int N, int K, int epi, int splits = 1, float* partial = nullptr) {
+                          int M, int N, int K, int epi, const QkvEpilogue* qkv, int splits = 1,
+                          float* partial = nullptr) {
     size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
     static bool configured = false;
     if (!configured) {
@@ -197,7 +237,8 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
     }
     dim3 grid(ceil_div(N, NT * 16), splits);
     gemm_skinny_kernel<MT, NT, NW, U><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
-                                                                          splits > 1 ? partial : nullptr);
+                                                                          splits > 1 ? partial : nullptr,
+                                                                          qkv ? *qkv : QkvEpilogue{});
     if (splits > 1) {
         size_t pairs = (size_t)M * ((N + 1) / 2);
         gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
@@ -338,8 +379,14 @@ static int launch_tiled(hipStream_t stream, const bf16* A, int lda, const bf16* 
 }
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                         int M, int N, int K, int epi, void* workspace, size_t workspace_bytes) {
+                         int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
+                         const QkvEpilogue* qkv) {
     if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return 0;
+    if (epi == LLMRS_EPI_QKV) {   // only the skinny kernel fuses it; its 8-byte stores need aligned rows
+        if (M > 64 || qkv == nullptr || qkv->head_dim % 4 || ldc % 4 || ((uintptr_t)out & 7) ||
+            ((uintptr_t)qkv->k_cache & 7) || qkv->rotary_dim % 4)
+            return 0;
+    }
     int rc = 0;
     if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
@@ -351,7 +398,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // (Measured on MI355X at the 8B shapes; see profiles/.)
         bool wide = N >= 16384;
         bool eight = !wide && K >= 2048;
-#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi)
+#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv)
         if (M <= 16) {
             if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else SKINNY(1, 4, 4, 2); }
             else if (eight) SKINNY(1, 1, 8, 4);
@@ -367,8 +414,9 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64);
             int splits = 1;
             while (blocks <= 64 && blocks * splits < 512 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
-            if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
-                launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
+            if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
+                workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+                launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
             } else if (wide) SKINNY(4, 4, 4, 2);
             else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
             else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }

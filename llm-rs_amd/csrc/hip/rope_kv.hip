@@ -10,6 +10,7 @@
 // The cache write replaces scatter_kv (shaders/ops.metal:841-853).
 #include "cache_layout.h"
 #include "common.h"
+#include "gemm.h"
 
 struct RopeKvArgs {
     int n_tokens, n_heads, n_kv_heads, head_dim;
@@ -94,4 +95,37 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
         return llmrs_fail("rope_kv_write: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("rope_kv_write");
     return 0;
+}
+
+extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
+                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma);
+
+// qkv = x W^T for W = [q heads; k heads; v heads], then what llmrs_rope_kv_write does,
+// with pairs (2i, 2i+1): in one kernel when the product is one the rotation fuses into
+// (bfloat16, up to 64 tokens), else as two.  In the fused case only q is written to
+// `qkv`; k and v go to the cache alone.
+extern "C" int llmrs_qkv_rope_cache(hipStream_t stream, int dtype, const void* x, int lda, const void* w, void* qkv,
+                                    int row_stride, int M, int K, const int* positions, const int* slot_map,
+                                    const float* inv_freq, int rotary_dim, void* k_cache, void* v_cache,
+                                    int n_heads, int n_kv_heads, int head_dim, int page_size, int num_pages,
+                                    int write_kv, void* workspace, size_t workspace_bytes, int allow_mfma) {
+    int N = (n_heads + 2 * n_kv_heads) * head_dim;
+    LLMRS_REQUIRE(M >= 0 && K > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "qkv_rope_cache: bad sizes");
+    LLMRS_REQUIRE(row_stride >= N && lda >= K, "qkv_rope_cache: row stride too short");
+    LLMRS_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+                  "qkv_rope_cache: rotary_dim %d does not fit head_dim %d", rotary_dim, head_dim);
+    LLMRS_REQUIRE(page_size > 0 && num_pages > 0, "qkv_rope_cache: bad cache geometry");
+    if (M == 0) return 0;
+    if (dtype == LLMRS_BF16 && allow_mfma) {
+        QkvEpilogue qe{positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, n_heads, n_kv_heads, head_dim,
+                       rotary_dim, page_size, num_pages, write_kv};
+        int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)x, lda, (const bf16*)w, qkv, row_stride, M, N, K,
+                                        LLMRS_EPI_QKV, nullptr, 0, &qe);
+        if (took != 0) return took < 0 ? -1 : 0;
+    }
+    int rc = llmrs_gemm(stream, dtype, x, lda, w, qkv, row_stride, M, N, K, LLMRS_EPI_STORE, workspace, workspace_bytes,
+                        allow_mfma);
+    if (rc != 0) return rc;
+    return llmrs_rope_kv_write(stream, dtype, qkv, row_stride, positions, slot_map, inv_freq, rotary_dim, 1, k_cache,
+                               v_cache, M, n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv);
 }

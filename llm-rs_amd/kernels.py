@@ -53,6 +53,7 @@ class HipKernels:
             "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
+            "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I],
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
         }
@@ -135,6 +136,22 @@ class HipKernels:
             self._stream(), _code(qkv.dtype), _p(qkv), qkv.stride(0), _p(positions), _p(slot_map), _p(inv_freq),
             rotary_dim, int(interleaved), _p(k_cache), _p(v_cache), qkv.shape[0], n_heads, n_kv_heads, head_dim,
             page_size, num_pages, int(write_kv)))
+
+    def qkv_rope_cache(self, x, w, qkv, positions, slot_map, inv_freq, rotary_dim, k_cache, v_cache,
+                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv, workspace=None) -> None:
+        """qkv = x @ w.T, q and k rotated by adjacent pairs (2i, 2i+1), k and v written to the cache: fused into
+        one kernel where the product allows.  Afterwards only the q part of `qkv` is certain to be filled."""
+        assert x.stride(1) == 1 and qkv.stride(1) == 1 and w.is_contiguous() and x.dtype == w.dtype == qkv.dtype
+        assert w.shape[0] == (n_heads + 2 * n_kv_heads) * head_dim and w.shape[1] == x.shape[1] and qkv.shape[0] == x.shape[0]
+        assert rotary_dim == 0 or (inv_freq.dtype == torch.float32 and inv_freq.shape[0] == rotary_dim // 2)
+        if write_kv:
+            assert k_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
+            assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
+        self._check(self.lib.llmrs_qkv_rope_cache(
+            self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(w), _p(qkv), qkv.stride(0), x.shape[0], x.shape[1],
+            _p(positions), _p(slot_map), _p(inv_freq), rotary_dim, _p(k_cache), _p(v_cache), n_heads, n_kv_heads,
+            head_dim, page_size, num_pages, int(write_kv), _p(workspace),
+            0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma)))
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1) -> None:

@@ -6,9 +6,16 @@ earlier key), position (a position-encoding spec or None), scale (None:
 v of its own and only reads a cache that another run wrote).
 
 One step (src/arch/llama.rs:153-163): q, k, v = x Wq^T, x Wk^T, x Wv^T in one
-product over the row-concatenated weight; rotate q and k and write k, v into
-their pages in one kernel; attention of every query token over its request's
-pages; h += o Wo^T with the sum fused into the product.  No biases.
+product over the row-concatenated weight; q and k rotated and k, v written into
+their pages by the same kernel (for a few tokens) or the next; attention of
+every query token over its request's pages; h += o Wo^T with the sum fused into
+the product.  No biases.
+
+The rotation kernels pair neighbours (2i, 2i+1).  Where the encoding pairs
+(i, i + rotary_dim/2), the rows of Wq and Wk are reordered within each head at
+load so that those two features become neighbours: q.k is a sum over features
+and does not care in which order q and k list them, as long as it is the same;
+the reference runs files converted for exactly this order (src/arch/llama.rs:156).
 """
 from __future__ import annotations
 
@@ -53,9 +60,22 @@ class Attention(Mixer):
             t[self.name("v_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
         return t
 
+    def _pair_neighbours(self, w: torch.Tensor, heads: int) -> torch.Tensor:
+        """Rows of a q or k weight reordered so that each rotation pair is (2i, 2i+1)."""
+        rotary = self.position.rotary() if self.position is not None else None
+        if rotary is None or rotary[2] or rotary[1] == 0:
+            return w          # no rotation here, or the pairs are neighbours already
+        rot = rotary[1]
+        order = torch.stack([torch.arange(rot // 2), torch.arange(rot // 2) + rot // 2], dim=1).flatten()
+        order = torch.cat([order, torch.arange(rot, self.head_dim)]).to(w.device)
+        return w.view(heads, self.head_dim, -1)[:, order, :].reshape(w.shape)
+
     def load(self, tensors, device):
-        names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.kv_proj else [])
-        self.w_qkv = torch.cat([tensors[self.name(n)].to(device=device, dtype=self.dtype) for n in names], dim=0).contiguous()
+        get = lambda n: tensors[self.name(n)].to(device=device, dtype=self.dtype)
+        parts = [self._pair_neighbours(get("q_proj.weight"), self.heads)]
+        if self.kv_proj:
+            parts += [self._pair_neighbours(get("k_proj.weight"), self.kv_heads), get("v_proj.weight")]
+        self.w_qkv = torch.cat(parts, dim=0).contiguous()
         self.w_o = tensors[self.name("o_proj.weight")].to(device=device, dtype=self.dtype).contiguous()
         if self.position is not None:
             self.position.to(device)
@@ -69,20 +89,21 @@ class Attention(Mixer):
         write = self.kv_proj and cache.writes
         n_kv = self.kv_heads if self.kv_proj else 0
         qkv = ctx.workspace("attn.qkv", (T, self.q_size + 2 * n_kv * self.head_dim), self.dtype)
-        k.gemm(x, self.w_qkv, qkv, EPI_STORE, ctx.gemm_workspace(x, self.w_qkv))
         rotary = self.position.rotary() if self.position is not None else None
-        if rotary is None:
-            if self.position is not None:
-                q3 = qkv[:, :self.q_size].unflatten(1, (self.heads, self.head_dim))
-                k3 = qkv[:, self.q_size:self.q_size + self.kv_size].unflatten(1, (self.kv_heads, self.head_dim)) if n_kv else None
-                self.position.apply(ctx, q3, k3)
-            inv_freq, rotary_dim, interleaved = None, 0, False
-        else:
-            inv_freq, rotary_dim, interleaved = rotary
         g = cache.group
-        if write or rotary_dim:
-            k.rope_kv_write(qkv, ctx.positions, ctx.slot_maps[g], inv_freq, rotary_dim, interleaved,
-                            cache.k, cache.v, self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
+        if self.position is None or rotary is not None:
+            inv_freq, rotary_dim = (None, 0) if rotary is None else rotary[:2]
+            k.qkv_rope_cache(x, self.w_qkv, qkv, ctx.positions, ctx.slot_maps[g], inv_freq, rotary_dim, cache.k, cache.v,
+                             self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write,
+                             ctx.gemm_workspace(x, self.w_qkv))
+        else:     # an encoding of its own: it changes q and k between the product and the cache write
+            k.gemm(x, self.w_qkv, qkv, EPI_STORE, ctx.gemm_workspace(x, self.w_qkv))
+            q3 = qkv[:, :self.q_size].unflatten(1, (self.heads, self.head_dim))
+            k3 = qkv[:, self.q_size:self.q_size + self.kv_size].unflatten(1, (self.kv_heads, self.head_dim)) if n_kv else None
+            self.position.apply(ctx, q3, k3)
+            if write:
+                k.rope_kv_write(qkv, ctx.positions, ctx.slot_maps[g], None, 0, False, cache.k, cache.v,
+                                self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
         o = ctx.workspace("attn.out", (T, self.q_size), self.dtype)
         # room for the partial results of single-token entries, which the kernel splits by key range
         need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len) if ctx.n_single else 0

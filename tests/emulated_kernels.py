@@ -72,6 +72,12 @@ class EmulatedKernels:
             kc[page[t], :, off[t], :] = x[t, n_heads:, :]
             vc[page[t], :, :, off[t]] = heads[t, n_rot:, :]
 
+    def qkv_rope_cache(self, x, w, qkv, positions, slot_map, inv_freq, rotary_dim, k_cache, v_cache,
+                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv, workspace=None):
+        self.gemm(x, w, qkv, EPI_STORE)
+        self.rope_kv_write(qkv, positions, slot_map, inv_freq, rotary_dim, True, k_cache, v_cache,
+                           n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv)
+
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1):
         T = q.shape[0]

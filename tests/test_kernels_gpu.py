@@ -368,3 +368,40 @@ def test_sample_rows_frequencies():
     freq = torch.bincount(out.cpu().long(), minlength=V).double() / n
     p = torch.softmax(row.double(), 0)
     assert (freq - p).abs().max() < 4 * (p * (1 - p) / n).sqrt().max() + 1e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M", [1, 8, 20, 50, 100])
+@pytest.mark.parametrize("n_heads,n_kv,hd,rot,K", [(4, 2, 32, 32, 256), (8, 2, 128, 128, 512), (3, 1, 64, 32, 96), (2, 2, 16, 0, 64)])
+def test_qkv_rope_cache(dtype, M, n_heads, n_kv, hd, rot, K):
+    """The product, the rotation by neighbouring pairs and the cache write, as one call: for a few
+    bfloat16 tokens it is one kernel that rotates the 32-bit sums; else product, then rotation."""
+    page_size, num_pages = 16, 12
+    N = (n_heads + 2 * n_kv) * hd
+    x = rnd((M, K), dtype, 30)
+    w = rnd((N, K), dtype, 31, 0.1)
+    positions = torch.randint(0, 400, (M,), generator=torch.Generator().manual_seed(32)).to(torch.int32).to(DEV)
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(33))[:M].to(torch.int32).to(DEV)
+    inv_freq = plain_inv_freq(rot, 10000.0, None).to(DEV) if rot else None
+    qkv = torch.zeros((M, N + 8), dtype=dtype, device=DEV)
+    kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=dtype, device=DEV)
+    vc = torch.zeros((num_pages, n_kv, hd, page_size), dtype=dtype, device=DEV)
+    kernels().qkv_rope_cache(x, w, qkv[:, :N], positions, slots, inv_freq, rot, kc, vc, n_heads, n_kv, hd,
+                             page_size, num_pages, True)
+    acc = x.double().cpu() @ w.double().cpu().T
+    q = acc[:, :n_heads * hd].view(M, n_heads, hd)
+    k = acc[:, n_heads * hd:(n_heads + n_kv) * hd].view(M, n_kv, hd)
+    v = acc[:, (n_heads + n_kv) * hd:].view(M, n_kv, hd)
+    if rot:
+        q = plain_rope(q, positions.cpu(), inv_freq.cpu(), "interleaved")
+        k = plain_rope(k, positions.cpu(), inv_freq.cpu(), "interleaved")
+    floor = 2e-6 * math.sqrt(K) if dtype == torch.float32 else 2e-2
+    page, off = (slots // page_size).long().cpu(), (slots % page_size).long().cpu()
+    got_q = qkv[:, :n_heads * hd].double().cpu().view(M, n_heads, hd)
+    got_k = kc.double().cpu()[page, :, off, :]
+    got_v = vc.double().cpu()[page, :, :, off]
+    rel = 1.0 / 40 if dtype == torch.bfloat16 else 1e-5       # bfloat16 may round twice (product, then rotation)
+    for name, got, ref in (("q", got_q, q), ("k", got_k, k), ("v", got_v, v)):
+        err = (got - ref).abs()
+        assert (err <= ref.abs() * rel + floor).all(), f"{name}: max err {float(err.max())}"
+    assert (qkv[:, N:] == 0).all(), "padding touched"
