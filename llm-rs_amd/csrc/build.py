@@ -134,7 +134,8 @@ def build_hip(force: bool = False) -> str:
         with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
             objs = list(ex.map(compile_one, srcs))
         tmp = f"{lib}.{os.getpid()}.tmp"
-        _run([hipcc, "-shared", "-fPIC", f"--offload-arch={GPU_ARCH}", "-o", tmp, *objs], "linking the kernel library")
+        _run([hipcc, "-shared", "-fPIC", f"--offload-arch={GPU_ARCH}", "-Wl,--no-undefined", "-o", tmp, *objs],
+             "linking the kernel library")
         _finish(lib, tmp, "hip")
     finally:
         shutil.rmtree(objdir, ignore_errors=True)

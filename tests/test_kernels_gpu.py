@@ -36,7 +36,7 @@ def test_embed_rows(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("D,eps", [(200, 1e-5), (4104, 1e-6), (64, 1e-2)])
+@pytest.mark.parametrize("D,eps", [(200, 1e-5), (4104, 1e-6), (64, 1e-2), (4098, 1e-5), (20000, 1e-5)])
 def test_rmsnorm(dtype, D, eps):
     x = rnd((9, D), torch.float32, 1, 3.0)
     w = rnd((D,), torch.float32, 2) * 0.1 + 1
