@@ -63,6 +63,54 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
     }
 }
 
+// A few tokens (decoding): a wave for each pair of weight rows, every weight read once.
+// Lanes stride over k, four elements at a time, and each keeps one 32-bit sum per token and
+// row; the lanes' sums are added by a butterfly.  The order depends on K only.
+#define GEMV_MAX_M 8
+template <class T>
+__global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W,
+                                                        void* __restrict__ out, int ldc, int M, int N, int K, int epi) {
+    int lane = threadIdx.x & 63;
+    int n = 2 * (blockIdx.x * 4 + (threadIdx.x >> 6));
+    if (n >= N) return;
+    bool two = n + 1 < N;
+    const T* w0 = W + (size_t)n * K;
+    const T* w1 = W + (size_t)(two ? n + 1 : n) * K;
+    float acc0[GEMV_MAX_M] = {}, acc1[GEMV_MAX_M] = {};
+    for (int k = lane * 4; k < K; k += 256) {
+        float a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            bool in = k + j < K;
+            a[j] = in ? to_f32(w0[k + j]) : 0.0f;
+            b[j] = in ? to_f32(w1[k + j]) : 0.0f;
+        }
+#pragma unroll
+        for (int m = 0; m < GEMV_MAX_M; ++m) {
+            if (m >= M) break;
+            const T* x = A + (size_t)m * lda + k;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float xv = k + j < K ? to_f32(x[j]) : 0.0f;
+                acc0[m] = fmaf(a[j], xv, acc0[m]);
+                acc1[m] = fmaf(b[j], xv, acc1[m]);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < GEMV_MAX_M; ++m) {
+        if (m >= M) break;
+        float v0 = wave_sum(acc0[m]), v1 = wave_sum(acc1[m]);
+        if (lane != 0) continue;
+        if (epi == LLMRS_EPI_SWIGLU) {
+            if (two) ((T*)out)[(size_t)m * ldc + n / 2] = from_f32<T>(silu_f32(v0) * v1);
+        } else {
+            epilogue_store<T>(epi, out, ldc, m, n, v0);
+            if (two) epilogue_store<T>(epi, out, ldc, m, n + 1, v1);
+        }
+    }
+}
+
 // A: [M, K] with row stride lda; W: [N, K] dense; out: row stride ldc (elements of
 // its own type; for SWIGLU the output has N/2 columns).  workspace: optional device
 // memory (16 * 64 * N * 4 bytes is always enough) for products that split K over blocks.
@@ -82,6 +130,17 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi, workspace,
                                         workspace_bytes);
         if (took != 0) return took < 0 ? -1 : 0;
+    }
+    if (M <= GEMV_MAX_M) {
+        int blocks = ceil_div(N, 8);
+        if (dtype == LLMRS_F32)
+            gemm_rows_kernel<float><<<blocks, 256, 0, stream>>>((const float*)A, lda, (const float*)W, out, ldc, M, N, K, epi);
+        else if (dtype == LLMRS_BF16)
+            gemm_rows_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
+        else
+            return llmrs_fail("gemm: unknown dtype %d", dtype);
+        LLMRS_LAUNCH_CHECK("gemm");
+        return 0;
     }
     dim3 grid(ceil_div(N, TILE), ceil_div(M, TILE));
     LLMRS_REQUIRE(grid.y <= 65535, "gemm: M=%d is too large for one launch", M);
