@@ -6,7 +6,8 @@
 //            its waves split K, so a layer's product has enough loads in flight to
 //            keep HBM busy.  v_mfma_f32_16x16x32_bf16, weights as the A operand.
 //   M  > 64  "tiled": prompts.  128x128 tiles of the output, K in steps of 64
-//            through double-buffered LDS, v_mfma_f32_32x32x16_bf16.
+//            through double-buffered LDS, v_mfma_f32_32x32x16_bf16; the tiles are
+//            loaded straight into LDS (global_load_lds) when K % 64 == 0.
 // Both need K % 8 == 0 and 16-byte aligned rows (16-byte loads); otherwise the
 // caller falls back to the plain kernel.
 //
@@ -378,6 +379,146 @@ static int launch_tiled(hipStream_t stream, const bf16* A, int lda, const bf16* 
     return 0;
 }
 
+// ---------------------------------------------------------------------------
+// tiled, loads straight into LDS: for K % 64 == 0.
+// global_load_lds_dwordx4 moves 16 bytes per lane from memory into LDS without
+// passing through registers; the 64 lanes of an instruction fill 1 KB of LDS in
+// lane order, which is 8 tile rows of 64 k.  Rows therefore lie 128 bytes apart,
+// unpadded, and bank conflicts are avoided by a swizzle instead: the 16-byte
+// chunk c of row r lies in slot c ^ ((r >> 1) & 7) of its row (each lane simply
+// fetches the chunk that belongs in its slot), so the 16 lanes of an operand read,
+// which want the same chunk of 16 consecutive rows, hit 16 different bank groups.
+// STAGES tiles are in LDS; the loads of the tile STAGES-1 ahead are issued
+// before this tile's products and waited for (s_waitcnt vmcnt) only as far as the
+// next tile needs.  No staging registers, no LDS store instructions.
+// ---------------------------------------------------------------------------
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N_ >= 0 && N_ < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
+}
+
+template <int BM, int BN, int STAGES>
+__global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16* __restrict__ A, int lda,
+                                                       const bf16* __restrict__ W, void* __restrict__ out,
+                                                       int ldc, int M, int N, int K, int epi) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char dma_smem[];
+    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
+    constexpr int STAGE_BYTES = (BM + BN) * 128;
+    constexpr int A_GROUPS = BM / 8 / 4, W_GROUPS = BN / 8 / 4;   // 8-row groups per wave
+    constexpr int LOADS = A_GROUPS + W_GROUPS;                     // load instructions per wave per tile
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int wm = wave >> 1, wn = wave & 1;
+    int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    int lrow = lane >> 3, lslot = lane & 7;
+
+    // this lane's part of a tile: for each of its row groups, the row's global address of the
+    // chunk that belongs in the lane's slot
+    const bf16* ga[A_GROUPS];
+    const bf16* gw[W_GROUPS];
+#pragma unroll
+    for (int i = 0; i < A_GROUPS; ++i) {
+        int row = (wave * A_GROUPS + i) * 8 + lrow;
+        ga[i] = A + (size_t)min(m0 + row, M - 1) * lda + ((lslot ^ ((row >> 1) & 7)) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+        int row = (wave * W_GROUPS + i) * 8 + lrow;
+        gw[i] = W + (size_t)min(n0 + row, N - 1) * K + ((lslot ^ ((row >> 1) & 7)) * 8);
+    }
+    auto issue = [&](int kt, int stage) {
+        unsigned base = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + wave * A_GROUPS * 1024);
+#pragma unroll
+        for (int i = 0; i < A_GROUPS; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ga[i] + kt * 64),
+                                             (__attribute__((address_space(3))) void*)(dma_smem + base + i * 1024), 16, 0, 0);
+        unsigned wbase = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + BM * 128 + wave * W_GROUPS * 1024);
+#pragma unroll
+        for (int i = 0; i < W_GROUPS; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gw[i] + kt * 64),
+                                             (__attribute__((address_space(3))) void*)(dma_smem + wbase + i * 1024), 16, 0, 0);
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    int nk = K / 64;
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if (p < nk) issue(p, p);
+    if (nk >= STAGES - 1) wait_vmcnt<(STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
+    __syncthreads();
+
+    int frow = lane & 31, h = lane >> 5;
+    for (int kt = 0; kt < nk; ++kt) {
+        int stage = kt % STAGES;
+        if (kt + STAGES - 1 < nk) issue(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+        const unsigned char* as = dma_smem + stage * STAGE_BYTES;
+        const unsigned char* ws = as + BM * 128;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            bf16x8 a[FM], b[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+                int row = wm * TM + i * 32 + frow;
+                a[i] = *(const bf16x8*)(as + row * 128 + (((ks * 2 + h) ^ ((row >> 1) & 7)) * 16));
+            }
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                int row = wn * TN + j * 32 + frow;
+                b[j] = *(const bf16x8*)(ws + row * 128 + (((ks * 2 + h) ^ ((row >> 1) & 7)) * 16));
+            }
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        // the next tile must have landed before anybody reads it; later tiles may still be on their way
+        if (kt + STAGES - 1 < nk) wait_vmcnt<(STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
+        __syncthreads();
+    }
+
+    static_for<0, FM * FN>([&](auto idx) {
+        constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
+        int n = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            float v = acc[i][j][r];
+            if (epi == LLMRS_EPI_SWIGLU) {
+                float other = __shfl_xor(v, 1, 64);
+                if (!(lane & 1) && m < M && n + 1 < N)
+                    ((bf16*)out)[(size_t)m * ldc + n / 2] = (bf16)(silu_f32(v) * other);
+            } else if (m < M && n < N) {
+                epilogue_store<bf16>(epi, out, ldc, m, n, v);
+            }
+        }
+    });
+}
+
+template <int BM, int BN, int STAGES>
+static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
+                      int M, int N, int K, int epi) {
+    static bool configured = false;
+    size_t bytes = (size_t)STAGES * (BM + BN) * 128;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_dma_kernel<BM, BN, STAGES>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+        configured = true;
+    }
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
+    if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
+    gemm_dma_kernel<BM, BN, STAGES><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    return 0;
+}
+
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
                          const QkvEpilogue* qkv) {
@@ -425,7 +566,11 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
     } else {
         // 128 x 128 x 64 with one tile of loads in flight measured best of the tile shapes
         // tried here (larger tiles need a path without bounds checks to pay off).
-        rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        // K % 64 == 0: loads straight into LDS, 128 x 128 tiles, two tiles in LDS (measured best of
+        // 128x128, 256x128, 128x256 and 256x256 with 2 or 3 tiles: two blocks fit a CU and hide each
+        // other's waits).  Other K: through registers, with zero-filled tails.
+        if (K % 64 == 0) rc = launch_dma<128, 128, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        else rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
     if (rc != 0) return -1;
     hipError_t e = hipGetLastError();

@@ -54,7 +54,8 @@ def test_rmsnorm(dtype, D, eps):
 GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256, 128), (65, 130, 1024),
                (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20),
                (64, 200, 2048), (40, 1000, 1096), (64, 4096, 4096), (24, 520, 2048), (50, 64, 8200),
-               (8, 38, 100), (3, 130, 4099), (1, 6, 20)]
+               (8, 38, 100), (3, 130, 4099), (1, 6, 20),
+               (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
