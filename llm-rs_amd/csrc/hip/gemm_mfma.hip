@@ -398,17 +398,18 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
 }
 
-template <int BM, int BN, int STAGES>
-__global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16* __restrict__ A, int lda,
+template <int BM, int BN, int WGM, int WGN, int STAGES>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __restrict__ A, int lda,
                                                        const bf16* __restrict__ W, void* __restrict__ out,
                                                        int ldc, int M, int N, int K, int epi) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char dma_smem[];
-    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
+    constexpr int WAVES = WGM * WGN;                              // waves of a block, as a WGM x WGN grid over the tile
+    constexpr int TM = BM / WGM, TN = BN / WGN, FM = TM / 32, FN = TN / 32;
     constexpr int STAGE_BYTES = (BM + BN) * 128;
-    constexpr int A_GROUPS = BM / 8 / 4, W_GROUPS = BN / 8 / 4;   // 8-row groups per wave
+    constexpr int A_GROUPS = BM / 8 / WAVES, W_GROUPS = BN / 8 / WAVES;   // 8-row groups per wave
     constexpr int LOADS = A_GROUPS + W_GROUPS;                     // load instructions per wave per tile
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int wm = wave >> 1, wn = wave & 1;
+    int wm = wave / WGN, wn = wave % WGN;
     int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     int lrow = lane >> 3, lslot = lane & 7;
 
@@ -502,20 +503,20 @@ __global__ __launch_bounds__(256) void gemm_dma_kernel(const bf16* __restrict__ 
     });
 }
 
-template <int BM, int BN, int STAGES>
+template <int BM, int BN, int WGM, int WGN, int STAGES>
 static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                       int M, int N, int K, int epi) {
     static bool configured = false;
     size_t bytes = (size_t)STAGES * (BM + BN) * 128;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_dma_kernel<BM, BN, STAGES>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_dma_kernel<BM, BN, WGM, WGN, STAGES>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
         configured = true;
     }
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
-    gemm_dma_kernel<BM, BN, STAGES><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    gemm_dma_kernel<BM, BN, WGM, WGN, STAGES><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
     return 0;
 }
 
@@ -566,10 +567,14 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
     } else {
         // 128 x 128 x 64 with one tile of loads in flight measured best of the tile shapes
         // tried here (larger tiles need a path without bounds checks to pay off).
-        // K % 64 == 0: loads straight into LDS, 128 x 128 tiles, two tiles in LDS (measured best of
-        // 128x128, 256x128, 128x256 and 256x256 with 2 or 3 tiles: two blocks fit a CU and hide each
-        // other's waits).  Other K: through registers, with zero-filled tails.
-        if (K % 64 == 0) rc = launch_dma<128, 128, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        // K % 64 == 0: loads straight into LDS, two tiles in LDS.  Other K: through registers, with
+        // zero-filled tails.
+        // with 128 x 64 per wave (eight waves on a 256 x 256 tile) there is one LDS read per MFMA less
+        // than with 64 x 64 (four waves on 128 x 128), and the loop is bound by LDS bandwidth; it pays
+        // as soon as the larger tiles still fill most of the device (measured on MI355X)
+        long big_tiles = (long)ceil_div(M, 256) * ceil_div(N, 256);
+        if (K % 64 == 0 && big_tiles >= 160) rc = launch_dma<256, 256, 2, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        else if (K % 64 == 0) rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
         else rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
     if (rc != 0) return -1;
