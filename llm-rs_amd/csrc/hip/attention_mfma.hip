@@ -33,9 +33,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 extern "C" int llmrs_attention_chunk() { return ATTN_CHUNK; }
 
-struct TileState {
-    float m, l;
-};
+// all of this wave's vector memory operations, loads into LDS among them, have completed
+__device__ __forceinline__ void wait_vmcnt_all() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8)); }
 
 // One wave: keys [t_begin, t_end) (t_begin a multiple of 32) against its 32 columns.
 // pos / lo: this lane's column may see keys lo..pos (pos < 0: nothing).
@@ -171,6 +170,169 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
         }
 }
 
+// ---- the same for head sizes 64, 128, 256, with the four waves of a block sharing their keys --
+// The block's waves own four consecutive groups of tokens of one request and one kv head, so they
+// want the same keys and values (up to the causal edge).  Each 32-key tile (two pages) is
+// brought into LDS once, by global_load_lds straight from the cache's pages, while the tile
+// before it is worked on; all four waves read their MFMA operands from there.  A key's row
+// is 2*HD bytes and the rows lie unpadded, so chunk c of key kk is kept in slot c ^ swz(kk)
+// (swz: kk for 256-byte rows and longer, kk >> 1 for 128-byte rows): the 16 lanes of an operand
+// read want one chunk of 16 different keys and then hit 16 different bank groups.  Values are
+// [HD][16] per page and are read in lane order; they need no swizzle.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
+                                                             const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                                             const int* __restrict__ block_table,
+                                                             const int* __restrict__ positions,
+                                                             const int* __restrict__ q_starts, int n_entries,
+                                                             AttnArgs a, int G, int tpt, int skip_single) {
+    constexpr int CHUNKS = HD / 8;                  // 16-byte chunks in a key's row
+    constexpr int ROW_BYTES = HD * 2;
+    constexpr int PAGE_BYTES = 16 * ROW_BYTES;      // a page of one kv head: keys [16][HD], values [HD][16]
+    constexpr int STAGE_BYTES = 4 * PAGE_BYTES;     // K page 0, K page 1, V page 0, V page 1
+    constexpr int LOADS = PAGE_BYTES / 1024;        // load instructions per wave per tile (4 pages over 4 waves)
+    constexpr int SWZ_SHIFT = ROW_BYTES >= 256 ? 0 : 1;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE_BYTES];
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int c = lane & 31, h = lane >> 5;
+    int kvh = blockIdx.x % a.n_kv_heads;
+    int btile = blockIdx.x / a.n_kv_heads;          // a block's tile: 4 * tpt tokens of one entry
+    int e = 0, rem = btile;
+    for (; e < n_entries; ++e) {
+        int cnt = q_starts[e + 1] - q_starts[e];
+        int nt = (cnt == 1 && skip_single) ? 0 : (cnt + 4 * tpt - 1) / (4 * tpt);
+        if (rem < nt) break;
+        rem -= nt;
+    }
+    if (e == n_entries) return;
+    int e_end = q_starts[e + 1];
+    int btok0 = q_starts[e] + rem * 4 * tpt;
+    int btok_last = min(btok0 + 4 * tpt, e_end) - 1;
+    // this wave's tokens (it may have none, at the end of an entry: it still helps to load)
+    int tok0 = btok0 + wave * tpt;
+    int ntok = max(0, min(tpt, e_end - tok0));
+    bool wave_active = ntok > 0;
+    int tq = c / G, hg = c - tq * G;
+    bool cvalid = tq < ntok;
+    int token = wave_active ? tok0 + min(tq, ntok - 1) : btok0;
+    int head = kvh * G + hg;
+    int pos = cvalid ? positions[token] : -1;
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int b_first = positions[btok0], b_last = positions[btok_last];
+    int t_end = b_last + 1;                                          // keys the block needs: [t_begin, t_end)
+    int t_begin = ((a.window > 0 && b_first + 1 > a.window) ? b_first + 1 - a.window : 0) & ~31;
+    int w_end = wave_active ? positions[tok0 + ntok - 1] + 1 : 0;     // keys this wave needs end here
+    int w_begin = wave_active ? (((a.window > 0 && positions[tok0] + 1 > a.window) ? positions[tok0] + 1 - a.window : 0) & ~31) : 0;
+    const int* table = block_table + (size_t)e * a.table_width;
+
+    bf16x8 qf[HD / 16];
+    const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+    f32x16 O[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    // Wave w brings page w of a tile's four (K0, K1, V0, V1) into LDS.
+    auto issue = [&](int t0, int stage) {
+        int lp = t0 >> 4;
+        int p0 = table[min(lp, a.table_width - 1)];
+        int p1 = (t0 + 16 < t_end) ? table[min(lp + 1, a.table_width - 1)] : p0;
+        int page = (wave & 1) ? p1 : p0;
+        page = min(max(page, 0), a.num_pages - 1);
+        const unsigned char* src = (const unsigned char*)((wave < 2 ? kc : vc) + ((size_t)page * a.n_kv_heads + kvh) * (16 * HD));
+        unsigned base = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + wave * PAGE_BYTES);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            int off = i * 1024 + lane * 16;          // the lane's place in the page's LDS image
+            int goff = off;
+            if (wave < 2) {                          // keys: fetch the chunk that belongs in this slot
+                int kk = off / ROW_BYTES, slot = (off % ROW_BYTES) / 16;
+                goff = kk * ROW_BYTES + ((slot ^ ((kk >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);
+            }
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + goff),
+                                             (__attribute__((address_space(3))) void*)(lds + base + i * 1024), 16, 0, 0);
+        }
+    };
+
+    int r = lane & 31;
+    int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
+    issue(t_begin, 0);
+    wait_vmcnt_all();
+    __syncthreads();
+    int stage = 0;
+    for (int t0 = t_begin; t0 < t_end; t0 += 32, stage ^= 1) {
+        if (t0 + 32 < t_end) issue(t0 + 32, stage ^ 1);
+        if (t0 >= w_begin && t0 < w_end) {
+            const unsigned char* kb = lds + stage * STAGE_BYTES + (kk >> 4) * PAGE_BYTES + (kk & 15) * ROW_BYTES;
+            const unsigned char* vb = lds + stage * STAGE_BYTES + 2 * PAGE_BYTES + r * 32 + h * 16;
+            int kswz = ((kk & 15) >> SWZ_SHIFT) & (CHUNKS - 1) & 15;
+            f32x16 S;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < HD / 16; ++ks) {
+                bf16x8 kf = *(const bf16x8*)(kb + (((ks * 2 + h) ^ kswz) * 16));
+                S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
+                float sv = S[i] * a.scale;
+                sv = (key > pos || key < lo) ? -INFINITY : sv;
+                S[i] = sv;
+                mx = fmaxf(mx, sv);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            float m_new = fmaxf(m, mx);
+            float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+            float alpha = expf(m - m_safe);
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                S[i] = expf(S[i] - m_safe);
+                sum += S[i];
+            }
+            sum += __shfl_xor(sum, 32, 64);
+            l = l * alpha + sum;
+            m = m_new;
+            bf16x8 pf[2];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pf[0][i] = (bf16)S[i];
+                pf[1][i] = (bf16)S[8 + i];
+            }
+#pragma unroll
+            for (int dt = 0; dt < HD / 32; ++dt) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                bf16x8 v0 = *(const bf16x8*)(vb + dt * 32 * 32);
+                bf16x8 v1 = *(const bf16x8*)(vb + PAGE_BYTES + dt * 32 * 32);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pf[0], O[dt], 0, 0, 0);
+                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pf[1], O[dt], 0, 0, 0);
+            }
+        }
+        wait_vmcnt_all();      // the next tile has landed ...
+        __syncthreads();       // ... for everybody, and everybody is done with this one
+    }
+    if (!cvalid) return;
+    float inv = 1.0f / l;
+    bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+            bf16x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = (bf16)(O[dt][i4 * 4 + j] * inv);
+            *(bf16x4*)(op + o_feature(dt, i4 * 4, h)) = v;
+        }
+}
+
 // ---- entries with one token: a wave for each (entry, kv head, chunk of keys) --
 // partial: [(entry * n_heads + head) * max_chunks + chunk][HD + 2] = m, l, O (not yet divided)
 template <int HD>
@@ -262,9 +424,15 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
     int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
     if (!only_single) {
-        int tiles = a.n_tokens / tpt + n_entries;
-        int blocks = ((tiles + 3) / 4) * a.n_kv_heads;
-        attn_tiles_kernel<HD><<<blocks, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts, n_entries, a, G, tpt, split);
+        if constexpr (HD == 64 || HD == 128 || HD == 256) {
+            int btiles = a.n_tokens / (4 * tpt) + n_entries;
+            attn_tiles_lds_kernel<HD><<<btiles * a.n_kv_heads, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
+                                                                                 n_entries, a, G, tpt, split);
+        } else {
+            int tiles = a.n_tokens / tpt + n_entries;
+            int blocks = ((tiles + 3) / 4) * a.n_kv_heads;
+            attn_tiles_kernel<HD><<<blocks, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts, n_entries, a, G, tpt, split);
+        }
     }
     if (split) {
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
