@@ -21,8 +21,9 @@
 // request's length only) and merged in ascending order by a second kernel.
 //
 // Math as in the reference's paged_attention (shaders/ops.metal:636-758): scale
-// after the dot, mask = loop bound, max/exp/sums in 32-bit.  Probabilities are
-// rounded to bfloat16 for the second product; their sum is not.
+// after the dot, mask = loop bound, max/exp/sums in 32-bit (the exponential as
+// 2^(x log2 e), one instruction).  Probabilities are rounded to bfloat16 for the
+// second product; their sum is not.
 #include "attention.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -35,6 +36,48 @@ extern "C" int llmrs_attention_chunk() { return ATTN_CHUNK; }
 
 // all of this wave's vector memory operations, loads into LDS among them, have completed
 __device__ __forceinline__ void wait_vmcnt_all() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8)); }
+// all but the last N_ of them have completed (they complete in order)
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt_n() {
+    static_assert(N_ >= 0 && N_ < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
+}
+
+// The softmax step of one 32-key tile for this lane's column.  S + S2 are the raw dots of the
+// lane's 16 keys; on return S holds their probabilities relative to the new running maximum
+// (not yet normalised), m and l are updated, alpha is what the older sums must be scaled by.
+// Scores are kept in the base-2 domain, (q.k) * scale * log2(e), so that the exponential is
+// one v_exp_f32; max, sums and scale factors are 32-bit as everywhere.  Keys outside
+// [lo, pos] are masked; the comparison is skipped for tiles that lie wholly inside every
+// column's range (all of a tile's lanes agree on that, so the branch is uniform).
+__device__ __forceinline__ void softmax_tile(f32x16& S, const f32x16& S2, float& m, float& l, int t0, int pos, int lo,
+                                             int h, float scale_log2e, float& alpha) {
+    bool edge = __any(t0 + 31 > pos || t0 < lo);
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        float sv = (S[i] + S2[i]) * scale_log2e;
+        if (edge) {
+            int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
+            sv = (key > pos || key < lo) ? -INFINITY : sv;
+        }
+        S[i] = sv;
+        mx = fmaxf(mx, sv);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float m_new = fmaxf(m, mx);
+    float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+    alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        S[i] = __builtin_amdgcn_exp2f(S[i] - m_safe);
+        sum += S[i];
+    }
+    sum += __shfl_xor(sum, 32, 64);
+    l = l * alpha + sum;
+    m = m_new;
+}
 
 // One wave: keys [t_begin, t_end) (t_begin a multiple of 32) against its 32 columns.
 // pos / lo: this lane's column may see keys lo..pos (pos < 0: nothing).
@@ -45,6 +88,8 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
                                              int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale) {
     int lane = threadIdx.x & 63;
     int r = lane & 31, h = lane >> 5;
+    float scale_log2e = scale * 1.44269504088896341f;
+    float alpha_out;
     int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
     for (int t0 = t_begin; t0 < t_end; t0 += 32) {
         int lp = t0 >> 4;
@@ -53,13 +98,15 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
         p0 = min(max(p0, 0), num_pages - 1);
         p1 = min(max(p1, 0), num_pages - 1);
         const bf16* kp = kc + (((size_t)(kk < 16 ? p0 : p1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8;
-        f32x16 S;
+        f32x16 S, S2;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+        for (int i = 0; i < 16; ++i) { S[i] = 0.0f; S2[i] = 0.0f; }
 #pragma unroll
-        for (int ks = 0; ks < HD / 16; ++ks) {
+        for (int ks = 0; ks < HD / 16; ks += 2) {      // two chains, so that an MFMA need not wait for the one before
             bf16x8 kf = *(const bf16x8*)(kp + ks * 16);
+            bf16x8 kf2 = *(const bf16x8*)(kp + (ks + 1) * 16);
             S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
+            S2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf2, qf[ks + 1], S2, 0, 0, 0);
         }
         // values of both pages: issued here so that their latency hides behind the softmax
         bf16x8 vf[HD / 32][2];
@@ -70,38 +117,21 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
             vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
         }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
-            float s = S[i] * scale;
-            s = (key > pos || key < lo) ? -INFINITY : s;
-            S[i] = s;
-            mx = fmaxf(mx, s);
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        float m_new = fmaxf(m, mx);
-        float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-        float alpha = expf(m - m_safe);
-        float sum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            S[i] = expf(S[i] - m_safe);
-            sum += S[i];
-        }
-        sum += __shfl_xor(sum, 32, 64);
-        l = l * alpha + sum;
-        m = m_new;
+        softmax_tile(S, S2, m, l, t0, pos, lo, h, scale_log2e, alpha_out);
+        float alpha = alpha_out;
         bf16x8 pf[2];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             pf[0][i] = (bf16)S[i];
             pf[1][i] = (bf16)S[8 + i];
         }
+        bool rescale = __any(alpha != 1.0f);     // the running maxima rarely move after the first tiles
 #pragma unroll
         for (int dt = 0; dt < HD / 32; ++dt) {
+            if (rescale) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+            }
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pf[0], O[dt], 0, 0, 0);
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pf[1], O[dt], 0, 0, 0);
         }
@@ -192,7 +222,8 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
     constexpr int STAGE_BYTES = 4 * PAGE_BYTES;     // K page 0, K page 1, V page 0, V page 1
     constexpr int LOADS = PAGE_BYTES / 1024;        // load instructions per wave per tile (4 pages over 4 waves)
     constexpr int SWZ_SHIFT = ROW_BYTES >= 256 ? 0 : 1;
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE_BYTES];
+    constexpr int STAGES = (4 * STAGE_BYTES <= 65536) ? 4 : 2;   // tiles in LDS: the loads run that far ahead
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int c = lane & 31, h = lane >> 5;
     int kvh = blockIdx.x % a.n_kv_heads;
@@ -235,6 +266,7 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
+    float scale_log2e = a.scale * 1.44269504088896341f;
 
     // Wave w brings page w of a tile's four (K0, K1, V0, V1) into LDS.
     auto issue = [&](int t0, int stage) {
@@ -260,64 +292,58 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
 
     int r = lane & 31;
     int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
-    issue(t_begin, 0);
-    wait_vmcnt_all();
-    __syncthreads();
+    // A trip to memory takes several times as long as a tile's products: STAGES - 1 tiles are
+    // kept on their way.  Loads complete in order, so "all but the last (STAGES-2) tiles' loads"
+    // is the next tile having landed.
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if (t_begin + 32 * p < t_end) issue(t_begin + 32 * p, p);
+    if (t_begin + 32 * (STAGES - 2) < t_end) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
+    __builtin_amdgcn_s_barrier();
     int stage = 0;
-    for (int t0 = t_begin; t0 < t_end; t0 += 32, stage ^= 1) {
-        if (t0 + 32 < t_end) issue(t0 + 32, stage ^ 1);
+    for (int t0 = t_begin; t0 < t_end; t0 += 32, stage = (stage + 1) % STAGES) {
+        if (t0 + 32 * (STAGES - 1) < t_end) issue(t0 + 32 * (STAGES - 1), (stage + STAGES - 1) % STAGES);
         if (t0 >= w_begin && t0 < w_end) {
             const unsigned char* kb = lds + stage * STAGE_BYTES + (kk >> 4) * PAGE_BYTES + (kk & 15) * ROW_BYTES;
             const unsigned char* vb = lds + stage * STAGE_BYTES + 2 * PAGE_BYTES + r * 32 + h * 16;
             int kswz = ((kk & 15) >> SWZ_SHIFT) & (CHUNKS - 1) & 15;
-            f32x16 S;
+            f32x16 S, S2;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+            for (int i = 0; i < 16; ++i) { S[i] = 0.0f; S2[i] = 0.0f; }
 #pragma unroll
-            for (int ks = 0; ks < HD / 16; ++ks) {
+            for (int ks = 0; ks < HD / 16; ks += 2) {
                 bf16x8 kf = *(const bf16x8*)(kb + (((ks * 2 + h) ^ kswz) * 16));
+                bf16x8 kf2 = *(const bf16x8*)(kb + ((((ks + 1) * 2 + h) ^ kswz) * 16));
                 S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
+                S2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf2, qf[ks + 1], S2, 0, 0, 0);
             }
-            float mx = -INFINITY;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
-                float sv = S[i] * a.scale;
-                sv = (key > pos || key < lo) ? -INFINITY : sv;
-                S[i] = sv;
-                mx = fmaxf(mx, sv);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            float m_new = fmaxf(m, mx);
-            float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-            float alpha = expf(m - m_safe);
-            float sum = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                S[i] = expf(S[i] - m_safe);
-                sum += S[i];
-            }
-            sum += __shfl_xor(sum, 32, 64);
-            l = l * alpha + sum;
-            m = m_new;
+            float alpha;
+            softmax_tile(S, S2, m, l, t0, pos, lo, h, scale_log2e, alpha);
             bf16x8 pf[2];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 pf[0][i] = (bf16)S[i];
                 pf[1][i] = (bf16)S[8 + i];
             }
+            bool rescale = __any(alpha != 1.0f);
 #pragma unroll
             for (int dt = 0; dt < HD / 32; ++dt) {
+                if (rescale) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                    for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                }
                 bf16x8 v0 = *(const bf16x8*)(vb + dt * 32 * 32);
                 bf16x8 v1 = *(const bf16x8*)(vb + PAGE_BYTES + dt * 32 * 32);
                 O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pf[0], O[dt], 0, 0, 0);
                 O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pf[1], O[dt], 0, 0, 0);
             }
         }
-        wait_vmcnt_all();      // the next tile has landed ...
-        __syncthreads();       // ... for everybody, and everybody is done with this one
+        // the next tile has landed (later ones may still be on their way) ...
+        if (t0 + 32 * (STAGES - 1) < t_end) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
+        // ... for everybody, and everybody is done with this one.  The bare barrier: __syncthreads()
+        // would also wait for the loads that are meant to stay in flight.  This wave's LDS reads of
+        // the tile have returned (their values went into the MFMAs above).
+        __builtin_amdgcn_s_barrier();
     }
     if (!cvalid) return;
     float inv = 1.0f / l;
@@ -398,7 +424,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
     M = wave_max(M);
     float L = 0.0f;
     for (int ch = lane; ch < n_chunks; ch += 64) {
-        float w = expf(pp[(size_t)ch * (hd + 2)] - M);
+        float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * (hd + 2)] - M);     // the maxima are base-2 logarithms
         weight[ch] = w;
         L += pp[(size_t)ch * (hd + 2) + 1] * w;
     }
