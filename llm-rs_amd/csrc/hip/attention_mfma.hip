@@ -43,38 +43,45 @@ __device__ __forceinline__ void wait_vmcnt_n() {
     __builtin_amdgcn_s_waitcnt((N_ & 15) | (7 << 4) | (15 << 8) | ((N_ >> 4) << 14));
 }
 
-// The softmax step of one 32-key tile for this lane's column.  S + S2 are the raw dots of the
-// lane's 16 keys; on return S holds their probabilities relative to the new running maximum
+// The maximum (or sum) of a value over a lane and its partner in the other half of the wave,
+// by the register swap of gfx950 (no trip through LDS).
+__device__ __forceinline__ float other_half(float x) {
+    unsigned u = __float_as_uint(x);
+    auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);   // {x of the low half, x of the high half} in every lane
+    return __uint_as_float((threadIdx.x & 32) ? sw[0] : sw[1]);
+}
+
+// The softmax step of one 32-key tile for this lane's column.  S holds the raw dots of the
+// lane's 16 keys; on return it holds their probabilities relative to the new running maximum
 // (not yet normalised), m and l are updated, alpha is what the older sums must be scaled by.
-// Scores are kept in the base-2 domain, (q.k) * scale * log2(e), so that the exponential is
-// one v_exp_f32; max, sums and scale factors are 32-bit as everywhere.  Keys outside
-// [lo, pos] are masked; the comparison is skipped for tiles that lie wholly inside every
-// column's range (all of a tile's lanes agree on that, so the branch is uniform).
-__device__ __forceinline__ void softmax_tile(f32x16& S, const f32x16& S2, float& m, float& l, int t0, int pos, int lo,
-                                             int h, float scale_log2e, float& alpha) {
-    bool edge = __any(t0 + 31 > pos || t0 < lo);
-    float mx = -INFINITY;
+// Scores are kept in the base-2 domain, (q.k) * c with c = scale * log2(e) > 0, so that the
+// exponential is one v_exp_f32 of one fused multiply-add; the maximum is taken over the raw dots
+// (c > 0 keeps the order).  Max, sums and scale factors are 32-bit as everywhere.  Keys outside
+// [lo, pos] are masked; that pass is skipped (edge false, the same in all lanes) for tiles that
+// lie wholly inside every column's range.
+__device__ __forceinline__ void softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
+                                             int h, float c, float& alpha, bool edge) {
+    if (edge) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        float sv = (S[i] + S2[i]) * scale_log2e;
-        if (edge) {
+        for (int i = 0; i < 16; ++i) {
             int key = t0 + 16 * (i >> 3) + 8 * h + 4 * ((i >> 2) & 1) + (i & 3);
-            sv = (key > pos || key < lo) ? -INFINITY : sv;
+            S[i] = (key > pos || key < lo) ? -INFINITY : S[i];
         }
-        S[i] = sv;
-        mx = fmaxf(mx, sv);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    float m_new = fmaxf(m, mx);
+    float mx = S[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[i]);
+    mx = fmaxf(mx, other_half(mx));
+    float m_new = fmaxf(m, mx * c);
     float m_safe = m_new == -INFINITY ? 0.0f : m_new;
     alpha = __builtin_amdgcn_exp2f(m - m_safe);
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-        S[i] = __builtin_amdgcn_exp2f(S[i] - m_safe);
+        S[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[i], c, -m_safe));
         sum += S[i];
     }
-    sum += __shfl_xor(sum, 32, 64);
+    sum += other_half(sum);
     l = l * alpha + sum;
     m = m_new;
 }
@@ -98,15 +105,13 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
         p0 = min(max(p0, 0), num_pages - 1);
         p1 = min(max(p1, 0), num_pages - 1);
         const bf16* kp = kc + (((size_t)(kk < 16 ? p0 : p1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8;
-        f32x16 S, S2;
+        f32x16 S;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { S[i] = 0.0f; S2[i] = 0.0f; }
+        for (int i = 0; i < 16; ++i) S[i] = 0.0f;
 #pragma unroll
-        for (int ks = 0; ks < HD / 16; ks += 2) {      // two chains, so that an MFMA need not wait for the one before
+        for (int ks = 0; ks < HD / 16; ++ks) {
             bf16x8 kf = *(const bf16x8*)(kp + ks * 16);
-            bf16x8 kf2 = *(const bf16x8*)(kp + (ks + 1) * 16);
             S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
-            S2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf2, qf[ks + 1], S2, 0, 0, 0);
         }
         // values of both pages: issued here so that their latency hides behind the softmax
         bf16x8 vf[HD / 32][2];
@@ -117,7 +122,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
             vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
         }
-        softmax_tile(S, S2, m, l, t0, pos, lo, h, scale_log2e, alpha_out);
+        softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo));
         float alpha = alpha_out;
         bf16x8 pf[2];
 #pragma unroll
@@ -125,13 +130,14 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             pf[0][i] = (bf16)S[i];
             pf[1][i] = (bf16)S[8 + i];
         }
-        bool rescale = __any(alpha != 1.0f);     // the running maxima rarely move after the first tiles
+        if (__any(alpha != 1.0f)) {              // the running maxima rarely move after the first tiles
 #pragma unroll
-        for (int dt = 0; dt < HD / 32; ++dt) {
-            if (rescale) {
+            for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
-            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < HD / 32; ++dt) {
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pf[0], O[dt], 0, 0, 0);
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pf[1], O[dt], 0, 0, 0);
         }
@@ -210,7 +216,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
 // read want one chunk of 16 different keys and then hit 16 different bank groups.  Values are
 // [HD][16] per page and are read in lane order; they need no swizzle.
 template <int HD>
-__global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attn_tiles_lds_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
                                                              const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                                              const int* __restrict__ block_table,
                                                              const int* __restrict__ positions,
@@ -224,10 +230,12 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
     constexpr int SWZ_SHIFT = ROW_BYTES >= 256 ? 0 : 1;
     constexpr int STAGES = (4 * STAGE_BYTES <= 65536) ? 4 : 2;   // tiles in LDS: the loads run that far ahead
     __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
-    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int lane = threadIdx.x & 63;
+    int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in all lanes: say so
     int c = lane & 31, h = lane >> 5;
     int kvh = blockIdx.x % a.n_kv_heads;
-    int btile = blockIdx.x / a.n_kv_heads;          // a block's tile: 4 * tpt tokens of one entry
+    // the longest tiles (the last of an entry) start first: they decide when the grid ends
+    int btile = (int)(gridDim.x / a.n_kv_heads) - 1 - (int)(blockIdx.x / a.n_kv_heads);   // 4 * tpt tokens of one entry
     int e = 0, rem = btile;
     for (; e < n_entries; ++e) {
         int cnt = q_starts[e + 1] - q_starts[e];
@@ -249,11 +257,16 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
     int head = kvh * G + hg;
     int pos = cvalid ? positions[token] : -1;
     int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    // An entry's positions rise by one from token to token, so the first and last token bound the rest.
     int b_first = positions[btok0], b_last = positions[btok_last];
     int t_end = b_last + 1;                                          // keys the block needs: [t_begin, t_end)
     int t_begin = ((a.window > 0 && b_first + 1 > a.window) ? b_first + 1 - a.window : 0) & ~31;
-    int w_end = wave_active ? positions[tok0 + ntok - 1] + 1 : 0;     // keys this wave needs end here
-    int w_begin = wave_active ? (((a.window > 0 && positions[tok0] + 1 > a.window) ? positions[tok0] + 1 - a.window : 0) & ~31) : 0;
+    int w_first = wave_active ? positions[tok0] : 0;                 // this wave's first and last position
+    int w_last = wave_active ? positions[tok0 + ntok - 1] : -1;
+    int w_end = w_last + 1;                                          // keys this wave needs: [w_begin, w_end)
+    int w_lo_first = (a.window > 0 && w_first + 1 > a.window) ? w_first + 1 - a.window : 0;
+    int w_lo_last = (a.window > 0 && w_last + 1 > a.window) ? w_last + 1 - a.window : 0;
+    int w_begin = w_lo_first & ~31;
     const int* table = block_table + (size_t)e * a.table_width;
 
     bf16x8 qf[HD / 16];
@@ -268,30 +281,50 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
     float m = -INFINITY, l = 0.0f;
     float scale_log2e = a.scale * 1.44269504088896341f;
 
-    // Wave w brings page w of a tile's four (K0, K1, V0, V1) into LDS.
+    // Wave w brings page w of a tile's four (K0, K1, V0, V1) into LDS.  What a lane fetches for
+    // its place in the page's LDS image does not change from tile to tile:
+    unsigned goff[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        int off = i * 1024 + lane * 16;
+        int krow = off / ROW_BYTES, slot = (off % ROW_BYTES) / 16;
+        int koff = krow * ROW_BYTES + ((slot ^ ((krow >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);   // keys: the chunk that belongs in this slot
+        goff[i] = wave < 2 ? koff : off;
+    }
+    const unsigned char* src_base = (const unsigned char*)((wave < 2 ? kc : vc) + (size_t)kvh * (16 * HD));
+    size_t page_stride = (size_t)a.n_kv_heads * (16 * HD) * sizeof(bf16);
+    // The request's page numbers for 64 logical pages at a time, one in each lane.
+    int pv_base = t_begin >> 4;
+    auto load_pages = [&](int first) {
+        int pg = table[min(first + lane, a.table_width - 1)];
+        return min(max(pg, 0), a.num_pages - 1);
+    };
+    int pv = load_pages(pv_base);
+    // Everything read from memory so far (the queries above all) is waited for here, once: a wait
+    // for it inside the loop would be a wait for all of the loop's own loads each time round.
+    wait_vmcnt_all();
     auto issue = [&](int t0, int stage) {
         int lp = t0 >> 4;
-        int p0 = table[min(lp, a.table_width - 1)];
-        int p1 = (t0 + 16 < t_end) ? table[min(lp + 1, a.table_width - 1)] : p0;
-        int page = (wave & 1) ? p1 : p0;
-        page = min(max(page, 0), a.num_pages - 1);
-        const unsigned char* src = (const unsigned char*)((wave < 2 ? kc : vc) + ((size_t)page * a.n_kv_heads + kvh) * (16 * HD));
-        unsigned base = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + wave * PAGE_BYTES);
+        if (lp - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
+        int idx = lp - pv_base + (((wave & 1) && t0 + 16 < t_end) ? 1 : 0);   // a tile's second page may lie past the end
+        int page = __builtin_amdgcn_readlane(pv, idx);
+        const unsigned char* src = src_base + (size_t)page * page_stride;
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            int off = i * 1024 + lane * 16;          // the lane's place in the page's LDS image
-            int goff = off;
-            if (wave < 2) {                          // keys: fetch the chunk that belongs in this slot
-                int kk = off / ROW_BYTES, slot = (off % ROW_BYTES) / 16;
-                goff = kk * ROW_BYTES + ((slot ^ ((kk >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);
-            }
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + goff),
-                                             (__attribute__((address_space(3))) void*)(lds + base + i * 1024), 16, 0, 0);
-        }
+        for (int i = 0; i < LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + goff[i]),
+                                             (__attribute__((address_space(3))) void*)(lds + stage * STAGE_BYTES + wave * PAGE_BYTES + i * 1024),
+                                             16, 0, 0);
     };
 
     int r = lane & 31;
     int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
+    int kswz = ((kk & 15) >> SWZ_SHIFT) & (CHUNKS - 1) & 15;
+    unsigned koffs[HD / 16];                                  // where this lane's K operands lie in a stage
+#pragma unroll
+    for (int ks = 0; ks < HD / 16; ++ks)
+        koffs[ks] = (kk >> 4) * PAGE_BYTES + (kk & 15) * ROW_BYTES + (((ks * 2 + h) ^ kswz) * 16);
+    unsigned voff = 2 * PAGE_BYTES + r * 32 + h * 16;
+
     // A trip to memory takes several times as long as a tile's products: STAGES - 1 tiles are
     // kept on their way.  Loads complete in order, so "all but the last (STAGES-2) tiles' loads"
     // is the next tile having landed.
@@ -300,50 +333,53 @@ __global__ __launch_bounds__(256) void attn_tiles_lds_kernel(const bf16* __restr
         if (t_begin + 32 * p < t_end) issue(t_begin + 32 * p, p);
     if (t_begin + 32 * (STAGES - 2) < t_end) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
     __builtin_amdgcn_s_barrier();
-    int stage = 0;
-    for (int t0 = t_begin; t0 < t_end; t0 += 32, stage = (stage + 1) % STAGES) {
-        if (t0 + 32 * (STAGES - 1) < t_end) issue(t0 + 32 * (STAGES - 1), (stage + STAGES - 1) % STAGES);
-        if (t0 >= w_begin && t0 < w_end) {
-            const unsigned char* kb = lds + stage * STAGE_BYTES + (kk >> 4) * PAGE_BYTES + (kk & 15) * ROW_BYTES;
-            const unsigned char* vb = lds + stage * STAGE_BYTES + 2 * PAGE_BYTES + r * 32 + h * 16;
-            int kswz = ((kk & 15) >> SWZ_SHIFT) & (CHUNKS - 1) & 15;
-            f32x16 S, S2;
+    for (int tb = t_begin; tb < t_end; tb += 32 * STAGES) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { S[i] = 0.0f; S2[i] = 0.0f; }
+        for (int stage = 0; stage < STAGES; ++stage) {       // unrolled: a stage's LDS addresses are immediates
+            int t0 = tb + 32 * stage;
+            if (t0 >= t_end) break;
+            bool more = t0 + 32 * (STAGES - 1) < t_end;
+            if (more) issue(t0 + 32 * (STAGES - 1), (stage + STAGES - 1) % STAGES);
+            if (t0 >= w_begin && t0 < w_end) {
+                const unsigned char* st = lds + stage * STAGE_BYTES;
+                bf16x8 kf[HD / 16];
 #pragma unroll
-            for (int ks = 0; ks < HD / 16; ks += 2) {
-                bf16x8 kf = *(const bf16x8*)(kb + (((ks * 2 + h) ^ kswz) * 16));
-                bf16x8 kf2 = *(const bf16x8*)(kb + ((((ks + 1) * 2 + h) ^ kswz) * 16));
-                S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
-                S2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf2, qf[ks + 1], S2, 0, 0, 0);
-            }
-            float alpha;
-            softmax_tile(S, S2, m, l, t0, pos, lo, h, scale_log2e, alpha);
-            bf16x8 pf[2];
+                for (int ks = 0; ks < HD / 16; ++ks) kf[ks] = *(const bf16x8*)(st + koffs[ks]);
+                f32x16 S;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                pf[0][i] = (bf16)S[i];
-                pf[1][i] = (bf16)S[8 + i];
-            }
-            bool rescale = __any(alpha != 1.0f);
+                for (int i = 0; i < 16; ++i) S[i] = 0.0f;
 #pragma unroll
-            for (int dt = 0; dt < HD / 32; ++dt) {
-                if (rescale) {
+                for (int ks = 0; ks < HD / 16; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], S, 0, 0, 0);
+                float alpha;
+                bool edge = t0 + 31 > w_first || t0 < w_lo_last;     // some column of the wave has a key of this tile masked
+                softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha, edge);
+                bf16x8 pf[2];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                for (int i = 0; i < 8; ++i) {
+                    pf[0][i] = (bf16)S[i];
+                    pf[1][i] = (bf16)S[8 + i];
                 }
-                bf16x8 v0 = *(const bf16x8*)(vb + dt * 32 * 32);
-                bf16x8 v1 = *(const bf16x8*)(vb + PAGE_BYTES + dt * 32 * 32);
-                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pf[0], O[dt], 0, 0, 0);
-                O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pf[1], O[dt], 0, 0, 0);
+                if (__any(alpha != 1.0f)) {
+#pragma unroll
+                    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+                }
+#pragma unroll
+                for (int dt = 0; dt < HD / 32; ++dt) {
+                    bf16x8 v0 = *(const bf16x8*)(st + voff + dt * 32 * 32);
+                    bf16x8 v1 = *(const bf16x8*)(st + voff + PAGE_BYTES + dt * 32 * 32);
+                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pf[0], O[dt], 0, 0, 0);
+                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pf[1], O[dt], 0, 0, 0);
+                }
             }
+            // the next tile has landed (later ones may still be on their way) ...
+            if (more) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
+            // ... for everybody, and everybody is done with this one.  The bare barrier: __syncthreads()
+            // would also wait for the loads that are meant to stay in flight.  This wave's LDS reads of
+            // the tile have returned (their values went into the MFMAs above).
+            __builtin_amdgcn_s_barrier();
         }
-        // the next tile has landed (later ones may still be on their way) ...
-        if (t0 + 32 * (STAGES - 1) < t_end) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
-        // ... for everybody, and everybody is done with this one.  The bare barrier: __syncthreads()
-        // would also wait for the loads that are meant to stay in flight.  This wave's LDS reads of
-        // the tile have returned (their values went into the MFMAs above).
-        __builtin_amdgcn_s_barrier();
     }
     if (!cvalid) return;
     float inv = 1.0f / l;
