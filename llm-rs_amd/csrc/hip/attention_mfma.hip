@@ -52,14 +52,21 @@ __device__ __forceinline__ float other_half(float x) {
 }
 
 // The softmax step of one 32-key tile for this lane's column.  S holds the raw dots of the
-// lane's 16 keys; on return it holds their probabilities relative to the new running maximum
+// lane's 16 keys; on return it holds their probabilities relative to the reference value m
 // (not yet normalised), m and l are updated, alpha is what the older sums must be scaled by.
 // Scores are kept in the base-2 domain, (q.k) * c with c = scale * log2(e) > 0, so that the
 // exponential is one v_exp_f32 of one fused multiply-add; the maximum is taken over the raw dots
-// (c > 0 keeps the order).  Max, sums and scale factors are 32-bit as everywhere.  Keys outside
-// [lo, pos] are masked; that pass is skipped (edge false, the same in all lanes) for tiles that
-// lie wholly inside every column's range.
-__device__ __forceinline__ void softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
+// (c > 0 keeps the order).  Max, sums and scale factors are 32-bit as everywhere.
+// m is a reference, not always the maximum: it follows the running maximum only when some
+// column of the wave has outgrown it by more than 8 (a factor 256, far from the range's end in
+// 32-bit sums and in the probabilities' bfloat16), which happens in the first tiles and then
+// hardly ever; all columns move together, so whether the older sums need scaling is one
+// answer for the wave (the return value; alpha is 1 everywhere otherwise).  The result is the
+// same softmax: every term and the sum carry the same factor 2^(max - m).
+// Keys outside [lo, pos] are masked; that pass is skipped (edge false, the same in all lanes)
+// for tiles that lie wholly inside every column's range.
+#define SOFTMAX_SLACK 8.0f
+__device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
                                              int h, float c, float& alpha, bool edge) {
     if (edge) {
 #pragma unroll
@@ -71,10 +78,15 @@ __device__ __forceinline__ void softmax_tile(f32x16& S, float& m, float& l, int 
     float mx = S[0];
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[i]);
-    mx = fmaxf(mx, other_half(mx));
-    float m_new = fmaxf(m, mx * c);
-    float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-    alpha = __builtin_amdgcn_exp2f(m - m_safe);
+    mx = fmaxf(mx, other_half(mx)) * c;
+    bool move = __any(mx > m + SOFTMAX_SLACK);        // (-inf + 8 is -inf: a column's first key always moves it)
+    alpha = 1.0f;
+    if (__builtin_expect(move, 0)) {
+        float m_new = fmaxf(m, mx);
+        alpha = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.0f : m_new));
+        m = m_new;
+    }
+    float m_safe = m == -INFINITY ? 0.0f : m;
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -83,7 +95,7 @@ __device__ __forceinline__ void softmax_tile(f32x16& S, float& m, float& l, int 
     }
     sum += other_half(sum);
     l = l * alpha + sum;
-    m = m_new;
+    return move;
 }
 
 // One wave: keys [t_begin, t_end) (t_begin a multiple of 32) against its 32 columns.
@@ -122,7 +134,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             vf[dt][0] = *(const bf16x8*)(vp0 + dt * 32 * 16);
             vf[dt][1] = *(const bf16x8*)(vp1 + dt * 32 * 16);
         }
-        softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo));
+        bool moved = softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha_out, __any(t0 + 31 > pos || t0 < lo));
         float alpha = alpha_out;
         bf16x8 pf[2];
 #pragma unroll
@@ -130,7 +142,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             pf[0][i] = (bf16)S[i];
             pf[1][i] = (bf16)S[8 + i];
         }
-        if (__any(alpha != 1.0f)) {              // the running maxima rarely move after the first tiles
+        if (moved) {                             // the reference rarely moves after the first tiles
 #pragma unroll
             for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
@@ -221,21 +233,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
                                                              const int* __restrict__ block_table,
                                                              const int* __restrict__ positions,
                                                              const int* __restrict__ q_starts, int n_entries,
-                                                             AttnArgs a, int G, int tpt, int skip_single) {
+                                                             AttnArgs a, int G, int tpt, int skip_single,
+                                                             int round_blocks) {
     constexpr int CHUNKS = HD / 8;                  // 16-byte chunks in a key's row
     constexpr int ROW_BYTES = HD * 2;
     constexpr int PAGE_BYTES = 16 * ROW_BYTES;      // a page of one kv head: keys [16][HD], values [HD][16]
-    constexpr int STAGE_BYTES = 4 * PAGE_BYTES;     // K page 0, K page 1, V page 0, V page 1
-    constexpr int LOADS = PAGE_BYTES / 1024;        // load instructions per wave per tile (4 pages over 4 waves)
+    constexpr int TILE_BYTES = 2 * PAGE_BYTES;      // a tile's keys, or its values: two pages
+    constexpr int HALF = PAGE_BYTES / 2048;         // load instructions of a wave for its half page
     constexpr int SWZ_SHIFT = ROW_BYTES >= 256 ? 0 : 1;
-    constexpr int STAGES = (4 * STAGE_BYTES <= 65536) ? 4 : 2;   // tiles in LDS: the loads run that far ahead
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[STAGES * STAGE_BYTES];
+    constexpr int R = (8 * TILE_BYTES <= 65536) ? 4 : 2;   // tiles in each of the two rings (keys, values)
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * R * TILE_BYTES];
     int lane = threadIdx.x & 63;
     int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // the same in all lanes: say so
     int c = lane & 31, h = lane >> 5;
     int kvh = blockIdx.x % a.n_kv_heads;
-    // the longest tiles (the last of an entry) start first: they decide when the grid ends
-    int btile = (int)(gridDim.x / a.n_kv_heads) - 1 - (int)(blockIdx.x / a.n_kv_heads);   // 4 * tpt tokens of one entry
+    // Order of work.  A tile's work grows with its place in its entry, so the tiles are handed out
+    // from the last to the first: the longest start first, they decide when the grid ends.  All
+    // blocks of the first two rounds (a round: as many blocks as the device holds at once in one
+    // layer, `round_blocks`) are resident together, the second round beside the first on the same
+    // units, so the second round runs in the opposite order and puts the shortest beside the longest.
+    int n_btiles = 0;
+    for (int i = 0; i < n_entries; ++i) {
+        int cnt = q_starts[i + 1] - q_starts[i];
+        n_btiles += (cnt == 1 && skip_single) ? 0 : (cnt + 4 * tpt - 1) / (4 * tpt);
+    }
+    int g = blockIdx.x / a.n_kv_heads;
+    if (g >= n_btiles) return;                       // the grid is sized for the most tiles the tokens could make
+    int gr = round_blocks / a.n_kv_heads;
+    if (g >= gr && g < 2 * gr) g = gr + (min(2 * gr, n_btiles) - 1 - g);
+    int btile = n_btiles - 1 - g;                    // 4 * tpt tokens of one entry
     int e = 0, rem = btile;
     for (; e < n_entries; ++e) {
         int cnt = q_starts[e + 1] - q_starts[e];
@@ -263,10 +289,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     int t_begin = ((a.window > 0 && b_first + 1 > a.window) ? b_first + 1 - a.window : 0) & ~31;
     int w_first = wave_active ? positions[tok0] : 0;                 // this wave's first and last position
     int w_last = wave_active ? positions[tok0 + ntok - 1] : -1;
-    int w_end = w_last + 1;                                          // keys this wave needs: [w_begin, w_end)
-    int w_lo_first = (a.window > 0 && w_first + 1 > a.window) ? w_first + 1 - a.window : 0;
     int w_lo_last = (a.window > 0 && w_last + 1 > a.window) ? w_last + 1 - a.window : 0;
-    int w_begin = w_lo_first & ~31;
     const int* table = block_table + (size_t)e * a.table_width;
 
     bf16x8 qf[HD / 16];
@@ -281,20 +304,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     float m = -INFINITY, l = 0.0f;
     float scale_log2e = a.scale * 1.44269504088896341f;
 
-    // Wave w brings page w of a tile's four (K0, K1, V0, V1) into LDS.  What a lane fetches for
-    // its place in the page's LDS image does not change from tile to tile:
-    unsigned goff[LOADS];
+    // ---- loads.  A tile's keys are two pages and so are its values; each wave brings half a page
+    // of both (page wave & 1, half wave >> 1).  What a lane fetches for its place in the page's
+    // LDS image does not change from tile to tile:
+    unsigned goff_k[HALF], goff_v[HALF];
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        int off = i * 1024 + lane * 16;
+    for (int i = 0; i < HALF; ++i) {
+        int off = (wave >> 1) * (PAGE_BYTES / 2) + i * 1024 + lane * 16;
         int krow = off / ROW_BYTES, slot = (off % ROW_BYTES) / 16;
-        int koff = krow * ROW_BYTES + ((slot ^ ((krow >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);   // keys: the chunk that belongs in this slot
-        goff[i] = wave < 2 ? koff : off;
+        goff_k[i] = krow * ROW_BYTES + ((slot ^ ((krow >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);   // keys: the chunk that belongs in this slot
+        goff_v[i] = off;
     }
-    const unsigned char* src_base = (const unsigned char*)((wave < 2 ? kc : vc) + (size_t)kvh * (16 * HD));
+    unsigned lds_part = (wave & 1) * PAGE_BYTES + (wave >> 1) * (PAGE_BYTES / 2);   // this wave's part of a tile's image
+    const unsigned char* k_base = (const unsigned char*)(kc + (size_t)kvh * (16 * HD));
+    const unsigned char* v_base = (const unsigned char*)(vc + (size_t)kvh * (16 * HD));
     size_t page_stride = (size_t)a.n_kv_heads * (16 * HD) * sizeof(bf16);
+    int n = (t_end - t_begin + 31) >> 5;             // tiles of the block, numbered from 0
+    int lp0 = t_begin >> 4;                          // the first tile's first logical page
     // The request's page numbers for 64 logical pages at a time, one in each lane.
-    int pv_base = t_begin >> 4;
+    int pv_base = lp0;
     auto load_pages = [&](int first) {
         int pg = table[min(first + lane, a.table_width - 1)];
         return min(max(pg, 0), a.num_pages - 1);
@@ -303,84 +331,137 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     // Everything read from memory so far (the queries above all) is waited for here, once: a wait
     // for it inside the loop would be a wait for all of the loop's own loads each time round.
     wait_vmcnt_all();
-    auto issue = [&](int t0, int stage) {
-        int lp = t0 >> 4;
-        if (lp - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
-        int idx = lp - pv_base + (((wave & 1) && t0 + 16 < t_end) ? 1 : 0);   // a tile's second page may lie past the end
-        int page = __builtin_amdgcn_readlane(pv, idx);
-        const unsigned char* src = src_base + (size_t)page * page_stride;
+    auto page_of = [&](int tile) {                   // the page this wave loads from, for a tile in [0, n)
+        int lp = lp0 + 2 * tile;
+        // a tile's second page may lie past the request's last key: then it is not looked up
+        int idx = lp - pv_base + (((wave & 1) && t_begin + 32 * tile + 16 < t_end) ? 1 : 0);
+        return (size_t)__builtin_amdgcn_readlane(pv, idx) * page_stride;
+    };
+    auto load_part = [&](const unsigned char* src, const unsigned (&goff)[HALF], int lds_off) {
 #pragma unroll
-        for (int i = 0; i < LOADS; ++i)
+        for (int i = 0; i < HALF; ++i)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + goff[i]),
-                                             (__attribute__((address_space(3))) void*)(lds + stage * STAGE_BYTES + wave * PAGE_BYTES + i * 1024),
+                                             (__attribute__((address_space(3))) void*)(lds + lds_off + lds_part + i * 1024),
                                              16, 0, 0);
     };
+    // What iteration t starts on their way: keys of tile t + R (into the slot whose tile, t, went
+    // into the products of iteration t - 1), values of tile t + R - 1 (tile t - 1 was used in
+    // iteration t - 1).  `t mod R` is passed apart, as a constant.  Every iteration starts the
+    // same number of loads: where the tile would lie outside [0, n) the nearest real one is
+    // loaded once more, into a slot that nobody reads; that costs less than telling the cases apart.
+    auto issue = [&](int t, int t_mod) {
+        int tk = min(t + R, n - 1), tv = min(max(t + R - 1, 0), n - 1);
+        if (__builtin_expect(lp0 + 2 * tk + 1 - pv_base >= 64, 0)) {      // tv <= tk: its pages stay in the window
+            pv_base = lp0 + 2 * tv;
+            pv = load_pages(pv_base);
+        }
+        load_part(k_base + page_of(tk), goff_k, ((t_mod + R) % R) * TILE_BYTES);
+        load_part(v_base + page_of(tv), goff_v, (R + (t_mod + R - 1) % R) * TILE_BYTES);
+    };
+    // At the end of iteration t the keys of tile t + 2 and the values of tile t + 1 must have
+    // landed: all that iteration t + 2 - R and those before it started.  Loads complete in order,
+    // so the wave may leave behind what it has started since then.
+    auto wait_landed = [&]() { wait_vmcnt_n<2 * (R - 2) * HALF>(); };
+    // All waves are done with what they read from LDS (the reads have returned), and what each
+    // waited for above is there for everybody.  A bare s_barrier: __syncthreads() would also wait
+    // for the loads that are meant to stay in flight.
+    auto block_sync = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
     int r = lane & 31;
     int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
     int kswz = ((kk & 15) >> SWZ_SHIFT) & (CHUNKS - 1) & 15;
-    unsigned koffs[HD / 16];                                  // where this lane's K operands lie in a stage
+    unsigned koffs[HD / 16];                                  // where this lane's K operands lie in a tile's image
 #pragma unroll
     for (int ks = 0; ks < HD / 16; ++ks)
         koffs[ks] = (kk >> 4) * PAGE_BYTES + (kk & 15) * ROW_BYTES + (((ks * 2 + h) ^ kswz) * 16);
-    unsigned voff = 2 * PAGE_BYTES + r * 32 + h * 16;
+    unsigned voff = r * 32 + h * 16;
 
-    // A trip to memory takes several times as long as a tile's products: STAGES - 1 tiles are
-    // kept on their way.  Loads complete in order, so "all but the last (STAGES-2) tiles' loads"
-    // is the next tile having landed.
+    // S^T of a tile from the keys in ring slot `slot`
+    auto scores = [&](int slot) {
+        const unsigned char* st = lds + slot * TILE_BYTES;
+        bf16x8 kf[HD / 16];
 #pragma unroll
-    for (int p = 0; p < STAGES - 1; ++p)
-        if (t_begin + 32 * p < t_end) issue(t_begin + 32 * p, p);
-    if (t_begin + 32 * (STAGES - 2) < t_end) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
-    __builtin_amdgcn_s_barrier();
-    for (int tb = t_begin; tb < t_end; tb += 32 * STAGES) {
+        for (int ks = 0; ks < HD / 16; ++ks) kf[ks] = *(const bf16x8*)(st + koffs[ks]);
+        f32x16 S;
 #pragma unroll
-        for (int stage = 0; stage < STAGES; ++stage) {       // unrolled: a stage's LDS addresses are immediates
-            int t0 = tb + 32 * stage;
-            if (t0 >= t_end) break;
-            bool more = t0 + 32 * (STAGES - 1) < t_end;
-            if (more) issue(t0 + 32 * (STAGES - 1), (stage + STAGES - 1) % STAGES);
-            if (t0 >= w_begin && t0 < w_end) {
-                const unsigned char* st = lds + stage * STAGE_BYTES;
-                bf16x8 kf[HD / 16];
+        for (int i = 0; i < 16; ++i) S[i] = 0.0f;
 #pragma unroll
-                for (int ks = 0; ks < HD / 16; ++ks) kf[ks] = *(const bf16x8*)(st + koffs[ks]);
-                f32x16 S;
+        for (int ks = 0; ks < HD / 16; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], S, 0, 0, 0);
+        return S;
+    };
+    // The values in ring slot `slot` as operands, and O^T += V^T P^T with them.  The two are
+    // apart so that the reads can be started before the softmax arithmetic and return behind it.
+    constexpr int VF = HD / 32 * 2;
+    auto read_values = [&](int slot, bf16x8 (&vf)[VF]) {
+        const unsigned char* st = lds + (R + slot) * TILE_BYTES + voff;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+        for (int dt = 0; dt < HD / 32; ++dt) {
+            vf[2 * dt] = *(const bf16x8*)(st + dt * 32 * 32);
+            vf[2 * dt + 1] = *(const bf16x8*)(st + PAGE_BYTES + dt * 32 * 32);
+        }
+    };
+    auto accumulate = [&](const bf16x8 (&vf)[VF], const bf16x8 (&pf)[2]) {
 #pragma unroll
-                for (int ks = 0; ks < HD / 16; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], S, 0, 0, 0);
-                float alpha;
-                bool edge = t0 + 31 > w_first || t0 < w_lo_last;     // some column of the wave has a key of this tile masked
-                softmax_tile(S, m, l, t0, pos, lo, h, scale_log2e, alpha, edge);
-                bf16x8 pf[2];
+        for (int dt = 0; dt < HD / 32; ++dt) {
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[2 * dt], pf[0], O[dt], 0, 0, 0);
+            O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[2 * dt + 1], pf[1], O[dt], 0, 0, 0);
+        }
+    };
+    auto rescale = [&](bool moved, float alpha) {
+        if (__builtin_expect(moved, 0)) {             // the reference rarely moves after the first tiles
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    pf[0][i] = (bf16)S[i];
-                    pf[1][i] = (bf16)S[8 + i];
-                }
-                if (__any(alpha != 1.0f)) {
+            for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
-                    for (int dt = 0; dt < HD / 32; ++dt)
+                for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
+        }
+    };
+    // some column of the wave has a key of tile t masked (tiles beyond a wave's own keys are
+    // masked as a whole: every wave walks all of the block's tiles)
+    auto is_edge = [&](int t) { int t0 = t_begin + 32 * t; return t0 + 31 > w_first || t0 < w_lo_last; };
+    auto to_bf16 = [&](const f32x16& S, bf16x8 (&pf)[2]) {
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) O[dt][i] *= alpha;
-                }
+        for (int i = 0; i < 8; ++i) {
+            pf[0][i] = (bf16)S[i];
+            pf[1][i] = (bf16)S[8 + i];
+        }
+    };
+
+    // The score products of a tile and the softmax arithmetic of the tile before do not depend on
+    // each other, so the loop is skewed: iteration t starts the scores of tile t + 1 (matrix
+    // cores) beside the softmax of tile t (vector unit), then adds tile t's values.
 #pragma unroll
-                for (int dt = 0; dt < HD / 32; ++dt) {
-                    bf16x8 v0 = *(const bf16x8*)(st + voff + dt * 32 * 32);
-                    bf16x8 v1 = *(const bf16x8*)(st + voff + PAGE_BYTES + dt * 32 * 32);
-                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v0, pf[0], O[dt], 0, 0, 0);
-                    O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(v1, pf[1], O[dt], 0, 0, 0);
-                }
+    for (int j = 0; j < R; ++j) issue(j - R, j);                    // keys 0 .. R-1, values 0 .. R-2
+    wait_landed();                                                   // keys of tiles 0 and 1, values of tile 0
+    block_sync();
+    f32x16 S_next = scores(0);
+    block_sync();                                                    // tile 0's keys may be overwritten
+    for (int tb = 0; tb < n; tb += R) {
+#pragma unroll
+        for (int s = 0; s < R; ++s) {                 // unrolled: the ring slots are constants, LDS addresses immediates
+            int t = tb + s;                           // t mod R == s
+            if (t >= n) break;
+            issue(t, s);
+            f32x16 S_cur = S_next;
+            float alpha;
+            bf16x8 pf[2], vf[VF];
+            bool moved;
+            if (is_edge(t)) {
+                S_next = scores((s + 1) % R);         // (nothing real for the last tile: not used then)
+                read_values(s, vf);
+                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, true);
+            } else {
+                S_next = scores((s + 1) % R);
+                read_values(s, vf);
+                moved = softmax_tile(S_cur, m, l, t_begin + 32 * t, pos, lo, h, scale_log2e, alpha, false);
             }
-            // the next tile has landed (later ones may still be on their way) ...
-            if (more) wait_vmcnt_n<(STAGES - 2) * LOADS>(); else wait_vmcnt_all();
-            // ... for everybody, and everybody is done with this one.  The bare barrier: __syncthreads()
-            // would also wait for the loads that are meant to stay in flight.  This wave's LDS reads of
-            // the tile have returned (their values went into the MFMAs above).
-            __builtin_amdgcn_s_barrier();
+            to_bf16(S_cur, pf);
+            rescale(moved, alpha);
+            accumulate(vf, pf);
+            wait_landed();
+            block_sync();
         }
     }
+
     if (!cvalid) return;
     float inv = 1.0f / l;
     bf16* op = out + (size_t)token * a.out_stride + (size_t)head * HD;
@@ -474,6 +555,17 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
     }
 }
 
+// Compute units of the current device (asked once).
+static int compute_units() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+    }
+    return n;
+}
+
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
                   const int* positions, const int* q_starts, int n_entries, float* scratch, size_t scratch_bytes,
@@ -489,7 +581,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
         if constexpr (HD == 64 || HD == 128 || HD == 256) {
             int btiles = a.n_tokens / (4 * tpt) + n_entries;
             attn_tiles_lds_kernel<HD><<<btiles * a.n_kv_heads, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
-                                                                                 n_entries, a, G, tpt, split);
+                                                                                 n_entries, a, G, tpt, split, compute_units());
         } else {
             int tiles = a.n_tokens / tpt + n_entries;
             int blocks = ((tiles + 3) / 4) * a.n_kv_heads;
