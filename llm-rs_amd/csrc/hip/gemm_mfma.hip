@@ -64,7 +64,7 @@ template <int MT, int NT, int NW, int U>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
                                                               int ldc, int M, int N, int K, int epi,
-                                                              float* __restrict__ partial, QkvEpilogue qe) {
+                                                              float* __restrict__ partial, QkvEpilogue qe, int rot_feats) {
     extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
     float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -85,14 +85,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     int full = K / 64;             // blocks of 64 k that need no bounds
     int nkb = (K + 63) / 64;
     int per = (nkb + gridDim.y - 1) / gridDim.y;
-    int kb_hi = min(nkb, (int)(blockIdx.y + 1) * per);     // this block's k-blocks: [blockIdx.y * per, kb_hi)
-    int full_hi = min(full, kb_hi);
-    int kb = blockIdx.y * per + wave;
-    for (; kb + (U - 1) * NW < full_hi; kb += U * NW) {
+    int lo = blockIdx.y * per;
+    int kb_hi = min(nkb, lo + per);                        // this block's k-blocks: [lo, kb_hi)
+    int cnt = max(min(full, kb_hi) - lo, 0);               // the full ones among them
+    // The block walks its full k-blocks starting at `rot` and wraps round: with rot_feats > 0,
+    // neighbouring groups of rot_feats features are at different places of their rows at any
+    // moment.  Rows are a multiple of the memory channels' interleave apart, so blocks in step
+    // would all ask the same few channels at once.  The start depends on the features alone
+    // (a block's features lie within one group), not on how many of them a block takes.
+    int rot = (cnt > 0 && rot_feats > 0) ? (n0 / rot_feats) % cnt : 0;
+    auto turn = [&](int j) { int x = j + rot; return lo + (x >= cnt ? x - cnt : x); };
+    int j = wave;
+    for (; j + (U - 1) * NW < cnt; j += U * NW) {
         bf16x8 w[U][NT][2], x[U][MT][2];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            int k = (kb + u * NW) * 64 + g * 8;
+            int k = turn(j + u * NW) * 64 + g * 8;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) { w[u][nt][0] = load8(wp[nt] + k); w[u][nt][1] = load8(wp[nt] + k + 32); }
 #pragma unroll
@@ -109,8 +117,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                     acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][nt][1], x[u][mt][1], acc[mt][nt], 0, 0, 0);
                 }
     }
-    for (; kb < kb_hi; kb += NW) {   // what is left of this wave's turns, and the partial block if it is its turn
-        int k = kb * 64 + g * 8;
+    // what is left of this wave's turns, then the partial block if it is the wave's turn
+    for (;; j += NW) {
+        bool partial_turn = j == cnt && kb_hi > lo + cnt;   // one k-block past the full ones, cut by K
+        if (j >= cnt && !partial_turn) break;
+        int k = (partial_turn ? lo + cnt : turn(j)) * 64 + g * 8;
         bool v0 = k < K, v1 = k + 32 < K;
         bf16x8 w0[NT], w1[NT];
 #pragma unroll
@@ -127,6 +138,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                 acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[nt], x1, acc[mt][nt], 0, 0, 0);
             }
         }
+        if (partial_turn) break;
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -228,7 +240,7 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
 template <int MT, int NT, int NW, int U>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                           int M, int N, int K, int epi, const QkvEpilogue* qkv, int splits = 1,
-                          float* partial = nullptr) {
+                          float* partial = nullptr, int rot_feats = 0) {
     size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
     static bool configured = false;
     if (!configured) {
@@ -239,7 +251,7 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
     dim3 grid(ceil_div(N, NT * 16), splits);
     gemm_skinny_kernel<MT, NT, NW, U><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                           splits > 1 ? partial : nullptr,
-                                                                          qkv ? *qkv : QkvEpilogue{});
+                                                                          qkv ? *qkv : QkvEpilogue{}, rot_feats);
     if (splits > 1) {
         size_t pairs = (size_t)M * ((N + 1) / 2);
         gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
@@ -520,6 +532,17 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
     return 0;
 }
 
+// Compute units of the current device (asked once).
+static int compute_unit_count() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+    }
+    return n;
+}
+
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
                          const QkvEpilogue* qkv) {
@@ -540,13 +563,20 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // (Measured on MI355X at the 8B shapes; see profiles/.)
         bool wide = N >= 16384;
         bool eight = !wide && K >= 2048;
-#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv)
+        // A wide weight's blocks take 7 or 4 feature tiles: whichever number of blocks fills the
+        // device's compute units more evenly (28672 features are 256 blocks of 7 tiles).  Its blocks
+        // start their walk along k at staggered places, by groups of that many features.
+        int cus = compute_unit_count();
+        auto evenness = [&](int nt) { int b = ceil_div(N, 16 * nt); return (double)b / ((double)ceil_div(b, cus) * cus); };
+        int wide_nt = (wide && evenness(7) >= evenness(4)) ? 7 : 4;
+        int rot = wide ? 16 * wide_nt : 0;
+#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot)
         if (M <= 16) {
-            if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else SKINNY(1, 4, 4, 2); }
+            if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else if (wide_nt == 7) SKINNY(1, 7, 4, 1); else SKINNY(1, 4, 4, 2); }
             else if (eight) SKINNY(1, 1, 8, 4);
             else SKINNY(1, 1, 4, 4);
         } else if (M <= 32) {
-            if (wide) SKINNY(2, 4, 4, 2);
+            if (wide) { if (wide_nt == 7) SKINNY(2, 7, 4, 1); else SKINNY(2, 4, 4, 2); }
             else if (N > 4096) { if (eight) SKINNY(2, 2, 8, 2); else SKINNY(2, 2, 4, 2); }
             else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {
@@ -559,7 +589,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
                 launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
-            } else if (wide) SKINNY(4, 4, 4, 2);
+            } else if (wide) { if (wide_nt == 7) SKINNY(4, 7, 4, 1); else SKINNY(4, 4, 4, 2); }
             else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
             else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
         }
