@@ -556,7 +556,8 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
     if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
         // waves in turn and their sums are added in wave order, so for a given weight an
-        // output's sum has one order whatever M, MT, NT and U are.
+        // output's sum has one order whatever M, MT, NT and U are (up to 32 rows; with more, a
+        // weight with few rows may have its k-blocks shared out over blocks as well).
         // Features per block (NT*16) grow with N and M: a block reads its tokens' rows
         // again for every 16*NT features, which costs L2 bandwidth once M is large, but
         // a weight with few rows needs small blocks to have enough of them.

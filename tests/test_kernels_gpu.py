@@ -55,7 +55,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20),
                (64, 200, 2048), (40, 1000, 1096), (64, 4096, 4096), (24, 520, 2048), (50, 64, 8200),
                (8, 38, 100), (3, 130, 4099), (1, 6, 20),
-               (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128)]
+               (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128),
+               # many features: blocks of several feature tiles that start their walk along k at staggered places
+               (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -103,6 +105,25 @@ def test_gemm_rows_do_not_depend_on_batch(dtype):
         kernels().gemm(sub, w, out, EPI_STORE_F32)
         outs.append(out[rows.index(7)].cpu())
     assert (outs[0] - outs[1]).abs().max() <= 2e-5 and (outs[0] - outs[2]).abs().max() <= 2e-5
+
+
+@pytest.mark.parametrize("N,K", [(200, 320), (1000, 4096), (16500, 328), (28672, 256)])
+def test_gemm_small_batches_sum_in_one_order(N, K):
+    """Up to 32 rows the matrix-core kernels add a feature's k-blocks in an order that the
+    weight's shape fixes: a row's result is the same bits alone, among 8, 20 or 32 rows.
+    (With more rows a weight with few features has its k-blocks shared out over several
+    blocks, and from 65 rows on the tiles are others: equal to rounding only.)"""
+    a = rnd((32, K), torch.bfloat16, 16)
+    w = rnd((N, K), torch.bfloat16, 17, 0.1)
+    outs = []
+    for rows in ([7], list(range(4, 12)), list(range(20)), list(range(32))):
+        sub = a[rows].contiguous()
+        out = torch.zeros((len(rows), N), dtype=torch.float32, device=DEV)
+        ws = torch.empty(max(1, kernels().gemm_workspace_floats(len(rows), N, K)), dtype=torch.float32, device=DEV)
+        kernels().gemm(sub, w, out, EPI_STORE_F32, ws)
+        outs.append(out[rows.index(7)].cpu())
+    for o in outs[1:]:
+        assert torch.equal(outs[0], o)
 
 
 def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, scaling=None):
