@@ -603,9 +603,24 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // with 128 x 64 per wave (eight waves on a 256 x 256 tile) there is one LDS read per MFMA less
         // than with 64 x 64 (four waves on 128 x 128), and the loop is bound by LDS bandwidth; it pays
         // as soon as the larger tiles still fill most of the device (measured on MI355X)
-        long big_tiles = (long)ceil_div(M, 256) * ceil_div(N, 256);
-        if (K % 64 == 0 && big_tiles >= 160) rc = launch_dma<256, 256, 2, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
-        else if (K % 64 == 0) rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        // One large tile runs on a compute unit at a time, so a grid of them works in rounds and the
+        // last round may be far from full (896 tiles on 256 units: 3.5 rounds cost 4).  Then the large
+        // tiles get the features that make whole rounds and the small tiles, two to a unit, the rest.
+        long m_tiles = ceil_div(M, 256), big_tiles = m_tiles * ceil_div(N, 256);
+        int cus = compute_unit_count();
+        if (K % 64 == 0 && big_tiles >= 160) {
+            long whole = big_tiles / cus * cus, rest = big_tiles - whole;
+            int n_split = (int)(whole / m_tiles) * 256;        // features of the whole rounds
+            if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4) {
+                size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
+                void* out_rest = (char*)out + (size_t)(epi == LLMRS_EPI_SWIGLU ? n_split / 2 : n_split) * elt;
+                rc = launch_dma<256, 256, 2, 4, 2>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
+                if (rc == 0)
+                    rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
+            } else {
+                rc = launch_dma<256, 256, 2, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+            }
+        } else if (K % 64 == 0) rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
         else rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
     if (rc != 0) return -1;

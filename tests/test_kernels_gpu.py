@@ -57,7 +57,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (8, 38, 100), (3, 130, 4099), (1, 6, 20),
                (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128),
                # many features: blocks of several feature tiles that start their walk along k at staggered places
-               (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192)]
+               (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192),
+               # more large tiles than compute units, the last round not full: the features are split between two tile sizes
+               (513, 25600, 64)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
