@@ -497,6 +497,35 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
         __syncthreads();
     }
 
+    if (epi == LLMRS_EPI_ACCUM_F32) {
+        // out += acc: a row block's old values are all asked for before the first sum is stored
+        // (left to itself the compiler waits for each load before the store that follows it,
+        // a trip to memory per value).
+        float* o = (float*)out;
+        static_for<0, FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            float old[FN][16];
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                int n = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    old[j][r] = o[(size_t)min(m, M - 1) * ldc + min(n, N - 1)];
+                }
+            }
+            static_for<0, FN>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                int n = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < M && n < N) o[(size_t)m * ldc + n] = old[j][r] + acc[i][j][r];
+                }
+            });
+        });
+        return;
+    }
     static_for<0, FM * FN>([&](auto idx) {
         constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
         int n = n0 + wn * TN + j * 32 + (lane & 31);
