@@ -60,9 +60,11 @@ __device__ __forceinline__ float other_half(float x) {
 // m is a reference, not always the maximum: it follows the running maximum only when some
 // column of the wave has outgrown it by more than 8 (a factor 256, far from the range's end in
 // 32-bit sums and in the probabilities' bfloat16), which happens in the first tiles and then
-// hardly ever; all columns move together, so whether the older sums need scaling is one
-// answer for the wave (the return value; alpha is 1 everywhere otherwise).  The result is the
-// same softmax: every term and the sum carry the same factor 2^(max - m).
+// hardly ever.  Each column moves by its own rule, so its result does not depend on which
+// other columns share its wave; whether any column moved is one answer for the wave (the
+// return value: only then the older sums need scaling, by alpha, which is 1 in the columns
+// that stayed).  The result is the same softmax: every term and the sum carry the same
+// factor 2^(max - m).
 // Keys outside [lo, pos] are masked; that pass is skipped (edge false, the same in all lanes)
 // for tiles that lie wholly inside every column's range.
 #define SOFTMAX_SLACK 8.0f
@@ -79,10 +81,11 @@ __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int 
 #pragma unroll
     for (int i = 1; i < 16; ++i) mx = fmaxf(mx, S[i]);
     mx = fmaxf(mx, other_half(mx)) * c;
-    bool move = __any(mx > m + SOFTMAX_SLACK);        // (-inf + 8 is -inf: a column's first key always moves it)
+    bool mine = mx > m + SOFTMAX_SLACK;               // (-inf + 8 is -inf: a column's first key always moves it)
+    bool move = __any(mine);
     alpha = 1.0f;
     if (__builtin_expect(move, 0)) {
-        float m_new = fmaxf(m, mx);
+        float m_new = mine ? mx : m;                  // each column by its own rule: nothing depends on its neighbours
         alpha = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.0f : m_new));
         m = m_new;
     }
