@@ -413,7 +413,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 template <int BM, int BN, int WGM, int WGN, int STAGES>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __restrict__ A, int lda,
                                                        const bf16* __restrict__ W, void* __restrict__ out,
-                                                       int ldc, int M, int N, int K, int epi) {
+                                                       int ldc, int M, int N, int K, int epi,
+                                                       float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char dma_smem[];
     constexpr int WAVES = WGM * WGN;                              // waves of a block, as a WGM x WGN grid over the tile
     constexpr int TM = BM / WGM, TN = BN / WGN, FM = TM / 32, FN = TN / 32;
@@ -439,7 +440,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
         int row = (wave * W_GROUPS + i) * 8 + lrow;
         gw[i] = W + (size_t)min(n0 + row, N - 1) * K + ((lslot ^ ((row >> 1) & 7)) * 8);
     }
+    // With gridDim.z > 1 the k-tiles are shared out over that many blocks (contiguous ranges): each
+    // writes its 32-bit sums to `partial` [gridDim.z][M][N] and gemm_splitk_finish_kernel adds them
+    // in order and applies the epilogue.  That is for products with too few tiles to fill the device.
+    int nk_all = K / 64, per_split = (nk_all + gridDim.z - 1) / gridDim.z;
+    int kt_lo = blockIdx.z * per_split;
+    int nk = max(0, min(nk_all, kt_lo + per_split) - kt_lo);       // this block's k-tiles: [kt_lo, kt_lo + nk)
     auto issue = [&](int kt, int stage) {
+        kt += kt_lo;
         unsigned base = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + wave * A_GROUPS * 1024);
 #pragma unroll
         for (int i = 0; i < A_GROUPS; ++i)
@@ -460,7 +468,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    int nk = K / 64;
 #pragma unroll
     for (int p = 0; p < STAGES - 1; ++p)
         if (p < nk) issue(p, p);
@@ -497,6 +504,19 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
         __syncthreads();
     }
 
+    if (partial != nullptr) {       // one part of the sum: as it is, for the kernel that adds the parts
+        float* part = partial + (size_t)blockIdx.z * M * N;
+        static_for<0, FM * FN>([&](auto idx) {
+            constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
+            int n = n0 + wn * TN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M && n < N) part[(size_t)m * N + n] = acc[i][j][r];
+            }
+        });
+        return;
+    }
     if (epi == LLMRS_EPI_ACCUM_F32) {
         // out += acc: a row block's old values are all asked for before the first sum is stored
         // (left to itself the compiler waits for each load before the store that follows it,
@@ -546,7 +566,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
 
 template <int BM, int BN, int WGM, int WGN, int STAGES>
 static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                      int M, int N, int K, int epi) {
+                      int M, int N, int K, int epi, int splits = 1, float* partial = nullptr) {
     static bool configured = false;
     size_t bytes = (size_t)STAGES * (BM + BN) * 128;
     if (!configured) {
@@ -555,9 +575,38 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
         if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
         configured = true;
     }
-    dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM), splits);
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
-    gemm_dma_kernel<BM, BN, WGM, WGN, STAGES><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    gemm_dma_kernel<BM, BN, WGM, WGN, STAGES><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
+                                                                                      splits > 1 ? partial : nullptr);
+    if (splits > 1) {
+        size_t pairs = (size_t)M * ((N + 1) / 2);
+        gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
+    }
+    return 0;
+}
+
+// Into how many parts the k range is split over blocks (1: not at all), by the product's shape alone.
+// Up to 64 rows (skinny kernel, 64 x 64 outputs per block): when the features give no more than 64
+// blocks (measured: it pays for N = 4096, K = 14336, and no longer for N = 6144).
+static int skinny_splits(int N, int K) {
+    int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64), splits = 1;
+    while (blocks <= 64 && blocks * splits < 512 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
+    return splits;
+}
+// Above (128 x 128 tiles, two to a compute unit): until the tiles fill the 512 places, each part at
+// least 8 k-tiles long.
+static int tiled_splits(int M, int N, int K) {
+    if (K % 64) return 1;
+    long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128);
+    int nk = K / 64, splits = 1;
+    while (tiles * splits * 2 <= 512 && splits < 16 && nk / (splits * 2) >= 8) splits *= 2;
+    return splits;
+}
+// Room (in floats) for the partial sums of a product that would be split: what the caller should bring.
+extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
+    if (M > 32 && M <= 64) { int s = skinny_splits(N, K); return s > 1 ? (long)s * M * N : 0; }
+    if (M > 64 && (long)ceil_div(M, 256) * ceil_div(N, 256) < 160) { int s = tiled_splits(M, N, K); return s > 1 ? (long)s * M * N : 0; }
     return 0;
 }
 
@@ -613,9 +662,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             // 64 x 64 outputs per block; when that leaves no more than 64 blocks, K is split
             // over blocks too, if the caller gave room for the partial sums (measured: it
             // pays for N = 4096, K = 14336, and no longer for N = 6144).
-            int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64);
-            int splits = 1;
-            while (blocks <= 64 && blocks * splits < 512 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
+            int splits = skinny_splits(N, K);
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
                 launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
@@ -649,7 +696,13 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             } else {
                 rc = launch_dma<256, 256, 2, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
             }
-        } else if (K % 64 == 0) rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        } else if (K % 64 == 0) {
+            int splits = tiled_splits(M, N, K);
+            if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
+                rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
+            else
+                rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+        }
         else rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
     if (rc != 0) return -1;

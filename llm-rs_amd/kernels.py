@@ -70,17 +70,13 @@ class HipKernels:
             raise KernelError(f"the kernel library is built for gfx950, the device is {self.arch!r}")
         self.allow_mfma = True  # tests switch the matrix-core kernels off to compare paths
         lib.llmrs_attention_chunk.restype = I
+        lib.llmrs_gemm_workspace_floats.restype = ctypes.c_long
+        lib.llmrs_gemm_workspace_floats.argtypes = [I, I, I]
         self.attention_chunk = lib.llmrs_attention_chunk()
 
-    @staticmethod
-    def gemm_workspace_floats(M: int, N: int, K: int) -> int:
-        """Room that lets a product with 33..64 tokens split K over blocks (the kernel's own rule)."""
-        if not 32 < M <= 64:
-            return 0
-        blocks, nkb, splits = -(-N // 64), -(-K // 64), 1
-        while blocks <= 64 and blocks * splits < 512 and splits < 16 and nkb // (splits * 2) >= 8:
-            splits *= 2
-        return splits * M * N if splits > 1 else 0
+    def gemm_workspace_floats(self, M: int, N: int, K: int) -> int:
+        """Room that lets a product with too few blocks split K over blocks (the kernels' own rule)."""
+        return int(self.lib.llmrs_gemm_workspace_floats(int(M), int(N), int(K)))
 
     def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int) -> int:
         """Room the split of single-token entries needs for its partial results."""

@@ -59,7 +59,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                # many features: blocks of several feature tiles that start their walk along k at staggered places
                (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192),
                # more large tiles than compute units, the last round not full: the features are split between two tile sizes
-               (513, 25600, 64)]
+               (513, 25600, 64),
+               # few tiles and a long k: the k range is split over blocks and the parts are added by a second kernel
+               (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
