@@ -80,7 +80,7 @@ class StepRunner:
         self._turn = 0
         self._dev_words = torch.zeros(words_capacity, dtype=torch.int32, device=self.device)
         self.ctx = StepContext(self)
-        # HIP graphs of decode steps: key -> (graph, logits); a key is recorded the second time it is seen
+        # HIP graphs of decode steps: key -> (graph, logits); a key is recorded when it has been seen a few times
         self.use_graphs = (self._pinned and os.environ.get("LLMRS_GRAPHS", "1") != "0" and not cache.state_tensors
                            and bool(getattr(model, "graph_safe", lambda: False)()))
         self.max_graph_batch = 512
@@ -237,9 +237,11 @@ class StepRunner:
             hit[0].replay()
             self.graph_replays += 1
             return hit[1]
+        # Recording costs about as much host time as ten eager steps save: a shape is recorded when it
+        # keeps coming back (small batches, where the launches are what a step costs, sooner).
         self._seen[key] = self._seen.get(key, 0) + 1
-        if self._seen[key] < 2:
-            return self.model.forward(ctx, self.cache.views)     # first time: run it, and let the workspace grow
+        if self._seen[key] < (2 if ctx.n_tokens <= 64 else 4):
+            return self.model.forward(ctx, self.cache.views)     # first times: run it, and let the workspace grow
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = self.model.forward(ctx, self.cache.views)
