@@ -103,6 +103,8 @@ __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int 
 
 // One wave: keys [t_begin, t_end) (t_begin a multiple of 32) against its 32 columns.
 // pos / lo: this lane's column may see keys lo..pos (pos < 0: nothing).
+// The request's page numbers are fetched 64 at a time, one in each lane, so that a tile's keys
+// need one trip to memory, not two in a row (page number, then keys).
 template <int HD>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16 (&O)[HD / 32], float& m, float& l,
                                              const bf16* __restrict__ kc, const bf16* __restrict__ vc,
@@ -113,12 +115,18 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
     float scale_log2e = scale * 1.44269504088896341f;
     float alpha_out;
     int kk = (r & ~12) | ((r & 4) << 1) | ((r & 8) >> 1);   // the key (within the tile) that K-operand row r holds
+    if (t_begin >= t_end) return;
+    int pv_base = t_begin >> 4;
+    auto load_pages = [&](int first) {
+        int pg = table[min(first + lane, table_width - 1)];
+        return min(max(pg, 0), num_pages - 1);
+    };
+    int pv = load_pages(pv_base);
     for (int t0 = t_begin; t0 < t_end; t0 += 32) {
         int lp = t0 >> 4;
-        int p0 = table[min(lp, table_width - 1)];
-        int p1 = (t0 + 16 < t_end) ? table[min(lp + 1, table_width - 1)] : p0;
-        p0 = min(max(p0, 0), num_pages - 1);
-        p1 = min(max(p1, 0), num_pages - 1);
+        if (lp + 1 - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
+        int p0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
+        int p1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : p0;   // a tile's second page may lie past the last key
         const bf16* kp = kc + (((size_t)(kk < 16 ? p0 : p1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8;
         f32x16 S;
 #pragma unroll
@@ -223,9 +231,11 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
 
 // ---- the same for head sizes 64, 128, 256, with the four waves of a block sharing their keys --
 // The block's waves own four consecutive groups of tokens of one request and one kv head, so they
-// want the same keys and values (up to the causal edge).  Each 32-key tile (two pages) is
-// brought into LDS once, by global_load_lds straight from the cache's pages, while the tile
-// before it is worked on; all four waves read their MFMA operands from there.  A key's row
+// want the same keys and values (up to the causal edge; every wave walks all of the block's
+// tiles, those beyond its own keys masked).  Each 32-key tile (two pages of keys, two of values)
+// is brought into LDS once, by global_load_lds straight from the cache's pages, several tiles
+// ahead of its use (a ring of R tiles of keys and one of values); all four waves read their
+// MFMA operands from there.  A key's row
 // is 2*HD bytes and the rows lie unpadded, so chunk c of key kk is kept in slot c ^ swz(kk)
 // (swz: kk for 256-byte rows and longer, kk >> 1 for 128-byte rows): the 16 lanes of an operand
 // read want one chunk of 16 different keys and then hit 16 different bank groups.  Values are
@@ -485,13 +495,13 @@ template <int HD>
 __global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
                                                         const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                                         const int* __restrict__ block_table,
-                                                        const int* __restrict__ positions,
+                                                        const int* __restrict__ seq_lens,
                                                         const int* __restrict__ q_starts, AttnArgs a, int G,
                                                         int max_chunks) {
     int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z;
-    if (q_starts[e + 1] - q_starts[e] != 1) return;
-    int token = q_starts[e];
-    int pos_t = positions[token];
+    int token = q_starts[e], count = q_starts[e + 1] - token;
+    int pos_t = seq_lens[e] - 1;                  // an entry with one token: its position is its length less one
+    if (count != 1) return;
     int lo_t = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
     int first_chunk = lo_t / ATTN_CHUNK;
     int n_chunks = pos_t / ATTN_CHUNK - first_chunk + 1;
@@ -527,33 +537,53 @@ __global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__
 #define MERGE_MAX_CHUNKS 1024
 
 // One wave for each (entry, head): lanes share out the chunks for the common maximum and
-// the sum, then the features.  Chunks are added in ascending order.
+// the sum, then the features.  Chunks are added in ascending order.  Everything a lane needs
+// from memory is asked for at once (a chunk's m and l, and its features' sums for the first
+// chunks): the kernel is a chain of trips to memory and little else.
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
-                                                        const int* __restrict__ positions,
+                                                        const int* __restrict__ seq_lens,
                                                         const int* __restrict__ q_starts, AttnArgs a, int max_chunks) {
     __shared__ float weight[MERGE_MAX_CHUNKS];
+    constexpr int AHEAD = 16;                     // chunks whose sums are asked for before the weights are known
     int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim, lane = threadIdx.x;
-    if (q_starts[e + 1] - q_starts[e] != 1) return;
-    int token = q_starts[e];
-    int pos = positions[token];
+    int token = q_starts[e], count = q_starts[e + 1] - token;
+    int pos = seq_lens[e] - 1;
+    if (count != 1) return;
     int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
     int n_chunks = pos / ATTN_CHUNK - lo / ATTN_CHUNK + 1;
     const float* pp = partial + (size_t)(e * a.n_heads + head) * max_chunks * (hd + 2);
+    int stride = hd + 2;
+    // this lane's features d = lane, lane + 64 (head sizes up to 128 in registers; the rest in the loop below)
+    float ahead[2][AHEAD];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int ch = 0; ch < AHEAD; ++ch) {
+            int d = lane + 64 * j;
+            ahead[j][ch] = (ch < n_chunks && d < hd) ? pp[(size_t)ch * stride + 2 + d] : 0.0f;
+        }
     float M = -INFINITY;
-    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * (hd + 2)]);
+    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * stride]);
     M = wave_max(M);
     float L = 0.0f;
     for (int ch = lane; ch < n_chunks; ch += 64) {
-        float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * (hd + 2)] - M);     // the maxima are base-2 logarithms
+        float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * stride] - M);     // the maxima are base-2 logarithms
         weight[ch] = w;
-        L += pp[(size_t)ch * (hd + 2) + 1] * w;
+        L += pp[(size_t)ch * stride + 1] * w;
     }
     L = wave_sum(L);
     __syncthreads();
     float inv = 1.0f / L;
-    for (int d = lane; d < hd; d += 64) {
+    for (int d = lane, j = 0; d < hd; d += 64, ++j) {
         float o = 0.0f;
-        for (int ch = 0; ch < n_chunks; ++ch) o = fmaf(pp[(size_t)ch * (hd + 2) + 2 + d], weight[ch], o);
+        int ch = 0;
+        if (j < 2) {
+#pragma unroll
+            for (int c = 0; c < AHEAD; ++c)
+                if (c < n_chunks) o = fmaf(ahead[j][c], weight[c], o);
+            ch = min(n_chunks, AHEAD);
+        }
+        for (; ch < n_chunks; ++ch) o = fmaf(pp[(size_t)ch * stride + 2 + d], weight[ch], o);
         out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o * inv);
     }
 }
@@ -571,14 +601,14 @@ static int compute_units() {
 
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
-                  const int* positions, const int* q_starts, int n_entries, float* scratch, size_t scratch_bytes,
-                  int max_seq_len, int n_single, const AttnArgs& a) {
+                  const int* positions, const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
+                  size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
     int tpt = 32 / G;
     int max_chunks = max_seq_len > 0 ? (max_seq_len + ATTN_CHUNK - 1) / ATTN_CHUNK : 0;
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.
-    int split = max_chunks > 0 && scratch != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
+    int split = max_chunks > 0 && scratch != nullptr && seq_lens != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
     int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
     if (!only_single) {
         if constexpr (HD == 64 || HD == 128 || HD == 256) {
@@ -593,8 +623,8 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     }
     if (split) {
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
-        attn_split_kernel<HD><<<grid, 64, 0, stream>>>(q, scratch, kc, vc, table, positions, q_starts, a, G, max_chunks);
-        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, positions, q_starts, a, max_chunks);
+        attn_split_kernel<HD><<<grid, 64, 0, stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks);
+        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks);
     }
     return 1;
 }
@@ -603,14 +633,14 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
                               const int* block_table, const int* token_entry, const int* positions,
                               const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
                               size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a) {
-    (void)token_entry; (void)seq_lens;
+    (void)token_entry;
     int G = a.n_heads / a.n_kv_heads;
     if (a.page_size != 16 || a.head_dim % 32 || G > 32 || q_starts == nullptr) return 0;
     if (a.q_stride % 8 || a.out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7)) return 0;
     if (n_entries > 65535 || a.n_kv_heads > 65535) return 0;
     int rc;
     switch (a.head_dim) {
-#define CASE(HD) case HD: rc = launch<HD>(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, n_entries, scratch, scratch_bytes, max_seq_len, n_single, a); break;
+#define CASE(HD) case HD: rc = launch<HD>(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, seq_lens, n_entries, scratch, scratch_bytes, max_seq_len, n_single, a); break;
         CASE(32) CASE(64) CASE(96) CASE(128) CASE(192) CASE(256)
 #undef CASE
         default: return 0;

@@ -50,15 +50,20 @@ __global__ void rmsnorm_rows_reg_kernel(T* __restrict__ out, const float* __rest
     int r = rows ? rows[blockIdx.x] : blockIdx.x;
     const f32x4* src = (const f32x4*)(x + (size_t)r * D);
     int n4 = D / 4;
-    f32x4 v[V4];
+    f32x4 v[V4], ww[V4];
     float ss = 0.0f;
+    // the norm's weight is asked for together with the row: a second trip to memory after the
+    // sum would cost a call with few rows as much again as the first
 #pragma unroll
     for (int i = 0; i < V4; ++i) {
         int idx = i * blockDim.x + threadIdx.x;
         v[i] = idx < n4 ? src[idx] : f32x4{0.f, 0.f, 0.f, 0.f};
+        ww[i] = idx < n4 ? ((const f32x4*)w)[idx] : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < V4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) ss = fmaf(v[i][j], v[i][j], ss);
-    }
     ss = wave_sum(ss);
     int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     if ((threadIdx.x & 63) == 0) partial[wave] = ss;
@@ -71,9 +76,18 @@ __global__ void rmsnorm_rows_reg_kernel(T* __restrict__ out, const float* __rest
     for (int i = 0; i < V4; ++i) {
         int idx = i * blockDim.x + threadIdx.x;
         if (idx < n4) {
-            f32x4 ww = ((const f32x4*)w)[idx];
+            if constexpr (sizeof(T) == 2) {       // four 16-bit results as one 8-byte store
+                typedef T T4 __attribute__((ext_vector_type(4)));
+                T4 o4;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) dst[idx * 4 + j] = from_f32<T>(v[i][j] * inv * ww[j]);
+                for (int j = 0; j < 4; ++j) o4[j] = from_f32<T>(v[i][j] * inv * ww[i][j]);
+                *(T4*)(dst + idx * 4) = o4;
+            } else {
+                f32x4 o4;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o4[j] = v[i][j] * inv * ww[i][j];
+                *(f32x4*)(dst + idx * 4) = o4;
+            }
         }
     }
 }
@@ -99,8 +113,9 @@ extern "C" int llmrs_rmsnorm(hipStream_t stream, int dtype, void* out, const flo
     LLMRS_REQUIRE(eps > 0.0f, "rmsnorm: eps must be positive, got %g", eps);
     if (n_rows == 0) return 0;
     if (dtype != LLMRS_F32 && dtype != LLMRS_BF16) return llmrs_fail("rmsnorm: unknown dtype %d", dtype);
-    int threads = D >= 2048 ? 1024 : 256;
-    bool in_registers = D % 4 == 0 && D <= 4 * 4 * threads && ((uintptr_t)x & 15) == 0 && ((uintptr_t)weight & 15) == 0;
+    int threads = D > 4096 ? 1024 : 256;     // a row of up to 4096 fits the registers of four waves: fewer waves to start and to wait for
+    bool in_registers = D % 4 == 0 && D <= 4 * 4 * threads && ((uintptr_t)x & 15) == 0 && ((uintptr_t)weight & 15) == 0 &&
+                        ((uintptr_t)out & 15) == 0;
     if (in_registers && dtype == LLMRS_F32)
         rmsnorm_rows_reg_kernel<float, 4><<<n_rows, threads, 0, stream>>>((float*)out, x, weight, rows, D, eps);
     else if (in_registers)
