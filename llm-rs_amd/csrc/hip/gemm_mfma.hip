@@ -546,6 +546,43 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
         });
         return;
     }
+    // 16-bit results: a lane holds one column of 16 rows, which stored as they lie would be 2 bytes
+    // per lane and store.  The wave puts its tile through LDS (free after the loop's last barrier; each
+    // wave has room for its own tile) and stores it row by row, 16 bytes per lane, whole lines at a time.
+    bool staged = (epi == LLMRS_EPI_STORE || epi == LLMRS_EPI_SWIGLU) && ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 &&
+                  (epi == LLMRS_EPI_SWIGLU ? N % 16 == 0 : N % 8 == 0);
+    if (staged) {
+        const bool glu = epi == LLMRS_EPI_SWIGLU;
+        const int cols = glu ? TN / 2 : TN;                       // columns of the wave's tile as stored
+        const int row_bytes = cols * 2;
+        static_assert(TN * 2 * TM * WAVES <= STAGES * STAGE_BYTES, "the waves' tiles must fit in the tile buffers");
+        unsigned char* mine = dma_smem + wave * (TN * 2 * TM);
+        static_for<0, FM * FN>([&](auto idx) {
+            constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
+            int c = j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int row = i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                float v = acc[i][j][r];
+                if (glu) {
+                    float other = __shfl_xor(v, 1, 64);           // even lane: gate here, up next door
+                    if (!(lane & 1)) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)(silu_f32(v) * other);
+                } else {
+                    *(bf16*)(mine + row * row_bytes + c * 2) = (bf16)v;
+                }
+            }
+        });
+        __builtin_amdgcn_s_waitcnt(0xc07f);                       // lgkmcnt(0): the wave's own LDS writes are done
+        int lanes_per_row = cols / 8, rows_per_pass = 64 / lanes_per_row;
+        int lr = lane / lanes_per_row, lc = (lane % lanes_per_row) * 8;
+        int n_out = (glu ? (n0 + wn * TN) / 2 : n0 + wn * TN) + lc, n_lim = glu ? N / 2 : N;
+        for (int row = lr; row < TM; row += rows_per_pass) {
+            int m = m0 + wm * TM + row;
+            if (m < M && n_out < n_lim)                           // (n_lim is a multiple of 8: a lane's 8 columns are in or out together)
+                *(bf16x8*)((bf16*)out + (size_t)m * ldc + n_out) = *(const bf16x8*)(mine + row * row_bytes + lc * 2);
+        }
+        return;
+    }
     static_for<0, FM * FN>([&](auto idx) {
         constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
         int n = n0 + wn * TN + j * 32 + (lane & 31);
