@@ -70,6 +70,59 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, const int* __restrict__ posi
     }
 }
 
+// The same for 16-bit rows whose pairs are neighbours (2i, 2i+1), eight features to a thread:
+// one block per token works out the token's cos / sin once (they are the same for all of
+// its heads) and then moves 16 bytes per thread and access.  Needs head_dim, rotary_dim and
+// the row stride to be multiples of 8 and 16-byte aligned rows.
+typedef __bf16 rope_bf16x8 __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qkv, const int* __restrict__ positions,
+                                                           const int* __restrict__ slot_map,
+                                                           const float* __restrict__ inv_freq,
+                                                           bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+                                                           RopeKvArgs a) {
+    extern __shared__ float2 cs[];                 // [rotary_dim / 2]: cos, sin of the token's angles
+    int t = blockIdx.x;
+    float pos = (float)positions[t];
+    for (int i = threadIdx.x; i < a.rotary_dim / 2; i += blockDim.x) {
+        float s, c;
+        sincosf(pos * inv_freq[i], &s, &c);
+        cs[i] = float2{c, s};
+    }
+    __syncthreads();
+    int slot = slot_map[t];
+    bool cache_ok = a.write_kv && slot >= 0 && slot < a.num_pages * a.page_size;   // never write outside the cache
+    int page = cache_ok ? slot / a.page_size : 0, off = cache_ok ? slot % a.page_size : 0;
+    int chunks_per_head = a.head_dim / 8;
+    int q_chunks = a.n_heads * chunks_per_head, all_chunks = (a.n_heads + 2 * a.n_kv_heads) * chunks_per_head;
+    bf16* row = qkv + (size_t)t * a.row_stride;
+    for (int ch = threadIdx.x; ch < all_chunks; ch += blockDim.x) {
+        int head = ch / chunks_per_head, d0 = (ch % chunks_per_head) * 8;
+        bool is_q = ch < q_chunks, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
+        if (!is_q && !cache_ok) continue;
+        rope_bf16x8 v = *(const rope_bf16x8*)(row + (size_t)head * a.head_dim + d0);
+        if ((is_q || is_k) && d0 < a.rotary_dim) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float2 w = cs[d0 / 2 + j];
+                float xa = (float)v[2 * j], xb = (float)v[2 * j + 1];
+                v[2 * j] = (bf16)(xa * w.x - xb * w.y);
+                v[2 * j + 1] = (bf16)(xa * w.y + xb * w.x);
+            }
+        }
+        if (is_q) {
+            *(rope_bf16x8*)(row + (size_t)head * a.head_dim + d0) = v;
+        } else if (is_k) {
+            int kvh = head - a.n_heads;
+            *(rope_bf16x8*)(k_cache + k_cache_index(page, kvh, off, d0, a.n_kv_heads, a.page_size, a.head_dim)) = v;
+        } else {
+            int kvh = head - a.n_heads - a.n_kv_heads;
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v_cache[v_cache_index(page, kvh, off, d0 + j, a.n_kv_heads, a.page_size, a.head_dim)] = v[j];
+        }
+    }
+}
+
 // qkv: [n_tokens, row_stride], a row is q heads, then k heads, then v heads.
 // q is rotated in place; k is rotated and written to k_cache; v is copied to
 // v_cache.  Slots outside [0, num_pages * page_size) are skipped.
@@ -89,6 +142,10 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
     dim3 grid(n_tokens, ceil_div(pairs, 256));
     if (dtype == LLMRS_F32)
         rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, positions, slot_map, inv_freq, (float*)k_cache, (float*)v_cache, a);
+    else if (dtype == LLMRS_BF16 && interleaved && n_tokens >= 16 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0 &&
+             ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && rotary_dim / 2 * sizeof(float2) <= 32768)
+        rope_kv_rows_kernel<<<n_tokens, 256, rotary_dim / 2 * sizeof(float2), stream>>>((bf16*)qkv, positions, slot_map, inv_freq,
+                                                                                        (bf16*)k_cache, (bf16*)v_cache, a);
     else if (dtype == LLMRS_BF16)
         rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
     else

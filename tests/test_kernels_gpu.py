@@ -130,12 +130,14 @@ def test_gemm_small_batches_sum_in_one_order(N, K):
         assert torch.equal(outs[0], o)
 
 
-def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, scaling=None):
-    T, num_pages = 11, 9
+def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, scaling=None, repeat=1):
+    """`repeat` > 1: more tokens, for the kernel that takes a token per block (16 tokens and more)."""
+    T, num_pages = 11 * repeat, 9 * repeat
     S = (n_heads + 2 * n_kv) * hd + 8
     qkv = rnd((T, S), dtype, 8)
     before = qkv.clone()
-    positions = torch.tensor([0, 1, 2, 3, 40, 41, 5, 6, 7, 300, 301], dtype=torch.int32, device=DEV)
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 5, 6, 7, 300, 301] * repeat, dtype=torch.int32, device=DEV)
+    positions = positions + 13 * torch.arange(T, dtype=torch.int32, device=DEV) // 11
     slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(9))[:T].to(torch.int32).to(DEV)
     inv_freq = plain_inv_freq(rot, theta, scaling).to(DEV)
     kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=dtype, device=DEV)
@@ -169,6 +171,13 @@ def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, 
     (6, 2, 80, 32, "split_half", 8), (2, 1, 128, 128, "interleaved", 16), (8, 2, 64, 0, "split_half", 16)])
 def test_rope_kv_write(dtype, n_heads, n_kv, hd, rot, layout, page_size):
     _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,rot,page_size", [(5, 5, 48, 48, 16), (2, 1, 128, 128, 16), (8, 2, 64, 32, 16),
+                                                           (32, 8, 128, 128, 16), (3, 1, 80, 0, 8)])
+def test_rope_kv_write_many_tokens(n_heads, n_kv, hd, rot, page_size):
+    _rope_case(torch.bfloat16, n_heads, n_kv, hd, rot, "interleaved", page_size, repeat=4)
+    _rope_case(torch.float32, n_heads, n_kv, hd, rot, "interleaved", page_size, repeat=4)
 
 
 def test_rope_kv_write_llama3_scaling():
