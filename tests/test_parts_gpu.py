@@ -1,8 +1,9 @@
 """Each part alone against the plain function of its formula, and the generality
 of how parts are put together: a sliding-window attention, a schedule that runs
 a layer twice and lets a run read another run's cache, and a toy mixer with
-state of its own that is defined and registered here, in the test, and built and
-stepped without a change to the package."""
+state of its own, a feed-forward that routes each token to one of several experts
+and a position encoding that is no rotation, all defined and registered here, in the
+test, and built and stepped without a change to the package."""
 import math
 from types import SimpleNamespace
 
@@ -12,8 +13,9 @@ import torch
 from llm_rs_amd import (Engine, FixedState, LayerSpec, ModelSpec, PartSpec, RunSpec, StepEntry, StepRunner,
                         register_architecture)
 from llm_rs_amd.cache import CacheManager, PagedKV
-from llm_rs_amd.parts import (Mixer, TensorSpec, build_block, build_feed_forward, build_mixer, build_norm,
-                              build_position, register_mixer)
+from llm_rs_amd.parts import (FeedForward, Mixer, PositionEncoding, TensorSpec, build_block, build_feed_forward,
+                              build_mixer, build_norm, build_position, register_feed_forward, register_mixer,
+                              register_position)
 from plain_llama import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope, plain_swiglu
 
 pytestmark = pytest.mark.gpu
@@ -296,3 +298,122 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
             assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), (cuts, i)
             eng.close_request(slots[i])
     assert eng.generate([seqs[1][:5]], max_new_tokens=4)[0] == eng.generate([seqs[1][:5]], max_new_tokens=4)[0]
+
+
+class RoutedLinear(FeedForward):
+    """Each token goes to the expert its router logit is largest for (lowest index on ties):
+    y = softmax(x R^T)[e] * (x W_e^T), router logits and softmax in 32-bit."""
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.hidden, self.experts = spec.params["hidden_size"], spec.params["experts"]
+
+    def tensors(self):
+        t = {self.name("router"): TensorSpec((self.experts, self.hidden))}
+        t.update({self.name(f"expert{e}"): TensorSpec((self.hidden, self.hidden)) for e in range(self.experts)})
+        return t
+
+    def load(self, tensors, device):
+        self.router = tensors[self.name("router")].to(device=device, dtype=torch.float32)
+        self.w = torch.stack([tensors[self.name(f"expert{e}")].to(device=device, dtype=torch.float32) for e in range(self.experts)])
+
+    def forward(self, ctx, x, h):
+        xf = x.float()
+        p = torch.softmax(xf @ self.router.T, dim=-1)
+        e = p.argmax(dim=-1)
+        y = torch.einsum("th,toh->to", xf, self.w[e])
+        h += y * p.gather(1, e[:, None])
+
+
+class KeyFade(PositionEncoding):
+    """No rotation: the key at position p is scaled by 1 / (1 + p / span), the query is left alone."""
+
+    def __init__(self, params, dtype):
+        super().__init__(params, dtype)
+        self.span = float(params["span"])
+
+    def apply(self, ctx, q, k):
+        if k is not None:
+            k.mul_((1.0 / (1.0 + ctx.positions.float() / self.span))[:, None, None].to(k.dtype))
+
+
+class ToyRoutedConfig:
+    """Two layers: attention whose keys fade with their position + a routed feed-forward, then
+    rotary attention over a window of 12 keys + SwiGLU."""
+
+    def __init__(self, d):
+        self.d = d
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        H, V = self.d["hidden_size"], self.d["vocab_size"]
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": H, "eps": 1e-6})
+        rope = {"kind": "rope", "head_dim": 16, "rotary_dim": 16, "theta": 1e4, "layout": "split_half"}
+        att0 = PartSpec("attention", "l0.att", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 3, "head_dim": 16,
+                                                "window": None, "position": {"kind": "test_key_fade", "span": 20.0}})
+        att1 = PartSpec("attention", "l1.att", {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                                "window": 12, "position": rope})
+        layers = [LayerSpec("prenorm", att0, PartSpec("test_routed", "l0.moe", {"hidden_size": H, "experts": 3}), norm("l0.n1"), norm("l0.n2")),
+                  LayerSpec("prenorm", att1, PartSpec("swiglu", "l1.mlp", {"hidden_size": H, "intermediate_size": 3 * H}), norm("l1.n1"), norm("l1.n2"))]
+        return ModelSpec(H, V, 256, layers, [RunSpec(0), RunSpec(1)], norm("final"), "embed", "head")
+
+
+def toy_routed_reference(ws, tokens):
+    w = {k: v.double() for k, v in ws.items()}
+    x = w["embed"][torch.tensor(tokens)]
+    T = len(tokens)
+    pos = torch.arange(T)
+    xn = plain_rmsnorm(x, w["l0.n1.weight"], 1e-6)
+    q = (xn @ w["l0.att.q_proj.weight"].T).view(T, 3, 16)
+    k = (xn @ w["l0.att.k_proj.weight"].T).view(T, 3, 16) / (1.0 + pos.double() / 20.0)[:, None, None]
+    v = (xn @ w["l0.att.v_proj.weight"].T).view(T, 3, 16)
+    x = x + plain_attention(q, k, v).reshape(T, 48) @ w["l0.att.o_proj.weight"].T
+    xn = plain_rmsnorm(x, w["l0.n2.weight"], 1e-6)
+    p = torch.softmax(xn @ w["l0.moe.router"].T, dim=-1)
+    e = p.argmax(dim=-1)
+    y = torch.stack([xn[t] @ w[f"l0.moe.expert{int(e[t])}"].T * p[t, e[t]] for t in range(T)])
+    x = x + y
+    xn = plain_rmsnorm(x, w["l1.n1.weight"], 1e-6)
+    inv = plain_inv_freq(16, 1e4, None)
+    q = plain_rope((xn @ w["l1.att.q_proj.weight"].T).view(T, 4, 16), pos, inv)
+    k = plain_rope((xn @ w["l1.att.k_proj.weight"].T).view(T, 2, 16), pos, inv)
+    v = (xn @ w["l1.att.v_proj.weight"].T).view(T, 2, 16)
+    x = x + plain_attention(q, k, v, window=12).reshape(T, 64) @ w["l1.att.o_proj.weight"].T
+    xn = plain_rmsnorm(x, w["l1.n2.weight"], 1e-6)
+    x = x + plain_swiglu(xn, w["l1.mlp.gate_proj.weight"], w["l1.mlp.up_proj.weight"], w["l1.mlp.down_proj.weight"])
+    return plain_rmsnorm(x, w["final.weight"], 1e-6) @ w["head"].T, e
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_routing_and_another_position_encoding(dtype):
+    register_feed_forward("test_routed", RoutedLinear)
+    register_position("test_key_fade", KeyFade)
+    register_architecture("TestToyRoutedForCausalLM", ToyRoutedConfig)
+    H, V = 56, 77
+    cfg = ToyRoutedConfig({"architectures": ["TestToyRoutedForCausalLM"], "hidden_size": H, "vocab_size": V})
+    from llm_rs_amd.engine import Model
+    names = Model(cfg.model_spec(), torch.float32, "cpu").tensors()
+    assert {"l0.moe.router", "l0.moe.expert2", "head"} <= set(names)
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.25)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    eng = Engine(cfg, ws, dtype=dtype, page_size=16, num_pages=24, max_requests=4)
+    assert len(eng.cache.groups) == 2, "all keys for one layer, a window of them for the other"
+    seq = torch.randint(0, V, (60,), generator=torch.Generator().manual_seed(5)).tolist()
+    ref, chosen = toy_routed_reference(ws, seq)
+    assert len(set(chosen.tolist())) == 3, "the test's tokens should reach every expert"
+    tol = 3e-5 if dtype == "float32" else 2.5e-2
+    for cuts in ([60], [7, 30, 1, 1, 2, 19]):
+        slot, pos, rows = eng.open_request(), 0, []
+        for n in cuts:
+            rows.append(eng.step([StepEntry(slot, pos, seq[pos:pos + n], list(range(n)))]).double().cpu())
+            pos += n
+        got = torch.cat(rows)
+        if dtype == "float32":
+            assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), cuts
+        else:
+            # a token whose two best router logits are close may go to another expert in 16-bit: leave those rows out
+            xs = (got - ref).abs().max(dim=1).values <= tol * max(float(ref.abs().max()), 1.0)
+            assert int((~xs).sum()) <= 3, (cuts, int((~xs).sum()))
+        eng.close_request(slot)
