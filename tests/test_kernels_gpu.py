@@ -280,6 +280,26 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
 
 
+@pytest.mark.parametrize("hd", [64, 96, 128, 256])
+def test_attention_prompt_portion_finds_far_keys(hd):
+    """A portion of a prompt far into a long sequence (page numbers are fetched 64 at a time, tiles
+    are loaded several ahead): each of its tokens matches one key, early, late or at a page's or a
+    fetch's edge, so strongly that its output must be that key's value."""
+    dtype, n_heads, n_kv, ps, n = torch.bfloat16, 4, 2, 16, 2300
+    case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=6)
+    far = [0, 15, 16, 31, 32, 500, 1023, 1024, 1025, 1039, 1040, 1100, 2047, 2048, 2063, 2064, 2200, 2251, 2252, 2260]
+    positions = list(range(n - 40, n))
+    q = torch.randn((len(positions), n_heads, hd), generator=torch.Generator().manual_seed(7)) * 0.1
+    for i, f in enumerate(far):
+        q[2 * i] = case.k[0][f, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
+    got = case.run([q.to(dtype)], [positions])
+    ref = case.reference(0, q.to(dtype), positions)
+    for i, f in enumerate(far):
+        want = case.v[0][f].float().repeat_interleave(n_heads // n_kv, dim=0)
+        assert (ref[2 * i].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
+    assert (got.float() - ref.float()).abs().max() <= 2e-2
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window", [1, 5, 16, 17, 64])
 def test_attention_window_edge(dtype, window):
