@@ -300,6 +300,24 @@ def test_attention_prompt_portion_finds_far_keys(hd):
     assert (got.float() - ref.float()).abs().max() <= 2e-2
 
 
+@pytest.mark.parametrize("hd", [64, 128, 256, 96])
+@pytest.mark.parametrize("window", [1, 31, 32, 33, 100, 1200])
+def test_attention_prompt_portion_with_a_window(hd, window):
+    """Portions of a prompt under a sliding window, with the tiled kernels: random queries against
+    the plain function, and for each token the key just outside its window must not be seen."""
+    dtype, n_heads, n_kv, ps, n = torch.bfloat16, 4, 2, 16, 1500
+    case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=8)
+    positions = list(range(n - 70, n))
+    q = torch.randn((len(positions), n_heads, hd), generator=torch.Generator().manual_seed(9))
+    for i in range(0, len(positions), 7):            # these tokens look hard at the key just outside their window
+        outside = positions[i] - window
+        if outside >= 0:
+            q[i] = case.k[0][outside, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
+    got = case.run([q.to(dtype)], [positions], window=window)
+    ref = case.reference(0, q.to(dtype), positions, window=window)
+    assert (got.float() - ref.float()).abs().max() <= 2.5e-2
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window", [1, 5, 16, 17, 64])
 def test_attention_window_edge(dtype, window):
