@@ -643,6 +643,10 @@ static int tiled_splits(int M, int N, int K) {
 // Room (in floats) for the partial sums of a product that would be split: what the caller should bring.
 extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
     if (M > 32 && M <= 64) { int s = skinny_splits(N, K); return s > 1 ? (long)s * M * N : 0; }
+    if (M >= 1024 && M % 256 > 32 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
+        int s = skinny_splits(N, K);            // the rows beyond whole large tiles go to the kernel for few rows
+        return s > 1 ? (long)s * (M % 256) * N : 0;
+    }
     if (M > 64 && (long)ceil_div(M, 256) * ceil_div(N, 256) < 160) { int s = tiled_splits(M, N, K); return s > 1 ? (long)s * M * N : 0; }
     return 0;
 }
@@ -721,6 +725,18 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // tiles get the features that make whole rounds and the small tiles, two to a unit, the rest.
         long m_tiles = ceil_div(M, 256), big_tiles = m_tiles * ceil_div(N, 256);
         int cus = compute_unit_count();
+        // A few rows beyond whole tiles (a prompt portion of 2048 tokens beside 16 decoded ones)
+        // would cost another row of tiles in full: they go to the kernel for few rows instead,
+        // which reads the weight once more at memory speed.
+        int over = M % 256;
+        if (K % 64 == 0 && M >= 1024 && over > 0 && over <= 64 && (m_tiles - 1) * ceil_div(N, 256) >= 160) {
+            size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
+            int whole_rows = M - over;
+            rc = llmrs_gemm_bf16_mfma(stream, A, lda, W, out, ldc, whole_rows, N, K, epi, workspace, workspace_bytes, qkv);
+            if (rc != 1) return rc;
+            return llmrs_gemm_bf16_mfma(stream, A + (size_t)whole_rows * lda, lda, W, (char*)out + (size_t)whole_rows * ldc * elt,
+                                        ldc, over, N, K, epi, workspace, workspace_bytes, qkv);
+        }
         if (K % 64 == 0 && big_tiles >= 160) {
             long whole = big_tiles / cus * cus, rest = big_tiles - whole;
             int n_split = (int)(whole / m_tiles) * 256;        // features of the whole rounds

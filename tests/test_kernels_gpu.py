@@ -61,7 +61,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                # more large tiles than compute units, the last round not full: the features are split between two tile sizes
                (513, 25600, 64),
                # few tiles and a long k: the k range is split over blocks and the parts are added by a second kernel
-               (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048)]
+               (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048),
+               # a few rows beyond whole large tiles: those rows go to the kernel for few rows
+               (1040, 10240, 128), (1080, 10500, 192), (2600, 4096, 1024)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
