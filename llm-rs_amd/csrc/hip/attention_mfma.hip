@@ -583,7 +583,14 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
                 if (c < n_chunks) o = fmaf(ahead[j][c], weight[c], o);
             ch = min(n_chunks, AHEAD);
         }
-        for (; ch < n_chunks; ++ch) o = fmaf(pp[(size_t)ch * stride + 2 + d], weight[ch], o);
+        for (; ch < n_chunks; ch += AHEAD) {      // the rest, a group's sums asked for together
+            float v[AHEAD];
+#pragma unroll
+            for (int c = 0; c < AHEAD; ++c) v[c] = (ch + c < n_chunks) ? pp[(size_t)(ch + c) * stride + 2 + d] : 0.0f;
+#pragma unroll
+            for (int c = 0; c < AHEAD; ++c)
+                if (ch + c < n_chunks) o = fmaf(v[c], weight[ch + c], o);
+        }
         out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o * inv);
     }
 }

@@ -63,7 +63,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                # few tiles and a long k: the k range is split over blocks and the parts are added by a second kernel
                (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048),
                # a few rows beyond whole large tiles: those rows go to the kernel for few rows
-               (1040, 10240, 128), (1080, 10500, 192), (2600, 4096, 1024)]
+               (1040, 10240, 128), (1080, 10500, 192), (2600, 4096, 1024),
+               # long rows: narrow weights walk along k from staggered places too, with two feature tiles to a block
+               (8, 300, 8256), (20, 8200, 16384), (3, 8200, 16400), (40, 520, 8192)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -113,7 +115,7 @@ def test_gemm_rows_do_not_depend_on_batch(dtype):
     assert (outs[0] - outs[1]).abs().max() <= 2e-5 and (outs[0] - outs[2]).abs().max() <= 2e-5
 
 
-@pytest.mark.parametrize("N,K", [(200, 320), (1000, 4096), (16500, 328), (28672, 256)])
+@pytest.mark.parametrize("N,K", [(200, 320), (1000, 4096), (16500, 328), (28672, 256), (500, 8192), (8200, 16448)])
 def test_gemm_small_batches_sum_in_one_order(N, K):
     """Up to 32 rows the matrix-core kernels add a feature's k-blocks in an order that the
     weight's shape fixes: a row's result is the same bits alone, among 8, 20 or 32 rows.
