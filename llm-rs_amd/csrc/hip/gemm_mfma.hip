@@ -640,9 +640,19 @@ static int tiled_splits(int M, int N, int K) {
     while (tiles * splits * 2 <= 512 && splits < 16 && nk / (splits * 2) >= 8) splits *= 2;
     return splits;
 }
+// 33..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
+// get blocks of many feature tiles): the 128 x 128 tiles with k split over blocks read the tokens'
+// rows less often than the few-row kernel's blocks of 32 features (measured at 64 rows:
+// 10240 x 8192 90 -> 51 us, 8192 x 8192 49 -> 38, 8192 x 28672 160 -> 99, 6144 x 4096 31 -> 21).
+static bool few_rows_take_tiles(int M, int N, int K) {
+    return M > 32 && M <= 64 && N > 4096 && N < 16384 && K % 64 == 0 && tiled_splits(M, N, K) > 1;
+}
 // Room (in floats) for the partial sums of a product that would be split: what the caller should bring.
 extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
-    if (M > 32 && M <= 64) { int s = skinny_splits(N, K); return s > 1 ? (long)s * M * N : 0; }
+    if (M > 32 && M <= 64) {
+        int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K);
+        return s > 1 ? (long)s * M * N : 0;
+    }
     if (M >= 1024 && M % 256 > 32 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
         int s = skinny_splits(N, K);            // the rows beyond whole large tiles go to the kernel for few rows
         return s > 1 ? (long)s * (M % 256) * N : 0;
@@ -670,9 +680,19 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         if (M > 64 || qkv == nullptr || qkv->head_dim % 4 || ldc % 4 || ((uintptr_t)out & 7) ||
             ((uintptr_t)qkv->k_cache & 7) || qkv->rotary_dim % 4)
             return 0;
+        // long rows and many tokens: the tiles with k split over blocks are so much faster that
+        // the separate rotation kernel is paid for (10240 x 8192 at 64 rows: 90 us fused, 51 + 6)
+        if (K >= 8192 && few_rows_take_tiles(M, N, K)) return 0;
     }
     int rc = 0;
-    if (M <= 64) {
+    bool tiles_for_few = false;
+    if (epi != LLMRS_EPI_QKV && few_rows_take_tiles(M, N, K)) {
+        int splits = tiled_splits(M, N, K);
+        tiles_for_few = workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float);
+    }
+    if (tiles_for_few) {
+        rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, tiled_splits(M, N, K), (float*)workspace);
+    } else if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
         // waves in turn and their sums are added in wave order, so for a given weight an
         // output's sum has one order whatever M, MT, NT and U are (up to 32 rows; with more, a
