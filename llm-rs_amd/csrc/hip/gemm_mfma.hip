@@ -56,7 +56,7 @@ __device__ __forceinline__ bf16x8 zero8() {
 // With gridDim.y > 1 the k-blocks are shared out over that many blocks as well
 // (contiguous ranges): each writes its 32-bit partial sums to `partial`
 // [gridDim.y][M][N] and gemm_splitk_finish_kernel adds them in order and applies
-// the epilogue.  That is for weights with few rows and many tokens (33..64),
+// the epilogue.  That is for weights with few rows and many tokens (17..64),
 // where blocks of 64 features are needed to keep the tokens' rows from being
 // read too often, and would otherwise be too few to fill the device.
 // ---------------------------------------------------------------------------
@@ -626,9 +626,11 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
 // Into how many parts the k range is split over blocks (1: not at all), by the product's shape alone.
 // Up to 64 rows (skinny kernel, 64 x 64 outputs per block): when the features give no more than 64
 // blocks (measured: it pays for N = 4096, K = 14336, and no longer for N = 6144).
-static int skinny_splits(int N, int K) {
-    int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64), splits = 1;
-    while (blocks <= 64 && blocks * splits < 512 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
+// With 17..32 rows the same, until there are 256 blocks (measured at 32 rows: 4096 x 14336 40 -> 28 us,
+// 2048 x 8192 24 -> 14, 4096 x 4096 14.3 -> 12.9).
+static int skinny_splits(int N, int K, int M = 64) {
+    int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64), splits = 1, enough = M > 32 ? 512 : 256;
+    while (blocks <= 64 && blocks * splits < enough && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
     return splits;
 }
 // Above (128 x 128 tiles, two to a compute unit): until the tiles fill the 512 places, each part at
@@ -640,17 +642,18 @@ static int tiled_splits(int M, int N, int K) {
     while (tiles * splits * 2 <= 512 && splits < 16 && nk / (splits * 2) >= 8) splits *= 2;
     return splits;
 }
-// 33..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
+// 17..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
 // get blocks of many feature tiles): the 128 x 128 tiles with k split over blocks read the tokens'
 // rows less often than the few-row kernel's blocks of 32 features (measured at 64 rows:
-// 10240 x 8192 90 -> 51 us, 8192 x 8192 49 -> 38, 8192 x 28672 160 -> 99, 6144 x 4096 31 -> 21).
+// 10240 x 8192 90 -> 51 us, 8192 x 8192 49 -> 38, 8192 x 28672 160 -> 99, 6144 x 4096 31 -> 21;
+// at 32 rows: 10240 x 8192 63 -> 48, 8192 x 28672 110 -> 90).
 static bool few_rows_take_tiles(int M, int N, int K) {
-    return M > 32 && M <= 64 && N > 4096 && N < 16384 && K % 64 == 0 && tiled_splits(M, N, K) > 1;
+    return M > 16 && M <= 64 && N > 4096 && N < 16384 && K % 64 == 0 && tiled_splits(M, N, K) > 1;
 }
 // Room (in floats) for the partial sums of a product that would be split: what the caller should bring.
 extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
-    if (M > 32 && M <= 64) {
-        int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K);
+    if (M > 16 && M <= 64) {
+        int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K, M);
         return s > 1 ? (long)s * M * N : 0;
     }
     if (M >= 1024 && M % 256 > 32 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
@@ -682,7 +685,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             return 0;
         // long rows and many tokens: the tiles with k split over blocks are so much faster that
         // the separate rotation kernel is paid for (10240 x 8192 at 64 rows: 90 us fused, 51 + 6)
-        if (K >= 8192 && few_rows_take_tiles(M, N, K)) return 0;
+        if (M > 32 && K >= 8192 && few_rows_take_tiles(M, N, K)) return 0;
     }
     int rc = 0;
     bool tiles_for_few = false;
@@ -695,7 +698,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
     } else if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
         // waves in turn and their sums are added in wave order, so for a given weight an
-        // output's sum has one order whatever M, MT, NT and U are (up to 32 rows; with more, a
+        // output's sum has one order whatever M, MT, NT and U are (up to 16 rows; with more, a
         // weight with few rows may have its k-blocks shared out over blocks as well).
         // Features per block (NT*16) grow with N and M: a block reads its tokens' rows
         // again for every 16*NT features, which costs L2 bandwidth once M is large, but
@@ -718,7 +721,11 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             else if (eight) { if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4); else SKINNY(1, 1, 8, 4); }   // 8192 x 28672: 90 -> 83 us
             else SKINNY(1, 1, 4, 4);
         } else if (M <= 32) {
-            if (wide) { if (wide_nt == 7) SKINNY(2, 7, 4, 1); else SKINNY(2, 4, 4, 2); }
+            int splits = skinny_splits(N, K, M);
+            if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
+                workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+                launch_skinny<2, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
+            } else if (wide) { if (wide_nt == 7) SKINNY(2, 7, 4, 1); else SKINNY(2, 4, 4, 2); }
             else if (N > 4096) { if (eight) SKINNY(2, 2, 8, 2); else SKINNY(2, 2, 4, 2); }
             else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {

@@ -66,8 +66,10 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (1040, 10240, 128), (1080, 10500, 192), (2600, 4096, 1024),
                # long rows: narrow weights walk along k from staggered places too, with two feature tiles to a block
                (8, 300, 8256), (20, 8200, 16384), (3, 8200, 16400), (40, 520, 8192),
-               # 33..64 rows on a weight of middling width: large tiles with the k range split over blocks
-               (50, 4160, 1024), (64, 6144, 4096), (40, 5000, 2048), (33, 8192, 8192)]
+               # 17..64 rows on a weight of middling width: large tiles with the k range split over blocks
+               (50, 4160, 1024), (64, 6144, 4096), (40, 5000, 2048), (33, 8192, 8192), (20, 6144, 4096),
+               # 17..32 rows on a weight with few features: blocks of 64 features with the k range split over blocks
+               (32, 4096, 4096), (20, 1000, 8200), (17, 2050, 2048)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -119,14 +121,14 @@ def test_gemm_rows_do_not_depend_on_batch(dtype):
 
 @pytest.mark.parametrize("N,K", [(200, 320), (1000, 4096), (16500, 328), (28672, 256), (500, 8192), (8200, 16448)])
 def test_gemm_small_batches_sum_in_one_order(N, K):
-    """Up to 32 rows the matrix-core kernels add a feature's k-blocks in an order that the
-    weight's shape fixes: a row's result is the same bits alone, among 8, 20 or 32 rows.
+    """Up to 16 rows the matrix-core kernels add a feature's k-blocks in an order that the
+    weight's shape fixes: a row's result is the same bits alone, among 8 or 16 rows.
     (With more rows a weight with few features has its k-blocks shared out over several
     blocks, and from 65 rows on the tiles are others: equal to rounding only.)"""
     a = rnd((32, K), torch.bfloat16, 16)
     w = rnd((N, K), torch.bfloat16, 17, 0.1)
     outs = []
-    for rows in ([7], list(range(4, 12)), list(range(20)), list(range(32))):
+    for rows in ([7], list(range(4, 12)), list(range(13)), list(range(16))):
         sub = a[rows].contiguous()
         out = torch.zeros((len(rows), N), dtype=torch.float32, device=DEV)
         ws = torch.empty(max(1, kernels().gemm_workspace_floats(len(rows), N, K)), dtype=torch.float32, device=DEV)
