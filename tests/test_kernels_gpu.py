@@ -288,6 +288,32 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
 
 
+@pytest.mark.parametrize("n_req", [70, 150])
+def test_attention_many_decoding_requests(n_req):
+    """With many decoding requests a wave of the split takes a longer range of keys (256 to 1024
+    instead of 128).  Each request's query matches one key strongly, chosen at the edges of such
+    ranges where the request is long enough: the output must be that key's value."""
+    n_heads, n_kv, hd, ps = 16, 8, 64, 16
+    g = torch.Generator().manual_seed(n_req)
+    lens = [int(x) for x in torch.randint(5, 1500, (n_req,), generator=g)]
+    lens[0], lens[1] = 1499, 1025
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=11)
+    edges = [0, 127, 128, 255, 256, 511, 512, 1023, 1024, 1279, 1280]
+    qs, fars = [], []
+    for r, n in enumerate(lens):
+        far = [e for e in edges if e < n][r % len([e for e in edges if e < n])] if r % 3 else int(torch.randint(0, n, (1,), generator=g))
+        fars.append(far)
+        qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16))
+    got = case.run(qs, [[n - 1] for n in lens])
+    for r in range(n_req):
+        want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
+        if r < 12:          # the case itself, and the kernel against the plain implementation
+            ref = case.reference(r, qs[r], [lens[r] - 1])[0].float()
+            assert (ref - want).abs().max() < 0.05
+            assert (got[r].float() - ref).abs().max() <= 2e-2, f"request {r}"
+        assert (got[r].float() - want).abs().max() < 0.07, f"request {r} of length {lens[r]}, key {fars[r]}"
+
+
 @pytest.mark.parametrize("hd", [64, 96, 128, 256])
 def test_attention_prompt_portion_finds_far_keys(hd):
     """A portion of a prompt far into a long sequence (page numbers are fetched 64 at a time, tiles
