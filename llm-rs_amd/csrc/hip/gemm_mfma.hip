@@ -624,13 +624,13 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
 }
 
 // Into how many parts the k range is split over blocks (1: not at all), by the product's shape alone.
-// Up to 64 rows (skinny kernel, 64 x 64 outputs per block): when the features give no more than 64
-// blocks (measured: it pays for N = 4096, K = 14336, and no longer for N = 6144).
-// With 17..32 rows the same, until there are 256 blocks (measured at 32 rows: 4096 x 14336 40 -> 28 us,
-// 2048 x 8192 24 -> 14, 4096 x 4096 14.3 -> 12.9).
-static int skinny_splits(int N, int K, int M = 64) {
-    int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64), splits = 1, enough = M > 32 ? 512 : 256;
-    while (blocks <= 64 && blocks * splits < enough && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
+// 17 to 64 rows (few-row kernel, 64 features per block): when the features give no more than 64
+// blocks, until there are 256 of them, each part at least 16 k-blocks long (measured at 64 rows:
+// 4096 x 14336 in 4 parts 35 us, in 8 parts 42; 2048 x 8192 in 8 parts 18 us, in 4 parts 23; at 32
+// rows 4096 x 14336 40 -> 28 us, 2048 x 8192 24 -> 14; it no longer pays for N = 6144).
+static int skinny_splits(int N, int K) {
+    int blocks = ceil_div(N, 64), nkb = ceil_div(K, 64), splits = 1;
+    while (blocks <= 64 && blocks * splits < 256 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
     return splits;
 }
 // Above (128 x 128 tiles, two to a compute unit): until the tiles fill the 512 places, each part at
@@ -653,7 +653,7 @@ static bool few_rows_take_tiles(int M, int N, int K) {
 // Room (in floats) for the partial sums of a product that would be split: what the caller should bring.
 extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
     if (M > 16 && M <= 64) {
-        int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K, M);
+        int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K);
         return s > 1 ? (long)s * M * N : 0;
     }
     if (M >= 1024 && M % 256 > 32 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
@@ -721,7 +721,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             else if (eight) { if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4); else SKINNY(1, 1, 8, 4); }   // 8192 x 28672: 90 -> 83 us
             else SKINNY(1, 1, 4, 4);
         } else if (M <= 32) {
-            int splits = skinny_splits(N, K, M);
+            int splits = skinny_splits(N, K);
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
                 launch_skinny<2, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
@@ -735,7 +735,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             int splits = skinny_splits(N, K);
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
-                launch_skinny<4, 4, 4, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
+                launch_skinny<4, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
             } else if (wide) { if (wide_nt == 7) SKINNY(4, 7, 4, 1); else SKINNY(4, 4, 4, 2); }
             else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
             else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
