@@ -34,6 +34,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=None, help="KV pages (default: sized from free memory)")
+    ap.add_argument("--max-batch-tokens", type=int, default=2048,
+                    help="tokens a step may run (the reference's MAX_TOKENS_PER_STEP); longer prompts are cut into portions")
     sub = ap.add_subparsers(dest="command", required=True)
     c = sub.add_parser("complete", help="Single-shot completion of a prompt given as token ids")
     c.add_argument("-p", "--prompt", required=True, help="token ids, e.g. \"1 15 27\"")
@@ -83,7 +85,7 @@ def main(argv=None) -> int:
         return 1
     try:
         engine = Engine.from_folder(args.model, dtype=args.dtype, page_size=args.page_size, num_pages=args.num_pages,
-                                    max_requests=8, log=True)
+                                    max_requests=8, max_batch_tokens=args.max_batch_tokens, log=True)
     except Exception as e:  # configuration, weights or kernels: one line, as the reference's main does
         print(f"Error: {e}", file=sys.stderr)
         return 1
