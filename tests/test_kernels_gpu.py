@@ -271,13 +271,14 @@ def test_attention_mixed_batch(dtype, n_heads, n_kv, hd, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hd,ps,n", [(64, 16, 700), (128, 16, 1500), (32, 4, 300)])
+@pytest.mark.parametrize("hd,ps,n", [(64, 16, 700), (128, 16, 1500), (32, 4, 300),
+                                     (128, 16, 2300), (64, 16, 5000)])    # more than 16 ranges of 128 keys to merge: the merge kernel's later groups
 def test_attention_finds_a_far_key(dtype, hd, ps, n):
     """Random keys hide a key that is skipped or read from the wrong page: here one
     early key matches the query so strongly that the output must be its value."""
     n_heads, n_kv = 4, 2
     case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=3)
-    for far in (0, ps - 1, ps, n // 2 + 1, n - 2):
+    for far in (0, ps - 1, ps, n // 2 + 1, n - 2) + ((2053, n - 300) if n > 2100 else ()):
         q = torch.zeros((1, n_heads, hd))
         q[0, :, :] = case.k[0][far, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
         got = case.run([q.to(dtype)], [[n - 1]])
