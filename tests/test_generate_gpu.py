@@ -188,3 +188,41 @@ def test_recorded_decode_steps_equal_eager_ones(folders, which, dtype):
             both(lambda sl: [StepEntry(sl[i], pos[i], [seqs[i][pos[i]]], [0]) for i in range(2)])
             pos[0] += 1; pos[1] += 1
     assert recorded.runner.graph_replays >= 30 and eager.runner.graph_replays == 0
+
+
+@pytest.mark.parametrize("hidden,heads,inter", [(4096, 32, 14336), (8192, 64, 28672)])
+def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
+    """The tiny configurations never reach the kernels that wide layers get at 17 to 64 tokens (k ranges
+    split over blocks, large tiles for few rows, a rotation kernel of its own after the qkv product).
+    One layer of an 8B and of a 70B model's widths: the same decoded token alone, among 8, 24 and 48 requests and beside a prompt
+    portion, in bfloat16, against the float32 engine."""
+    from llm_rs_amd import LlamaConfig
+    cfg = LlamaConfig.from_dict(dict(
+        architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=hidden, num_attention_heads=heads,
+        num_key_value_heads=8, head_dim=128, intermediate_size=inter, vocab_size=2000, rope_theta=500000.0,
+        max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=True))
+    n_req, plen = 48, 24
+    prompts = [random_tokens(2000, plen + 1, seed=300 + i) for i in range(n_req)]
+    portion = random_tokens(2000, 150, seed=399)
+    rows = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_random(cfg, 5, dtype=dtype, page_size=16, num_pages=256, max_requests=64)
+        slots = [eng.open_request() for _ in range(n_req)]
+        for s, p in zip(slots, prompts):
+            eng.step([StepEntry(s, 0, p[:plen], [])])
+        extra = eng.open_request()
+        decode = lambda n: [StepEntry(slots[i], plen, [prompts[i][plen]], [0]) for i in range(n)]
+        got = {n: eng.step(decode(n)).float().cpu().clone() for n in (1, 8, 24, 48)}
+        got["mixed"] = eng.step(decode(20) + [StepEntry(extra, 0, portion, [len(portion) - 1])]).float().cpu().clone()
+        rows[dtype] = got
+    ref = rows["float32"][48]
+    scale = float(ref.abs().max())
+    for key, got in rows["float32"].items():                   # float32: any batch, the same to rounding
+        n = min(len(got), n_req) if key != "mixed" else 20
+        assert float((got[:n] - ref[:n]).abs().max()) <= TOLERANCE["float32"] * scale, key
+    for key, got in rows["bfloat16"].items():
+        n = len(got) if key != "mixed" else 20
+        err = float((got[:n] - ref[:n]).abs().max()) / scale
+        assert err <= TOLERANCE["bfloat16"], f"bfloat16 batch {key}: error {err:.3e} of the largest logit"
+    err = float((rows["bfloat16"]["mixed"][20] - rows["float32"]["mixed"][20]).abs().max()) / scale
+    assert err <= TOLERANCE["bfloat16"], f"prompt portion beside decoded tokens: {err:.3e}"
