@@ -289,11 +289,13 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
 
 
+@pytest.mark.parametrize("window", [0, 300])
 @pytest.mark.parametrize("n_req", [70, 150])
-def test_attention_many_decoding_requests(n_req):
+def test_attention_many_decoding_requests(n_req, window):
     """With many decoding requests a wave of the split takes a longer range of keys (256 to 1024
     instead of 128).  Each request's query matches one key strongly, chosen at the edges of such
-    ranges where the request is long enough: the output must be that key's value."""
+    ranges (and of the window, if there is one) where the request is long enough: the output
+    must be that key's value."""
     n_heads, n_kv, hd, ps = 16, 8, 64, 16
     g = torch.Generator().manual_seed(n_req)
     lens = [int(x) for x in torch.randint(5, 1500, (n_req,), generator=g)]
@@ -302,14 +304,16 @@ def test_attention_many_decoding_requests(n_req):
     edges = [0, 127, 128, 255, 256, 511, 512, 1023, 1024, 1279, 1280]
     qs, fars = [], []
     for r, n in enumerate(lens):
-        far = [e for e in edges if e < n][r % len([e for e in edges if e < n])] if r % 3 else int(torch.randint(0, n, (1,), generator=g))
+        lo = max(0, n - window) if window else 0
+        seen = [e for e in edges + [lo, lo + 1, n - 1] if lo <= e < n]
+        far = seen[r % len(seen)] if r % 3 else int(torch.randint(lo, n, (1,), generator=g))
         fars.append(far)
         qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16))
-    got = case.run(qs, [[n - 1] for n in lens])
+    got = case.run(qs, [[n - 1] for n in lens], window=window)
     for r in range(n_req):
         want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
         if r < 12:          # the case itself, and the kernel against the plain implementation
-            ref = case.reference(r, qs[r], [lens[r] - 1])[0].float()
+            ref = case.reference(r, qs[r], [lens[r] - 1], window=window)[0].float()
             assert (ref - want).abs().max() < 0.05
             assert (got[r].float() - ref).abs().max() <= 2e-2, f"request {r}"
         assert (got[r].float() - want).abs().max() < 0.07, f"request {r} of length {lens[r]}, key {fars[r]}"
