@@ -135,16 +135,20 @@ class Engine:
         return self.runner.run(entries)
 
     # -- generation ----------------------------------------------------------------
-    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 256, temperature: float = 0.0,
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: Union[int, Sequence[int]] = 256, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, seed: Union[int, Sequence[int]] = 42,
                  stop_token_ids: Sequence[int] = (), return_reasons: bool = False):
         """Token ids generated for each prompt.  Every request has its own generator
         started from `seed` (one for all, or one each), so a prompt's output does not
-        depend on what it was batched with."""
+        depend on what it was batched with.  `max_new_tokens` too is one for all or one each
+        (a request of the reference carries its own max_tokens, serve/engine.rs:24,35)."""
         n = len(prompts)
         seeds = [seed] * n if isinstance(seed, int) else list(seed)
         if len(seeds) != n:
             raise ValueError("one seed, or one for each prompt")
+        limits = [max_new_tokens] * n if isinstance(max_new_tokens, int) else [int(m) for m in max_new_tokens]
+        if len(limits) != n:
+            raise ValueError("one max_new_tokens, or one for each prompt")
         vocab = self.model.spec.vocab_size
         for i, p in enumerate(prompts):
             if len(p) == 0:
@@ -153,11 +157,11 @@ class Engine:
                 raise ValueError(f"prompt {i}: token ids must be in [0, {vocab})")
         params = [SamplingParams(temperature, top_k, top_p, s) for s in seeds]
         results: List[Optional[Finished]] = [None] * n
-        if max_new_tokens <= 0:
-            results = [Finished([], "length") for _ in range(n)]
-            return [r.tokens for r in results] if not return_reasons else results
+        for i, m in enumerate(limits):          # nothing to generate: done before it starts
+            if m <= 0:
+                results[i] = Finished([], "length")
         core = self.cache.core
-        pending = list(range(n))
+        pending = [i for i in range(n) if results[i] is None]
         slot_of: Dict[int, int] = {}
         stats = GenerationStats(prompt_tokens=sum(len(p) for p in prompts))
         all_greedy = temperature == 0.0
@@ -166,7 +170,7 @@ class Engine:
         def admit():
             while pending:
                 i = pending[0]
-                slot = core.add_request(prompts[i], max_new_tokens, params[i].temperature, params[i].top_k,
+                slot = core.add_request(prompts[i], limits[i], params[i].temperature, params[i].top_k,
                                         params[i].top_p, params[i].seed, stop_token_ids)
                 if slot < 0:
                     return

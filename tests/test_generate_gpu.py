@@ -112,6 +112,9 @@ def test_batching_and_seeds_do_not_change_outputs(folders):
     assert other != together, "another seed draws other tokens"
     per_request = alone_eng.generate(prompts[:2], **{**kw, "seed": [42, 43]})
     assert per_request[0] == together[0] and per_request[1] == other[1]
+    limits = [5, 0, 24, 1, 13]                                   # a limit for each request
+    cut = alone_eng.generate(prompts, **{**kw, "max_new_tokens": limits})
+    assert cut == [t[:m] for t, m in zip(together, limits)]
 
 
 def test_sampled_tokens_follow_the_plain_sampler(folders):
