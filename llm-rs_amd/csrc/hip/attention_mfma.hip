@@ -596,17 +596,6 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
     }
 }
 
-// Compute units of the current device (asked once).
-static int compute_units() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
-    }
-    return n;
-}
-
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
                   const int* positions, const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
@@ -620,7 +609,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     // keys: 64 requests 6945 -> 7540 tokens/s, 256 requests 11960 -> 12740.)
     int chunk = ATTN_CHUNK;
     {
-        long places = (long)compute_units() * 8;
+        long places = (long)llmrs_compute_units() * 8;
         auto waves = [&](int c) { return (long)(n_single > 0 ? n_single : n_entries) * a.n_kv_heads * ((3L * max_seq_len / 4 + c - 1) / c); };
         while (chunk < 8 * ATTN_CHUNK && waves(chunk * 2) >= places) chunk *= 2;
     }
@@ -633,7 +622,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
         if constexpr (HD == 64 || HD == 128 || HD == 256) {
             int btiles = a.n_tokens / (4 * tpt) + n_entries;
             attn_tiles_lds_kernel<HD><<<btiles * a.n_kv_heads, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
-                                                                                 n_entries, a, G, tpt, split, compute_units());
+                                                                                 n_entries, a, G, tpt, split, llmrs_compute_units());
         } else {
             int tiles = a.n_tokens / tpt + n_entries;
             int blocks = ((tiles + 3) / 4) * a.n_kv_heads;

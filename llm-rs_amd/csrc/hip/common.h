@@ -14,6 +14,8 @@ enum LlmrsDtype { LLMRS_F32 = 0, LLMRS_BF16 = 1 };
 // Message of the last failed call on this thread; read through llmrs_hip_error().
 char* llmrs_error_buffer();
 int llmrs_fail(const char* fmt, ...);
+// Compute units of the current device (asked once; 256 if the device cannot be asked).
+int llmrs_compute_units();
 
 #define LLMRS_REQUIRE(cond, ...) \
     do {                         \

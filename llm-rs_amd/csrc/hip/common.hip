@@ -14,6 +14,16 @@ int llmrs_fail(const char* fmt, ...) {
 
 extern "C" const char* llmrs_hip_error() { return g_error; }
 
+int llmrs_compute_units() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
+    }
+    return n;
+}
+
 // Name of the architecture the current device reports, for the loader's check
 // that this library and the device fit each other.
 extern "C" int llmrs_device_arch(char* out, int cap) {

@@ -664,17 +664,6 @@ extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
     return 0;
 }
 
-// Compute units of the current device (asked once).
-static int compute_unit_count() {
-    static int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        n = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) ? prop.multiProcessorCount : 256;
-    }
-    return n;
-}
-
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
                          const QkvEpilogue* qkv) {
@@ -709,7 +698,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // A wide weight's blocks take 7 or 4 feature tiles: whichever number of blocks fills the
         // device's compute units more evenly (28672 features are 256 blocks of 7 tiles).  Its blocks
         // start their walk along k at staggered places, by groups of that many features.
-        int cus = compute_unit_count();
+        int cus = llmrs_compute_units();
         auto evenness = [&](int nt) { int b = ceil_div(N, 16 * nt); return (double)b / ((double)ceil_div(b, cus) * cus); };
         int wide_nt = (wide && evenness(7) >= evenness(4)) ? 7 : 4;
         // Other weights with long rows (measured at 8192 x 8192: 32.6 -> 28.6 us; nothing at K = 4096):
@@ -753,7 +742,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // last round may be far from full (896 tiles on 256 units: 3.5 rounds cost 4).  Then the large
         // tiles get the features that make whole rounds and the small tiles, two to a unit, the rest.
         long m_tiles = ceil_div(M, 256), big_tiles = m_tiles * ceil_div(N, 256);
-        int cus = compute_unit_count();
+        int cus = llmrs_compute_units();
         // A few rows beyond whole tiles (a prompt portion of 2048 tokens beside 16 decoded ones)
         // would cost another row of tiles in full: they go to the kernel for few rows instead,
         // which reads the weight once more at memory speed.
