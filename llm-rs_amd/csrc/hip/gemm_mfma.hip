@@ -656,7 +656,7 @@ extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
         int s = few_rows_take_tiles(M, N, K) ? tiled_splits(M, N, K) : skinny_splits(N, K);
         return s > 1 ? (long)s * M * N : 0;
     }
-    if (M >= 1024 && M % 256 > 32 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
+    if (M >= 1024 && M % 256 > 16 && M % 256 <= 64 && K % 64 == 0 && (long)(M / 256) * ceil_div(N, 256) >= 160) {
         int s = skinny_splits(N, K);            // the rows beyond whole large tiles go to the kernel for few rows
         return s > 1 ? (long)s * (M % 256) * N : 0;
     }
@@ -731,13 +731,12 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         }
 #undef SKINNY
     } else {
-        // 128 x 128 x 64 with one tile of loads in flight measured best of the tile shapes
-        // tried here (larger tiles need a path without bounds checks to pay off).
-        // K % 64 == 0: loads straight into LDS, two tiles in LDS.  Other K: through registers, with
-        // zero-filled tails.
-        // with 128 x 64 per wave (eight waves on a 256 x 256 tile) there is one LDS read per MFMA less
-        // than with 64 x 64 (four waves on 128 x 128), and the loop is bound by LDS bandwidth; it pays
-        // as soon as the larger tiles still fill most of the device (measured on MI355X)
+        // K % 64 == 0: tiles loaded straight into LDS, two k-tiles of 64 there.  Other K: through
+        // registers, with zero-filled tails.
+        // 256 x 256 tiles of eight waves (128 x 64 per wave: one LDS read per MFMA less than the
+        // 64 x 64 per wave of the 128 x 128 tiles) where they fill most of the device; else 128 x 128
+        // tiles of four waves, two blocks to a compute unit, with the k range split over blocks when
+        // even those are too few (measured on MI355X).
         // One large tile runs on a compute unit at a time, so a grid of them works in rounds and the
         // last round may be far from full (896 tiles on 256 units: 3.5 rounds cost 4).  Then the large
         // tiles get the features that make whole rounds and the small tiles, two to a unit, the rest.
