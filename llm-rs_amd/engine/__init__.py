@@ -1,6 +1,6 @@
-from .engine import Engine, Finished, GenerationStats, random_model_tensors
+from .engine import Emitted, Engine, Finished, GenerationStats, random_model_tensors
 from .model import Model
 from .step import OutOfPages, StepContext, StepEntry, StepRunner
 
-__all__ = ["Engine", "Finished", "GenerationStats", "random_model_tensors", "Model", "OutOfPages",
+__all__ = ["Emitted", "Engine", "Finished", "GenerationStats", "random_model_tensors", "Model", "OutOfPages",
            "StepContext", "StepEntry", "StepRunner"]

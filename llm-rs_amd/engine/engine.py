@@ -1,7 +1,8 @@
 """The engine: configuration -> model -> cache -> step function -> scheduler ->
-sampler, and `generate()` above them.  Its loop is the reference's serving loop
-without the HTTP channel (src/serve/engine.rs:161-231): plan, flatten, run,
-sample, commit, free what finished."""
+sampler.  `submit()` and `advance()` are the reference's serving loop without the
+HTTP channel (src/serve/engine.rs:161-231): requests come in at any time, a call
+of `advance()` plans, flattens, runs, samples, commits and frees what finished, and
+says which request got which token.  `generate()` is that loop for a list of prompts."""
 from __future__ import annotations
 
 import gc
@@ -38,6 +39,23 @@ class GenerationStats:
 class Finished:
     tokens: List[int]
     reason: str          # "stop" or "length"
+
+
+@dataclass
+class Emitted:
+    """What one step gave one request: a token (none when a stop token ended it: that token is
+    not part of the output) and, if the request is finished, why ("stop" or "length")."""
+    request: int
+    token: Optional[int]
+    finished: Optional[str] = None
+
+
+@dataclass
+class _Submitted:
+    prompt: Sequence[int]
+    limit: int
+    params: SamplingParams
+    stop: Sequence[int]
 
 
 _collector_quiet = False
@@ -83,6 +101,11 @@ class Engine:
         self.sampler = Sampler(self.device)
         self.max_batch_tokens = max_batch_tokens
         self.last_stats = GenerationStats()
+        self._next_request = 0
+        self._waiting: Dict[int, _Submitted] = {}          # submitted, no slot yet (in order of submission)
+        self._request_of: Dict[int, int] = {}              # slot -> request, for those the scheduler holds
+        self._samples_randomly: set = set()                 # of those, the slots that do not decode greedily
+        self._steps = 0
         if log:
             for g, grp in enumerate(self.cache.groups):
                 gb = grp.num_pages * page_size * grp.bytes_per_token() / 1e9
@@ -134,6 +157,84 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         return self.runner.run(entries)
 
+    # -- requests that come and go -----------------------------------------------------
+    def submit(self, prompt: Sequence[int], max_new_tokens: int = 256, temperature: float = 0.0, top_k: int = 0,
+               top_p: float = 1.0, seed: int = 42, stop_token_ids: Sequence[int] = ()) -> int:
+        """Hands a request to the scheduler; returns its number.  It joins the batch at the next
+        `advance()` that has a slot and pages for it.  Every request has its own generator started
+        from `seed`, so its output does not depend on what it is batched with."""
+        vocab = self.model.spec.vocab_size
+        if len(prompt) == 0:
+            raise ValueError("the prompt is empty")
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise ValueError(f"token ids must be in [0, {vocab})")
+        if max_new_tokens <= 0:
+            raise ValueError("max_new_tokens must be positive")
+        request = self._next_request
+        self._next_request += 1
+        self._waiting[request] = _Submitted(list(prompt), int(max_new_tokens),
+                                            SamplingParams(temperature, top_k, top_p, seed), list(stop_token_ids))
+        return request
+
+    def has_unfinished(self) -> bool:
+        return bool(self._waiting) or bool(self._request_of)
+
+    def cancel(self, request: int) -> None:
+        """Ends a request wherever it stands; its pages and its slot go back."""
+        if self._waiting.pop(request, None) is not None:
+            return
+        for slot, r in list(self._request_of.items()):
+            if r == request:
+                self.cache.core.abort_request(slot)
+                self._forget(slot)
+
+    def _forget(self, slot: int) -> None:
+        self._request_of.pop(slot)
+        self._samples_randomly.discard(slot)
+
+    def _admit(self) -> None:
+        core = self.cache.core
+        for request in list(self._waiting):
+            sub = self._waiting[request]
+            slot = core.add_request(sub.prompt, sub.limit, sub.params.temperature, sub.params.top_k, sub.params.top_p,
+                                    sub.params.seed, sub.stop)
+            if slot < 0:                # no slot free right now: this one and those behind it wait
+                return
+            del self._waiting[request]
+            self._request_of[slot] = request
+            if sub.params.temperature != 0.0:
+                self._samples_randomly.add(slot)
+
+    def advance(self) -> List[Emitted]:
+        """One step of the scheduler: admits what fits, runs the planned batch (prompt portions
+        beside decoded tokens), samples, and returns what each sampling request got.  Requests
+        still inside their prompts get nothing in that step."""
+        core = self.cache.core
+        self._admit()
+        if core.idle():
+            return []
+        logits, n_want, plan = self.runner.run_planned()
+        if not plan:
+            raise RuntimeError("the scheduler planned nothing although requests are waiting")
+        sampled = []
+        if n_want:
+            sampled = self.sampler.sample(logits, self.runner.ctx.sampling, not self._samples_randomly).cpu().numpy()
+        self._steps += 1
+        sampling_slots = [p[0] for p in plan if p[3]]
+        finished = set(core.commit(sampled))
+        out: List[Emitted] = []
+        for slot, token in zip(sampling_slots, sampled):
+            request = self._request_of[slot]
+            if slot in finished:
+                reason = "stop" if core.request_info(slot)["finish"] == 1 else "length"
+                out.append(Emitted(request, None if reason == "stop" else int(token), reason))
+                core.drop_request(slot)
+                self._forget(slot)
+            else:
+                out.append(Emitted(request, int(token)))
+        self._admit()
+        return out
+
     # -- generation ----------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: Union[int, Sequence[int]] = 256, temperature: float = 0.0,
                  top_k: int = 0, top_p: float = 1.0, seed: Union[int, Sequence[int]] = 42,
@@ -149,61 +250,45 @@ class Engine:
         limits = [max_new_tokens] * n if isinstance(max_new_tokens, int) else [int(m) for m in max_new_tokens]
         if len(limits) != n:
             raise ValueError("one max_new_tokens, or one for each prompt")
+        if self.has_unfinished():
+            raise RuntimeError("generate() needs the engine to itself: requests submitted earlier are still running")
         vocab = self.model.spec.vocab_size
         for i, p in enumerate(prompts):
             if len(p) == 0:
                 raise ValueError(f"prompt {i} is empty")
             if min(p) < 0 or max(p) >= vocab:
                 raise ValueError(f"prompt {i}: token ids must be in [0, {vocab})")
-        params = [SamplingParams(temperature, top_k, top_p, s) for s in seeds]
         results: List[Optional[Finished]] = [None] * n
-        for i, m in enumerate(limits):          # nothing to generate: done before it starts
-            if m <= 0:
-                results[i] = Finished([], "length")
-        core = self.cache.core
-        pending = [i for i in range(n) if results[i] is None]
-        slot_of: Dict[int, int] = {}
         stats = GenerationStats(prompt_tokens=sum(len(p) for p in prompts))
-        all_greedy = temperature == 0.0
         t0 = time.perf_counter()
-
-        def admit():
-            while pending:
-                i = pending[0]
-                slot = core.add_request(prompts[i], limits[i], params[i].temperature, params[i].top_k,
-                                        params[i].top_p, params[i].seed, stop_token_ids)
-                if slot < 0:
-                    return
-                slot_of[slot] = i
-                pending.pop(0)
-
+        steps0, preempt0 = self._steps, self.cache.core.preemptions()
+        index_of: Dict[int, int] = {}
+        tokens: Dict[int, List[int]] = {}
         try:
-            admit()
-            while not core.idle() or pending:
-                logits, n_want, plan = self.runner.run_planned()
-                if not plan:
-                    raise RuntimeError("the scheduler planned nothing although requests are waiting")
-                sampled = []
-                if n_want:
-                    sampled = self.sampler.sample(logits, self.runner.ctx.sampling, all_greedy).cpu().numpy()
+            for i, p in enumerate(prompts):
+                if limits[i] <= 0:              # nothing to generate: done before it starts
+                    results[i] = Finished([], "length")
+                    continue
+                r = self.submit(p, limits[i], temperature, top_k, top_p, seeds[i], stop_token_ids)
+                index_of[r], tokens[r] = i, []
+            while self.has_unfinished():
+                for e in self.advance():
                     if stats.first_token_seconds == 0.0:
                         stats.first_token_seconds = time.perf_counter() - t0
-                stats.steps += 1
-                for slot in core.commit(sampled):
-                    info = core.request_info(slot)
-                    i = slot_of.pop(slot)
-                    results[i] = Finished(core.request_output(slot), "stop" if info["finish"] == 1 else "length")
-                    core.drop_request(slot)
-                admit()
+                    if e.token is not None:
+                        tokens[e.request].append(e.token)
+                    if e.finished:
+                        results[index_of[e.request]] = Finished(tokens.pop(e.request), e.finished)
         except BaseException:
-            for slot in list(slot_of):      # leave the engine as it was found
-                core.abort_request(slot)
+            for r in index_of:                  # leave the engine as it was found
+                self.cancel(r)
             raise
         if self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         stats.seconds = time.perf_counter() - t0
+        stats.steps = self._steps - steps0
         stats.generated_tokens = sum(len(r.tokens) for r in results)
-        stats.preemptions = core.preemptions()
+        stats.preemptions = self.cache.core.preemptions() - preempt0
         self.last_stats = stats
         return results if return_reasons else [r.tokens for r in results]
 

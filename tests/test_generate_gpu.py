@@ -229,3 +229,39 @@ def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
         assert err <= TOLERANCE["bfloat16"], f"bfloat16 batch {key}: error {err:.3e} of the largest logit"
     err = float((rows["bfloat16"]["mixed"][20] - rows["float32"]["mixed"][20]).abs().max()) / scale
     assert err <= TOLERANCE["bfloat16"], f"prompt portion beside decoded tokens: {err:.3e}"
+
+
+def test_requests_that_come_and_go(folders):
+    """Requests submitted while others are running, one cancelled on its way: every output equals
+    the request generated alone, and all pages and slots come back."""
+    which = "B"
+    cfg, _ = read_model_folder(folders[which])
+    prompts = [random_tokens(cfg["vocab_size"], n, seed=400 + n) for n in (40, 3, 150, 21, 9, 77)]
+    kw = dict(temperature=0.9, top_k=50, top_p=0.95)
+    limits = [30, 12, 18, 25, 40, 10]
+    alone_eng = engine(folders[which], which, "float32")
+    alone = [alone_eng.generate([p], max_new_tokens=m, seed=60 + i, **kw)[0] for i, (p, m) in enumerate(zip(prompts, limits))]
+    eng = engine(folders[which], which, "float32", max_chunk=32, max_requests=4)     # fewer slots than requests: some wait for one
+    arrivals = {0: [0, 1], 3: [2], 10: [3, 4], 11: [5]}                               # step -> prompts submitted before it
+    number, got, reasons, step = {}, {}, {}, 0
+    cancelled = None
+    while step < 12 or eng.has_unfinished():
+        for i in arrivals.get(step, []):
+            number[eng.submit(prompts[i], limits[i], seed=60 + i, **kw)] = i
+            got[i] = []
+        if step == 14:                                  # prompt 2 is still running: take it out
+            cancelled = [r for r, i in number.items() if i == 2][0]
+            eng.cancel(cancelled)
+        for e in eng.advance():
+            assert e.request != cancelled
+            if e.token is not None:
+                got[number[e.request]].append(e.token)
+            if e.finished:
+                reasons[number[e.request]] = e.finished
+        step += 1
+    for i in (0, 1, 3, 4, 5):
+        assert got[i] == alone[i] and reasons[i] == "length", f"request {i}"
+    assert 0 < len(got[2]) < limits[2] and got[2] == alone[2][:len(got[2])] and 2 not in reasons
+    core = eng.cache.core
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0 and not eng.has_unfinished()
+    assert eng.advance() == []
