@@ -265,3 +265,34 @@ def test_requests_that_come_and_go(folders):
     core = eng.cache.core
     assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0 and not eng.has_unfinished()
     assert eng.advance() == []
+
+
+def test_bfloat16_under_preemption_follows_float32():
+    """A model of middling width (1024 wide, 6 layers), 60 requests, a pool so small that requests are
+    evicted and computed again, greedy in bfloat16: every chosen token is the float32 engine's choice
+    for the same prefix, or so close to it that rounding decides."""
+    import random
+    from llm_rs_amd import LlamaConfig
+    cfg = LlamaConfig.from_dict(dict(
+        architectures=["LlamaForCausalLM"], num_hidden_layers=6, hidden_size=1024, num_attention_heads=16,
+        num_key_value_heads=4, head_dim=64, intermediate_size=2816, vocab_size=5000, rope_theta=10000.0,
+        max_position_embeddings=2048, rms_norm_eps=1e-5, tie_word_embeddings=False))
+    rnd = random.Random(3)
+    prompts = [random_tokens(5000, rnd.randint(1, 600), seed=500 + i) for i in range(60)]
+    limits = [rnd.randint(1, 80) for _ in prompts]
+    bf = Engine.from_random(cfg, 1, dtype="bfloat16", page_size=16, num_pages=70, max_requests=64, max_batch_tokens=512, max_chunk=64)
+    out = bf.generate(prompts, max_new_tokens=limits)
+    assert bf.last_stats.preemptions > 0, "the case must make the scheduler evict"
+    core = bf.cache.core
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
+    del bf
+    ref = Engine.from_random(cfg, 1, dtype="float32", page_size=16, num_pages=64, max_requests=2)
+    for i, (p, o) in enumerate(zip(prompts, out)):
+        assert len(o) == limits[i]
+        slot = ref.open_request()
+        logits = ref.step([StepEntry(slot, 0, p + o, list(range(len(p) - 1, len(p) + len(o) - 1)))]).float()
+        ref.close_request(slot)
+        scale = max(float(logits.abs().max()), 1.0)
+        chosen = logits[torch.arange(len(o)), torch.tensor(o, device=logits.device)]
+        gap = float((logits.max(dim=1).values - chosen).max()) / scale
+        assert gap <= 2 * TOLERANCE["bfloat16"], f"request {i}: a chosen token lies {gap:.3e} of the logit scale below the float32 choice"
