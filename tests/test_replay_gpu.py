@@ -100,3 +100,24 @@ def test_trace_run_program(setup, tmp_path, dtype):
         f = out_dir / f"{s['step']}.f32"
         outputs.append(torch.from_numpy(np.fromfile(f, dtype="<f4").reshape(n, vocab).copy()) if n else None)
     check_rows(collect(steps, outputs), reference[which], dtype, requests[which])
+
+
+# ---- one layer of an 8B model's widths ------------------------------------------------
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    d = tmp_path_factory.mktemp("wide")
+    folder = make_folder(d, "W", seed=9)
+    requests = {f"w{i}": random_tokens(CONFIGS["W"]["vocab_size"], n, seed=40 + i) for i, n in enumerate([40, 100, 230, 70])}
+    return folder, requests, reference_rows(folder, requests)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail", "portions", "mixed"])
+def test_wide_layer(wide, dtype, cut):
+    """The four ways of cutting, on a layer as wide as an 8B model's, against the plain implementation."""
+    folder, requests, reference = wide
+    steps = {"whole": lambda: whole(requests), "tail": lambda: tail_decoded(requests, 32),
+             "portions": lambda: portions(requests), "mixed": lambda: mixed(requests, live=4)}[cut]()
+    rows, rep = run_trace(_make(folder, "W", dtype), steps)
+    print("worst", check_rows(rows, reference, dtype, requests))
+    _check_clean(rep)

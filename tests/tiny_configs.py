@@ -23,8 +23,18 @@ TINY_B = dict(
     max_position_embeddings=512, rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu",
     torch_dtype="bfloat16")
 
-PAGE_SIZE = {"A": 4, "B": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B}
+# One layer with the widths of an 8B model (and a small vocabulary): what the tiny configurations never
+# reach, the kernels that wide layers get (matrix-core products of every row count, head size 128).
+WIDE = dict(
+    architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=4096, num_attention_heads=32,
+    num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=512, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    max_position_embeddings=1024, rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act="silu",
+    torch_dtype="bfloat16")
+
+PAGE_SIZE = {"A": 4, "B": 16, "W": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "W": WIDE}
 
 
 def make_folder(tmp_path, which: str, seed: int = 0, dtype=torch.bfloat16) -> str:
