@@ -113,7 +113,8 @@ struct SampleShared {
     unsigned bcast[4];
     float cand_z[MAX_CAND];
     int cand_i[MAX_CAND];
-    unsigned char rank_drop[MAX_CAND];
+    float by_rank[MAX_CAND];
+    unsigned short rank[MAX_CAND];
 };
 
 __device__ float block_sum_f(float v, SampleShared& s) {
@@ -154,6 +155,41 @@ __device__ unsigned block_min_u(unsigned v, SampleShared& s) {
     __syncthreads();
     return t;
 }
+// The histogram's bin in which the count, taken from bin 255 downwards, reaches `remaining`
+// (bin 0 if it never does), and how many are still to take inside that bin: into bcast[0], bcast[1].
+// The first wave does it, four bins a lane (a walk by one thread is a chain of 256 trips to LDS,
+// 10 us a time).  The caller synchronises afterwards.
+__device__ __forceinline__ void select_bin(SampleShared& s, unsigned remaining) {
+    if (threadIdx.x >= 64) return;
+    int lane = threadIdx.x;
+    unsigned h[4], mine = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { h[j] = s.hist[4 * lane + j]; mine += h[j]; }
+    unsigned above = mine;                      // inclusive suffix sum over the lanes, then exclusive
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        unsigned o = __shfl_down(above, off, 64);
+        if (lane + off < 64) above += o;
+    }
+    above -= mine;
+    int bin = -1;
+    unsigned left = 0, seen = above;
+#pragma unroll
+    for (int j = 3; j >= 0; --j) {
+        if (bin < 0 && seen + h[j] >= remaining) { bin = 4 * lane + j; left = remaining - seen; }
+        seen += h[j];
+    }
+    unsigned long long found = __ballot(bin >= 0);
+    int top = found ? 63 - __clzll(found) : -1;  // the highest lane that holds a crossing: the first from above
+    if (top < 0 || (top == 0 && __shfl(bin, 0, 64) == 0)) {
+        // never reached above bin 0, or only inside it: bin 0, less everything above it
+        if (lane == 0) { s.bcast[0] = 0u; s.bcast[1] = remaining - (above + mine - h[0]); }
+    } else if (lane == top) {
+        s.bcast[0] = (unsigned)bin;
+        s.bcast[1] = left;
+    }
+}
+
 // Smallest index c with exactly `need` elements of key `key` at indices <= c.
 __device__ int index_cut(const float* row, int V, float inv_t, unsigned key, unsigned need, SampleShared& s) {
     int lo = 0, hi = V - 1;     // invariant: count(<= hi) >= need
@@ -167,54 +203,73 @@ __device__ int index_cut(const float* row, int V, float inv_t, unsigned key, uns
     return lo;
 }
 
-// One thread finishes a row whose candidates lie in LDS in index order (those with
-// rank_drop set are outside the top k): softmax, the top_p cut, the draw.
-__device__ void finish_candidates(SampleShared& s, int n, float zmax, float top_p, float u, int* result) {
-    float sum = 0.0f;
-    for (int c = 0; c < n; ++c) {
-        s.cand_z[c] = s.rank_drop[c] ? 0.0f : expf(s.cand_z[c] - zmax);
-        sum += s.cand_z[c];
+// The whole block finishes a row whose candidates lie in LDS in index order.  A candidate's rank
+// is the number of candidates before it in the order (value descending, index ascending); those of
+// rank >= top_k are outside.  Ranks, exponentials and scalings are shared out over the threads;
+// every sum is one thread's, sequential and in 32 bits, as the reference's loops are: the softmax
+// sum and the draw in index order, the top_p mass in descending order.
+__device__ void finish_candidates(SampleShared& s, int n, int top_k, float zmax, float top_p, float u, int* result) {
+    int tid = threadIdx.x;
+    for (int c = tid; c < n; c += SAMPLE_THREADS) {
+        float z = s.cand_z[c];
+        int idx = s.cand_i[c], rank = 0;
+        for (int j = 0; j < n; ++j) {
+            float zj = s.cand_z[j];
+            rank += zj > z || (zj == z && s.cand_i[j] < idx);
+        }
+        s.rank[c] = (unsigned short)rank;
     }
-    float inv = 1.0f / sum;
-    for (int c = 0; c < n; ++c) s.cand_z[c] *= inv;           // probabilities
+    __syncthreads();
+    for (int c = tid; c < n; c += SAMPLE_THREADS) s.cand_z[c] = s.rank[c] < top_k ? expf(s.cand_z[c] - zmax) : 0.0f;
+    __syncthreads();
+    if (tid == 0) {
+        float sum = 0.0f;
+        for (int c = 0; c < n; ++c) sum += s.cand_z[c];
+        s.f[0] = 1.0f / sum;
+    }
+    __syncthreads();
+    float inv = s.f[0];
+    for (int c = tid; c < n; c += SAMPLE_THREADS) s.cand_z[c] *= inv;           // probabilities
+    __syncthreads();
     if (top_p < 1.0f) {
-        // walk in descending order (equal values: lower index first) until the mass reaches top_p
-        float mass = 0.0f, last_p = INFINITY;
-        int last_i = -1, taken = 0;
-        while (taken < n) {
-            int best = -1;
-            for (int c = 0; c < n; ++c) {
-                float p = s.cand_z[c];
-                bool after_last = p < last_p || (p == last_p && s.cand_i[c] > last_i);
-                if (after_last && (best < 0 || p > s.cand_z[best])) best = c;
+        int m = min(n, top_k);                                                   // the candidates inside have ranks 0..m-1
+        for (int c = tid; c < n; c += SAMPLE_THREADS)
+            if (s.rank[c] < m) s.by_rank[s.rank[c]] = s.cand_z[c];
+        __syncthreads();
+        if (tid == 0) {     // descending order until the mass reaches top_p
+            float mass = 0.0f;
+            int last = 0;
+            for (; last < m - 1; ++last) {
+                mass += s.by_rank[last];
+                if (mass >= top_p) break;
             }
-            last_p = s.cand_z[best];
-            last_i = s.cand_i[best];
-            mass += last_p;
-            ++taken;
-            if (mass >= top_p) break;
+            s.bcast[0] = (unsigned)last;
         }
-        float kept_sum = 0.0f;
+        __syncthreads();
+        int last = (int)s.bcast[0];
+        for (int c = tid; c < n; c += SAMPLE_THREADS)
+            if (s.rank[c] > last) s.cand_z[c] = 0.0f;
+        __syncthreads();
+        if (tid == 0) {
+            float kept_sum = 0.0f;
+            for (int c = 0; c < n; ++c) kept_sum += s.cand_z[c];
+            s.f[0] = kept_sum > 0.0f ? 1.0f / kept_sum : 1.0f;
+        }
+        __syncthreads();
+        float inv2 = s.f[0];
+        for (int c = tid; c < n; c += SAMPLE_THREADS) s.cand_z[c] *= inv2;
+        __syncthreads();
+    }
+    if (tid == 0) {
+        float cum = 0.0f;
+        int pick = -1, last_kept = 0;
         for (int c = 0; c < n; ++c) {
-            float p = s.cand_z[c];
-            bool keep = p > last_p || (p == last_p && s.cand_i[c] <= last_i);
-            if (!keep) s.cand_z[c] = 0.0f;
-            kept_sum += s.cand_z[c];
+            if (s.cand_z[c] > 0.0f) last_kept = s.cand_i[c];
+            cum += s.cand_z[c];
+            if (u < cum) { pick = s.cand_i[c]; break; }
         }
-        if (kept_sum > 0.0f) {
-            float inv2 = 1.0f / kept_sum;
-            for (int c = 0; c < n; ++c) s.cand_z[c] *= inv2;
-        }
+        *result = pick >= 0 ? pick : last_kept;
     }
-    float cum = 0.0f;
-    int pick = -1, last_kept = 0;
-    for (int c = 0; c < n; ++c) {
-        if (s.cand_z[c] > 0.0f) last_kept = s.cand_i[c];
-        cum += s.cand_z[c];
-        if (u < cum) { pick = s.cand_i[c]; break; }
-    }
-    *result = pick >= 0 ? pick : last_kept;
-
 }
 
 // Exclusive prefix of v over the block's waves (wave order), and the total; v is a per-wave value.
@@ -261,8 +316,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     if (!(temp > 0.0f)) {   // greedy row: largest logit, lowest index on ties
         float best = -INFINITY;
         unsigned idx = 0xffffffffu;
-    #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) {
+#pragma unroll 8
+        for (int i = w_lo + lane; i < w_hi; i += 64) {
             float v = row[i];
             if (v > best || idx == 0xffffffffu) { best = v; idx = i; }
         }
@@ -273,9 +328,24 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     }
 
     float inv_t = 1.0f / temp;
-    float mine_max = -INFINITY;
+    // Rows that allow it are read 16 bytes a lane (a wave's round is 256 consecutive values, a lane's
+    // four of them consecutive): four times the bytes in flight of a block that has a row to itself.
+    bool vec = (((uintptr_t)row | (uintptr_t)V) & 3) == 0 && ((uintptr_t)row & 15) == 0;
+    float mine_max = -INFINITY;        // largest value of this thread's share (any sharing out will do here)
+    bool mine_any = false;
+    if (vec) {
+        const float4* row4 = (const float4*)row;
+#pragma unroll 4
+        for (int i = tid; i < (V >> 2); i += SAMPLE_THREADS) {
+            float4 v = row4[i];
+            mine_max = fmaxf(fmaxf(mine_max, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+            mine_any = true;
+        }
+    } else {
 #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) mine_max = fmaxf(mine_max, row[i] * inv_t);
+        for (int i = w_lo + lane; i < w_hi; i += 64) { mine_max = fmaxf(mine_max, row[i]); mine_any = true; }
+    }
+    mine_max *= inv_t;                 // scaling keeps the order: the largest scaled value is the scaled largest
     float zmax = block_max_f(mine_max, s);
     bool use_k = top_k > 0 && top_k < V;
 
@@ -284,14 +354,47 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     // they do not fit).
     auto gather = [&](unsigned bound, int cut) -> unsigned {
         auto in = [&](int i) { unsigned k = order_key(row[i] * inv_t); return k > bound || (k == bound && i <= cut); };
+        auto in_z = [&](float z, int i) { unsigned k = order_key(z); return k > bound || (k == bound && i <= cut); };
         unsigned cnt = 0;
-    #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) cnt += in(i);
+        if (vec) {      // (w_lo and w_hi are multiples of 4 here: V is, and the stretches are multiples of 64)
+#pragma unroll 4
+            for (int i = w_lo + lane * 4; i < w_hi; i += 256) {
+                float4 v = *(const float4*)(row + i);
+                cnt += in_z(v.x * inv_t, i) + in_z(v.y * inv_t, i + 1) + in_z(v.z * inv_t, i + 2) + in_z(v.w * inv_t, i + 3);
+            }
+        } else {
+#pragma unroll 8
+            for (int i = w_lo + lane; i < w_hi; i += 64) cnt += in(i);
+        }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, 64);
         unsigned total;
         unsigned base = wave_prefix_u(cnt, s, total);
         if (total > MAX_CAND) return total;
+        if (vec) {
+            unsigned long long below = (1ull << lane) - 1ull;
+            for (int i0 = w_lo; i0 < w_hi; i0 += 256) {
+                int i = i0 + lane * 4;
+                bool ok = i < w_hi;
+                float4 v = ok ? *(const float4*)(row + i) : float4{0.f, 0.f, 0.f, 0.f};
+                float z[4] = {v.x * inv_t, v.y * inv_t, v.z * inv_t, v.w * inv_t};
+                bool f[4];
+                unsigned long long b[4];
+                unsigned at = base;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    f[j] = ok && in_z(z[j], i + j);
+                    b[j] = __ballot(f[j]);
+                    at += __popcll(b[j] & below);          // those of the lanes before this one
+                    base += __popcll(b[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (f[j]) { s.cand_z[at] = z[j]; s.cand_i[at] = i + j; ++at; }
+            }
+            __syncthreads();
+            return total;
+        }
         for (int i0 = w_lo; i0 < w_hi; i0 += 64) {
             int i = i0 + lane;
             bool p = i < w_hi && in(i);
@@ -309,23 +412,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
 
     if (use_k && top_k <= SAMPLE_THREADS) {
         // ---- a lower bound of the k-th largest value: the k-th largest of the threads' maxima
-        unsigned mykey = w_lo + lane < w_hi ? order_key(mine_max) : 0u;
+        unsigned mykey = mine_any ? order_key(mine_max) : 0u;
         unsigned prefix = 0, mask = 0, remaining = top_k;
         for (int shift = 24; shift >= 0; shift -= 8) {
             for (int b = tid; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0;
             __syncthreads();
             if ((mykey & mask) == prefix) atomicAdd(&s.hist[(mykey >> shift) & 255], 1u);
             __syncthreads();
-            if (tid == 0) {
-                unsigned seen = 0;
-                int b = 255;
-                for (; b > 0; --b) {
-                    if (seen + s.hist[b] >= remaining) break;
-                    seen += s.hist[b];
-                }
-                s.bcast[0] = (unsigned)b;
-                s.bcast[1] = remaining - seen;
-            }
+            select_bin(s, remaining);
             __syncthreads();
             prefix |= s.bcast[0] << shift;
             mask |= 255u << shift;
@@ -334,20 +428,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         }
         // at least top_k values of the row have a key >= prefix
         unsigned n = gather(prefix, V);
-        if (n <= MAX_CAND) {
-            // ---- the k largest of the candidates: a candidate's rank is the number of
-            // candidates before it in the order (value descending, index ascending)
-            for (int c = tid; c < (int)n; c += SAMPLE_THREADS) {
-                float z = s.cand_z[c];
-                int idx = s.cand_i[c], rank = 0;
-                for (int j = 0; j < (int)n; ++j) {
-                    float zj = s.cand_z[j];
-                    rank += zj > z || (zj == z && s.cand_i[j] < idx);
-                }
-                s.rank_drop[c] = rank >= top_k;
-            }
-            __syncthreads();
-            if (tid == 0) finish_candidates(s, (int)n, zmax, top_p, u, &out[blockIdx.x]);
+        if (n <= MAX_CAND) {    // the k largest of the candidates, and the rest of the row's work, in LDS
+            finish_candidates(s, (int)n, top_k, zmax, top_p, u, &out[blockIdx.x]);
             return;
         }
         // too many equal or near values: the general path below handles it
@@ -361,22 +443,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         for (int shift = 24; shift >= 0; shift -= 8) {
             for (int b = tid; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0;
             __syncthreads();
-        #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) {
+#pragma unroll 8
+            for (int i = w_lo + lane; i < w_hi; i += 64) {
                 unsigned k = order_key(row[i] * inv_t);
                 if ((k & mask) == prefix) atomicAdd(&s.hist[(k >> shift) & 255], 1u);
             }
             __syncthreads();
-            if (tid == 0) {
-                unsigned seen = 0;
-                int b = 255;
-                for (; b > 0; --b) {
-                    if (seen + s.hist[b] >= remaining) break;
-                    seen += s.hist[b];
-                }
-                s.bcast[0] = (unsigned)b;
-                s.bcast[1] = remaining - seen;   // still to take inside bin b
-            }
+            select_bin(s, remaining);
             __syncthreads();
             prefix |= s.bcast[0] << shift;
             mask |= 255u << shift;
@@ -386,16 +459,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         kth = prefix;
         unsigned keep_eq = remaining;            // >= 1 of the values equal to the k-th stay
         unsigned n_eq = 0;
-    #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) n_eq += order_key(row[i] * inv_t) == kth;
+#pragma unroll 8
+        for (int i = w_lo + lane; i < w_hi; i += 64) n_eq += order_key(row[i] * inv_t) == kth;
         n_eq = block_sum_u(n_eq, s);
         if (n_eq > keep_eq) cut_k = index_cut(row, V, inv_t, kth, keep_eq, s);
         if (top_k <= MAX_CAND) {
             unsigned n = gather(kth, cut_k);     // exactly top_k values
-            if (tid == 0) {
-                for (int c = 0; c < (int)n; ++c) s.rank_drop[c] = 0;
-                finish_candidates(s, (int)n, zmax, top_p, u, &out[blockIdx.x]);
-            }
+            finish_candidates(s, (int)n, (int)n, zmax, top_p, u, &out[blockIdx.x]);
             return;
         }
     }
@@ -403,24 +473,24 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
 
     // ---- no top_k (or a huge one): work on the whole row
     float mine = 0.0f;
-#pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) {
-        float z = row[i] * inv_t;
-        if (kept_k(order_key(z), i)) mine += expf(z - zmax);
-    }
-    float S = block_sum_f(mine, s);
     unsigned pth = 0;       // keep: key > pth, or key == pth at indices <= cut_p
     int cut_p = V;
     bool use_p = top_p < 1.0f;
     if (use_p) {
+#pragma unroll 8
+        for (int i = w_lo + lane; i < w_hi; i += 64) {
+            float z = row[i] * inv_t;
+            if (kept_k(order_key(z), i)) mine += expf(z - zmax);
+        }
+        float S = block_sum_f(mine, s);
         float want = top_p * S;
         // largest key c with mass(key >= c) >= want, bit by bit
         unsigned prefix = 0;
         for (int bit = 31; bit >= 0; --bit) {
             unsigned cand = prefix | (1u << bit);
             float m = 0.0f;
-        #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) {
+#pragma unroll 8
+            for (int i = w_lo + lane; i < w_hi; i += 64) {
                 float z = row[i] * inv_t;
                 unsigned k = order_key(z);
                 if (k >= cand && kept_k(k, i)) m += expf(z - zmax);
@@ -430,8 +500,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         pth = prefix;
         float m_gt = 0.0f;
         unsigned n_eq = 0;
-    #pragma unroll 8
-    for (int i = w_lo + lane; i < w_hi; i += 64) {
+#pragma unroll 8
+        for (int i = w_lo + lane; i < w_hi; i += 64) {
             float z = row[i] * inv_t;
             unsigned k = order_key(z);
             if (!kept_k(k, i)) continue;
@@ -468,29 +538,70 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         if (tid == 0) out[blockIdx.x] = (int)last_kept;
         return;
     }
-    if ((unsigned)wave != owner) return;
-    float cum = before;
-    int pick = -1, last_in_wave = -1;
-    for (int i0 = w_lo; i0 < w_hi && pick < 0; i0 += 64) {
-        int i = i0 + lane;
-        float e = 0.0f;
-        if (i < w_hi) {
-            float z = row[i] * inv_t;
-            if (kept(order_key(z), i)) e = expf(z - zmax);
-        }
-        float inc = e;
+    // ---- the owner's stretch is shared out over all waves once more (a walk through all of it by one
+    // wave is a hundred rounds, one after the other): sub-stretches of at most WALK rounds, their
+    // masses, the one that holds the uniform, and a walk through that one from registers.
+    constexpr int WALK = 8;
+    if ((unsigned)wave == owner && lane == 0) s.bcast[0] = __float_as_uint(before);
+    __syncthreads();
+    float cum = __uint_as_float(s.bcast[0]);
+    __syncthreads();
+    int o_lo = min((int)owner * stretch, V), o_hi = min(o_lo + stretch, V);
+    int pick = -1;
+    while (pick < 0) {      // (one turn unless the stretch is longer than 16 * WALK rounds: then sub-stretch by sub-stretch)
+        int span = min(o_hi - o_lo, SAMPLE_WAVES * WALK * 64);
+        int sub = (((span + SAMPLE_WAVES - 1) / SAMPLE_WAVES) + 63) & ~63;
+        int s_lo = min(o_lo + wave * sub, o_lo + span), s_hi = min(s_lo + sub, o_lo + span);
+        float es[WALK];
+        float part = 0.0f;
+        int my_sub_last = -1;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            float o = __shfl_up(inc, off, 64);
-            if (lane >= off) inc += o;
+        for (int r = 0; r < WALK; ++r) {
+            int i = s_lo + 64 * r + lane;
+            es[r] = 0.0f;
+            if (i < s_hi) {
+                float z = row[i] * inv_t;
+                if (kept(order_key(z), i)) { es[r] = expf(z - zmax); my_sub_last = i; }
+            }
+            part += es[r];
         }
-        unsigned long long hit = __ballot(e > 0.0f && target < cum + inc);
-        unsigned long long any = __ballot(e > 0.0f);
-        if (any) last_in_wave = i0 + 63 - __clzll(any);
-        if (hit) pick = i0 + __ffsll((long long)hit) - 1;
-        cum += __shfl(inc, 63, 64);
+        float sub_mass = wave_sum(part);
+        float sub_total;
+        float sub_before = wave_prefix_f(sub_mass, s, sub_total);
+        unsigned sub_owner = block_min_u((sub_mass > 0.0f && target < cum + sub_before + sub_mass) ? (unsigned)wave : 0xffffffffu, s);
+        unsigned sub_last = V - 1 - block_min_u(my_sub_last >= 0 ? (unsigned)(V - 1 - my_sub_last) : 0xffffffffu, s);
+        if (sub_owner == 0xffffffffu) {
+            if (o_lo + span >= o_hi) {          // rounding left the uniform past the stretch's last sum
+                if (tid == 0) out[blockIdx.x] = sub_last < (unsigned)V ? (int)sub_last : (int)last_kept;
+                return;
+            }
+            cum += sub_total;                   // not in this part of the stretch: on to the next
+            o_lo += span;
+            continue;
+        }
+        if ((unsigned)wave != sub_owner) return;
+        float c = cum + sub_before;
+        int last_in_wave = -1;
+#pragma unroll
+        for (int r = 0; r < WALK; ++r) {
+            int i0 = s_lo + 64 * r;
+            if (pick >= 0) break;
+            float e = es[r], inc = e;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                float o = __shfl_up(inc, off, 64);
+                if (lane >= off) inc += o;
+            }
+            unsigned long long hit = __ballot(e > 0.0f && target < c + inc);
+            unsigned long long any = __ballot(e > 0.0f);
+            if (any) last_in_wave = i0 + 63 - __clzll(any);
+            if (hit) pick = i0 + __ffsll((long long)hit) - 1;
+            c += __shfl(inc, 63, 64);
+        }
+        if (pick < 0) pick = last_in_wave;      // rounding again: the sub-stretch's last kept value
+        if (lane == 0) out[blockIdx.x] = pick;
+        return;
     }
-    if (lane == 0) out[blockIdx.x] = pick >= 0 ? pick : last_in_wave;
 }
 
 // words: [n_rows, 4] = uniform (float bits), temperature (float bits), top_k, top_p (float bits)
