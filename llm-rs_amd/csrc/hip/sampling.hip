@@ -82,14 +82,17 @@ extern "C" int llmrs_argmax_rows(hipStream_t stream, const float* logits, int ld
 //     stretch of the row; the k-th largest of those 1024 maxima is a lower bound of
 //     the k-th largest value of the row, so everything at or above it (a few
 //     dozen values, typically) is gathered into LDS in index order, ranked there,
-//     and cut to the k largest; one thread then finishes the row exactly as the
-//     reference's loop does (descending order, sequential 32-bit cumulative sums).
-//     Three passes over the row in all;
+//     and cut to the k largest; the block then finishes the row as the reference's
+//     loops do (descending order, sequential 32-bit cumulative sums by one thread; ranks,
+//     exponentials and scalings shared out).  Three passes over the row in all;
+//   * top_p without top_k: the same with the 512 largest values as candidates and the
+//     softmax sum of the whole row taken in the gathering pass; if the top_p mass is
+//     reached inside the candidates (any row but a flat one), the row is finished there;
 //   * a larger top_k: the k-th largest value by a radix select over order-preserving
 //     keys (4 passes with a 256-bin histogram), survivors into LDS if they fit;
-//   * without top_k (or a very large one) the top_p cut is found by a bitwise
-//     search over keys with block-wide sums, and the draw by a scan over
-//     contiguous segments.
+//   * else (flat rows under top_p alone, a very large top_k) the top_p cut is found by a
+//     bitwise search over keys with block-wide sums (32 passes: 0.7-0.9 ms on a row of
+//     128 K), and the draw by a scan over contiguous segments, shared out twice.
 // Of equal values at a cut the lowest indices stay (the reference's unstable
 // sorts leave that open).  Every sum has a fixed order: a row's token depends on
 // its logits and its uniform only.
@@ -208,7 +211,11 @@ __device__ int index_cut(const float* row, int V, float inv_t, unsigned key, uns
 // rank >= top_k are outside.  Ranks, exponentials and scalings are shared out over the threads;
 // every sum is one thread's, sequential and in 32 bits, as the reference's loops are: the softmax
 // sum and the draw in index order, the top_p mass in descending order.
-__device__ void finish_candidates(SampleShared& s, int n, int top_k, float zmax, float top_p, float u, int* result) {
+// `total` > 0: the softmax sum of the whole row, of which the candidates are the largest values
+// (top_p without top_k); then, unless they are the whole row (`complete`), the top_p mass must be
+// reached inside them: if it is not, nothing is written and false comes back (to every thread).
+__device__ bool finish_candidates(SampleShared& s, int n, int top_k, float zmax, float top_p, float u, int* result,
+                                  float total = 0.0f, bool complete = true) {
     int tid = threadIdx.x;
     for (int c = tid; c < n; c += SAMPLE_THREADS) {
         float z = s.cand_z[c];
@@ -223,8 +230,11 @@ __device__ void finish_candidates(SampleShared& s, int n, int top_k, float zmax,
     for (int c = tid; c < n; c += SAMPLE_THREADS) s.cand_z[c] = s.rank[c] < top_k ? expf(s.cand_z[c] - zmax) : 0.0f;
     __syncthreads();
     if (tid == 0) {
-        float sum = 0.0f;
-        for (int c = 0; c < n; ++c) sum += s.cand_z[c];
+        float sum = total;
+        if (!(total > 0.0f)) {
+            sum = 0.0f;
+            for (int c = 0; c < n; ++c) sum += s.cand_z[c];
+        }
         s.f[0] = 1.0f / sum;
     }
     __syncthreads();
@@ -239,14 +249,19 @@ __device__ void finish_candidates(SampleShared& s, int n, int top_k, float zmax,
         if (tid == 0) {     // descending order until the mass reaches top_p
             float mass = 0.0f;
             int last = 0;
-            for (; last < m - 1; ++last) {
+            bool reached = false;
+            for (; last < m; ++last) {
                 mass += s.by_rank[last];
-                if (mass >= top_p) break;
+                if (mass >= top_p) { reached = true; break; }
             }
-            s.bcast[0] = (unsigned)last;
+            s.bcast[0] = (unsigned)min(last, m - 1);
+            s.bcast[1] = reached || complete;
         }
         __syncthreads();
         int last = (int)s.bcast[0];
+        bool enough = s.bcast[1] != 0;
+        __syncthreads();
+        if (!enough) return false;
         for (int c = tid; c < n; c += SAMPLE_THREADS)
             if (s.rank[c] > last) s.cand_z[c] = 0.0f;
         __syncthreads();
@@ -270,6 +285,7 @@ __device__ void finish_candidates(SampleShared& s, int n, int top_k, float zmax,
         }
         *result = pick >= 0 ? pick : last_kept;
     }
+    return true;
 }
 
 // Exclusive prefix of v over the block's waves (wave order), and the total; v is a per-wave value.
@@ -352,20 +368,27 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     // Gathers the values with key >= bound (and index <= cut among those equal to `bound`, if
     // cut < V) into LDS in index order; returns how many there are (nothing is written if
     // they do not fit).
-    auto gather = [&](unsigned bound, int cut) -> unsigned {
+    auto gather = [&](unsigned bound, int cut, float* row_mass = nullptr) -> unsigned {
         auto in = [&](int i) { unsigned k = order_key(row[i] * inv_t); return k > bound || (k == bound && i <= cut); };
         auto in_z = [&](float z, int i) { unsigned k = order_key(z); return k > bound || (k == bound && i <= cut); };
         unsigned cnt = 0;
+        float mass = 0.0f;      // with row_mass: the softmax sum of the whole row, in the same pass
         if (vec) {      // (w_lo and w_hi are multiples of 4 here: V is, and the stretches are multiples of 64)
 #pragma unroll 4
             for (int i = w_lo + lane * 4; i < w_hi; i += 256) {
                 float4 v = *(const float4*)(row + i);
-                cnt += in_z(v.x * inv_t, i) + in_z(v.y * inv_t, i + 1) + in_z(v.z * inv_t, i + 2) + in_z(v.w * inv_t, i + 3);
+                float z0 = v.x * inv_t, z1 = v.y * inv_t, z2 = v.z * inv_t, z3 = v.w * inv_t;
+                cnt += in_z(z0, i) + in_z(z1, i + 1) + in_z(z2, i + 2) + in_z(z3, i + 3);
+                if (row_mass) mass += (expf(z0 - zmax) + expf(z1 - zmax)) + (expf(z2 - zmax) + expf(z3 - zmax));
             }
         } else {
 #pragma unroll 8
-            for (int i = w_lo + lane; i < w_hi; i += 64) cnt += in(i);
+            for (int i = w_lo + lane; i < w_hi; i += 64) {
+                cnt += in(i);
+                if (row_mass) mass += expf(row[i] * inv_t - zmax);
+            }
         }
+        if (row_mass) *row_mass = block_sum_f(mass, s);
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, 64);
         unsigned total;
@@ -410,10 +433,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         return total;
     };
 
-    if (use_k && top_k <= SAMPLE_THREADS) {
+    // top_p alone: the values that matter are the largest few hundred in all rows but flat ones.  The 512
+    // largest (and what else is no smaller than the bound below) become candidates; if the top_p mass
+    // is reached inside them, the row is finished there; if not, by the search over the whole row below.
+    bool nucleus_try = !use_k && top_p < 1.0f;
+    if ((use_k && top_k <= SAMPLE_THREADS) || nucleus_try) {
         // ---- a lower bound of the k-th largest value: the k-th largest of the threads' maxima
         unsigned mykey = mine_any ? order_key(mine_max) : 0u;
-        unsigned prefix = 0, mask = 0, remaining = top_k;
+        unsigned prefix = 0, mask = 0, remaining = use_k ? top_k : 512;
         for (int shift = 24; shift >= 0; shift -= 8) {
             for (int b = tid; b < 256; b += SAMPLE_THREADS) s.hist[b] = 0;
             __syncthreads();
@@ -427,10 +454,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
             __syncthreads();
         }
         // at least top_k values of the row have a key >= prefix
-        unsigned n = gather(prefix, V);
+        float row_mass = 0.0f;
+        unsigned n = gather(prefix, V, nucleus_try ? &row_mass : nullptr);
         if (n <= MAX_CAND) {    // the k largest of the candidates, and the rest of the row's work, in LDS
-            finish_candidates(s, (int)n, top_k, zmax, top_p, u, &out[blockIdx.x]);
-            return;
+            if (!nucleus_try) {
+                finish_candidates(s, (int)n, top_k, zmax, top_p, u, &out[blockIdx.x]);
+                return;
+            }
+            if (finish_candidates(s, (int)n, (int)n, zmax, top_p, u, &out[blockIdx.x], row_mass, (int)n == V)) return;
         }
         // too many equal or near values: the general path below handles it
     }
