@@ -22,7 +22,9 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import gc
 import os
+import weakref
 
 import numpy as np
 import torch
@@ -46,7 +48,9 @@ class StepContext:
     """What parts see of the running step.  Device arrays are int32."""
 
     def __init__(self, runner: "StepRunner"):
-        self._runner = runner
+        # (not a reference that counts: runner and context would hold each other, and a dropped engine,
+        # with its recorded graphs and device memory, would wait for the cycle collector)
+        self._runner = weakref.proxy(runner)
         self.n_tokens = 0
         self.n_entries = 0
         self.n_want = 0
@@ -242,9 +246,19 @@ class StepRunner:
         self._seen[key] = self._seen.get(key, 0) + 1
         if self._seen[key] < (2 if ctx.n_tokens <= 64 else 4):
             return self.model.forward(ctx, self.cache.views)     # first times: run it, and let the workspace grow
+        # Nothing may be destroyed on the device while a stream is being recorded: an object that the
+        # cycle collector happened to free in the middle of it (another engine's graphs, say) ended the
+        # process.  What can be collected is collected before, and the collector rests meanwhile.
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = self.model.forward(ctx, self.cache.views)
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ctx, self.cache.views)
+        finally:
+            if was_enabled:
+                gc.enable()
         if key not in self._seen:       # the workspace grew while recording: those addresses are gone
             return self.model.forward(ctx, self.cache.views)
         self._graphs[key] = (graph, logits)
