@@ -17,6 +17,7 @@ struct RopeKvArgs {
     int rotary_dim, interleaved;
     int page_size, write_kv, num_pages;
     int row_stride;  // elements between tokens in qkv
+    int value_pages; // value_pages_kernel runs as well: it writes the values of pages that 16 tokens fill in order
 };
 
 template <class T>
@@ -70,18 +71,70 @@ __global__ void rope_kv_kernel(T* __restrict__ qkv, const int* __restrict__ posi
     }
 }
 
+typedef __bf16 rope_bf16x8 __attribute__((ext_vector_type(8)));
+
+// Values lie transposed in a page ([head_dim][slot]), so a token's values are head_dim scattered
+// 2-byte stores.  Where 16 consecutive tokens of the batch fill one 16-slot page in order (a prompt
+// portion, page after page), that page's values are written by value_pages_kernel instead: through
+// LDS, 16 bytes a lane, whole lines.  Both kernels ask this of the same 16 tokens and get the same
+// answer.  The first 16 lanes of a block's first wave look; the answer is the same in all of them.
+__device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict__ slot_map, int t16, const RopeKvArgs& a) {
+    int j = threadIdx.x & 15;
+    bool mine = false;
+    if (a.page_size == 16 && t16 + 15 < a.n_tokens) {
+        int s0 = slot_map[t16], sj = slot_map[t16 + j];
+        mine = s0 >= 0 && (s0 & 15) == 0 && s0 + 15 < a.num_pages * 16 && sj == s0 + j;
+    }
+    return (__ballot(mine) & 0xffffull) == 0xffffull;
+}
+
+// One block per (16 tokens, kv head): [16 tokens][head_dim] in, [head_dim][16 slots] out.
+__global__ __launch_bounds__(256) void value_pages_kernel(const bf16* __restrict__ qkv, const int* __restrict__ slot_map,
+                                                          bf16* __restrict__ v_cache, RopeKvArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char vp_smem[];
+    __shared__ int whole;
+    int t16 = blockIdx.x * 16, kvh = blockIdx.y, hd = a.head_dim;
+    if (threadIdx.x < 64) {
+        bool w = first_lanes_see_whole_page(slot_map, t16, a);
+        if (threadIdx.x == 0) whole = w;
+    }
+    __syncthreads();
+    if (!whole) return;
+    bf16* tile = (bf16*)vp_smem;                        // [16][hd + 8]: rows 16 bytes apart in banks
+    int ld = hd + 8, chunks = hd / 8;
+    const bf16* src = qkv + (size_t)t16 * a.row_stride + (size_t)(a.n_heads + a.n_kv_heads + kvh) * hd;
+    for (int c = threadIdx.x; c < 16 * chunks; c += blockDim.x) {
+        int j = c / chunks, d0 = (c % chunks) * 8;
+        *(rope_bf16x8*)(tile + j * ld + d0) = *(const rope_bf16x8*)(src + (size_t)j * a.row_stride + d0);
+    }
+    __syncthreads();
+    int page = slot_map[t16] / 16;
+    bf16* dst = v_cache + v_cache_index(page, kvh, 0, 0, a.n_kv_heads, 16, hd);     // this page and head: [hd][16], contiguous
+    for (int c = threadIdx.x; c < hd * 2; c += blockDim.x) {
+        int d = c >> 1, s0 = (c & 1) * 8;
+        rope_bf16x8 v;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = tile[(s0 + j) * ld + d];
+        *(rope_bf16x8*)(dst + d * 16 + s0) = v;
+    }
+}
+
 // The same for 16-bit rows whose pairs are neighbours (2i, 2i+1), eight features to a thread:
 // one block per token works out the token's cos / sin once (they are the same for all of
 // its heads) and then moves 16 bytes per thread and access.  Needs head_dim, rotary_dim and
 // the row stride to be multiples of 8 and 16-byte aligned rows.
-typedef __bf16 rope_bf16x8 __attribute__((ext_vector_type(8)));
 __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qkv, const int* __restrict__ positions,
                                                            const int* __restrict__ slot_map,
                                                            const float* __restrict__ inv_freq,
                                                            bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
                                                            RopeKvArgs a) {
     extern __shared__ float2 cs[];                 // [rotary_dim / 2]: cos, sin of the token's angles
+    __shared__ int values_elsewhere;               // this token's values are written by value_pages_kernel
     int t = blockIdx.x;
+    if (threadIdx.x < 64) {
+        bool w = a.write_kv && a.value_pages && first_lanes_see_whole_page(slot_map, t & ~15, a);
+        if (threadIdx.x == 0) values_elsewhere = w;
+    }
     float pos = (float)positions[t];
     for (int i = threadIdx.x; i < a.rotary_dim / 2; i += blockDim.x) {
         float s, c;
@@ -99,6 +152,7 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
         int head = ch / chunks_per_head, d0 = (ch % chunks_per_head) * 8;
         bool is_q = ch < q_chunks, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
         if (!is_q && !cache_ok) continue;
+        if (!is_q && !is_k && values_elsewhere) continue;
         rope_bf16x8 v = *(const rope_bf16x8*)(row + (size_t)head * a.head_dim + d0);
         if ((is_q || is_k) && d0 < a.rotary_dim) {
 #pragma unroll
@@ -137,15 +191,22 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
     LLMRS_REQUIRE(row_stride >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_kv_write: row stride %d too short", row_stride);
     LLMRS_REQUIRE(page_size > 0, "rope_kv_write: page_size %d", page_size);
     if (n_tokens == 0) return 0;
-    RopeKvArgs a{n_tokens, n_heads, n_kv_heads, head_dim, rotary_dim, interleaved, page_size, write_kv, num_pages, row_stride};
+    RopeKvArgs a{n_tokens, n_heads, n_kv_heads, head_dim, rotary_dim, interleaved, page_size, write_kv, num_pages, row_stride, 0};
     int pairs = (n_heads + 2 * n_kv_heads) * (head_dim / 2);
     dim3 grid(n_tokens, ceil_div(pairs, 256));
     if (dtype == LLMRS_F32)
         rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, positions, slot_map, inv_freq, (float*)k_cache, (float*)v_cache, a);
     else if (dtype == LLMRS_BF16 && interleaved && n_tokens >= 16 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0 &&
              ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && rotary_dim / 2 * sizeof(float2) <= 32768)
+    {
+        a.value_pages = write_kv && page_size == 16 && n_kv_heads > 0 && ((uintptr_t)v_cache & 15) == 0 &&
+                        (size_t)16 * (head_dim + 8) * 2 <= 65536;
         rope_kv_rows_kernel<<<n_tokens, 256, rotary_dim / 2 * sizeof(float2), stream>>>((bf16*)qkv, positions, slot_map, inv_freq,
                                                                                         (bf16*)k_cache, (bf16*)v_cache, a);
+        if (a.value_pages)
+            value_pages_kernel<<<dim3(n_tokens / 16, n_kv_heads), 256, (size_t)16 * (head_dim + 8) * 2, stream>>>(
+                (const bf16*)qkv, slot_map, (bf16*)v_cache, a);
+    }
     else if (dtype == LLMRS_BF16)
         rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
     else

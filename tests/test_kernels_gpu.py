@@ -146,7 +146,16 @@ def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, 
     before = qkv.clone()
     positions = torch.tensor([0, 1, 2, 3, 40, 41, 5, 6, 7, 300, 301] * repeat, dtype=torch.int32, device=DEV)
     positions = positions + 13 * torch.arange(T, dtype=torch.int32, device=DEV) // 11
-    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(9))[:T].to(torch.int32).to(DEV)
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(9))[:T]
+    if repeat > 1 and page_size == 16:
+        # groups of 16 tokens that fill a page in order (their values are written by the kernel that
+        # transposes whole pages), and one that does so but for two tokens in each other's places
+        taken = [3, 1, 5]
+        rest = [int(x) for x in slots if int(x) // 16 not in taken]
+        run = lambda pg: [pg * 16 + j for j in range(16)]
+        swapped = run(5); swapped[4], swapped[9] = swapped[9], swapped[4]
+        slots = torch.tensor((run(3) + run(1) + swapped + rest)[:T])
+    slots = slots.to(torch.int32).to(DEV)
     inv_freq = plain_inv_freq(rot, theta, scaling).to(DEV)
     kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=dtype, device=DEV)
     vc = torch.zeros((num_pages, n_kv, hd, page_size), dtype=dtype, device=DEV)
@@ -170,7 +179,8 @@ def _rope_case(dtype, n_heads, n_kv, hd, rot, layout, page_size, theta=10000.0, 
     written = torch.zeros(num_pages * page_size, dtype=torch.bool)
     written[slots.long().cpu()] = True
     kflat = kc.cpu().permute(0, 2, 1, 3).reshape(num_pages * page_size, -1)
-    assert (kflat[~written] == 0).all(), "a slot that no token maps to was written"
+    vflat = vc.cpu().permute(0, 3, 1, 2).reshape(num_pages * page_size, -1)
+    assert (kflat[~written] == 0).all() and (vflat[~written] == 0).all(), "a slot that no token maps to was written"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
