@@ -296,3 +296,26 @@ def test_bfloat16_under_preemption_follows_float32():
         chosen = logits[torch.arange(len(o)), torch.tensor(o, device=logits.device)]
         gap = float((logits.max(dim=1).values - chosen).max()) / scale
         assert gap <= 2 * TOLERANCE["bfloat16"], f"request {i}: a chosen token lies {gap:.3e} of the logit scale below the float32 choice"
+
+
+def test_a_dropped_engine_is_freed_at_once(folders):
+    """No cycle of references holds an engine: when the last name for it goes, its device memory and its
+    recorded graphs go too, without the cycle collector (which may run at any moment, and must not find
+    such things to destroy while another engine records a graph)."""
+    import gc
+    import weakref
+    gc.collect()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    gc.disable()
+    try:
+        eng = engine(folders["B"], "B", "bfloat16")
+        eng.generate([[1, 2, 3, 4, 5]], max_new_tokens=12)
+        assert eng.runner.graph_replays > 0, "the case must have recorded a graph"
+        gone = [weakref.ref(eng), weakref.ref(eng.runner), weakref.ref(eng.cache), weakref.ref(eng.model)]
+        del eng
+        assert all(r() is None for r in gone)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() <= before
+    finally:
+        gc.enable()
