@@ -19,6 +19,7 @@ width's capacity and leave early.
 """
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -88,7 +89,8 @@ class StepRunner:
         self.use_graphs = (self._pinned and os.environ.get("LLMRS_GRAPHS", "1") != "0" and not cache.state_tensors
                            and bool(getattr(model, "graph_safe", lambda: False)()))
         self.max_graph_batch = 512
-        self._graphs: Dict[tuple, tuple] = {}
+        self.max_graphs = 256            # recorded graphs kept (the least recently replayed goes first)
+        self._graphs: "OrderedDict[tuple, tuple]" = OrderedDict()
         self._seen: Dict[tuple, int] = {}
         self.graph_replays = 0
 
@@ -238,6 +240,7 @@ class StepRunner:
         key = (ctx.n_tokens, ctx.n_want, tuple(graph_widths), self._dev_words.data_ptr())
         hit = self._graphs.get(key)
         if hit is not None:
+            self._graphs.move_to_end(key)
             hit[0].replay()
             self.graph_replays += 1
             return hit[1]
@@ -261,6 +264,8 @@ class StepRunner:
                 gc.enable()
         if key not in self._seen:       # the workspace grew while recording: those addresses are gone
             return self.model.forward(ctx, self.cache.views)
+        while len(self._graphs) >= self.max_graphs:
+            self._graphs.popitem(last=False)
         self._graphs[key] = (graph, logits)
         graph.replay()                  # recording does not run the kernels
         self.graph_replays += 1

@@ -319,3 +319,30 @@ def test_a_dropped_engine_is_freed_at_once(folders):
         assert torch.cuda.memory_allocated() <= before
     finally:
         gc.enable()
+
+
+def test_only_so_many_recorded_graphs_are_kept(folders):
+    """More batch shapes than graphs may be kept: the least recently replayed one goes, comes back by being
+    recorded again, and every step still equals the eager engine's."""
+    which, dtype = "B", "bfloat16"
+    cfg, _ = read_model_folder(folders[which])
+    recorded, eager = engine(folders[which], which, dtype), engine(folders[which], which, dtype)
+    eager.runner.use_graphs = False
+    recorded.runner.max_graphs = 2
+    seqs = [random_tokens(cfg["vocab_size"], 100, seed=600 + i) for i in range(4)]
+    sr, se = [recorded.open_request() for _ in seqs], [eager.open_request() for _ in seqs]
+    for i, seq in enumerate(seqs):
+        for eng, sl in ((recorded, sr), (eager, se)):
+            eng.step([StepEntry(sl[i], 0, seq[:10], [])])
+    pos = [10] * 4
+    for turn in range(6):
+        for n in (4, 3, 2, 1):                       # four shapes, each seen three times in a row
+            for _ in range(3):
+                a = recorded.step([StepEntry(sr[i], pos[i], [seqs[i][pos[i]]], [0]) for i in range(n)]).clone()
+                b = eager.step([StepEntry(se[i], pos[i], [seqs[i][pos[i]]], [0]) for i in range(n)]).clone()
+                torch.cuda.synchronize()
+                assert torch.equal(a, b)
+                for i in range(n):
+                    pos[i] += 1
+            assert len(recorded.runner._graphs) <= 2
+    assert recorded.runner.graph_replays > 20
