@@ -58,29 +58,12 @@ class _Submitted:
     stop: Sequence[int]
 
 
-_collector_quiet = False
-
-
-def _quiet_collector() -> None:
-    """Once per process, before the first engine makes anything of its own: what exists by then
-    (the libraries' modules) lives as long as the process and is taken out of the collector's
-    sight, so that a full collection, when one falls into a run of steps, does not hold the host
-    for the 40 ms that walking all of it took (measured: one such pause among the first 30
-    decode steps of a process).  No engine's own objects are frozen: they can still be collected."""
-    global _collector_quiet
-    if not _collector_quiet:
-        gc.collect()
-        gc.freeze()
-        _collector_quiet = True
-
-
 class Engine:
     def __init__(self, config, tensors: Mapping[str, torch.Tensor], *, dtype="bfloat16", device="cuda",
                  page_size: int = 16, num_pages=None, kv_memory_fraction: float = 0.8, max_requests: int = 256,
                  max_batch_tokens: int = 2048, max_chunk: int = 0, max_seq_len: Optional[int] = None, log: bool = False):
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
-        _quiet_collector()
         self.config = config
         self.dtype = _DTYPES[dtype]
         self.device = torch.device(device)
@@ -106,6 +89,10 @@ class Engine:
         self._request_of: Dict[int, int] = {}              # slot -> request, for those the scheduler holds
         self._samples_randomly: set = set()                 # of those, the slots that do not decode greedily
         self._steps = 0
+        # A full collection now, while nothing waits for it: building the model has made so many
+        # objects that the collector would otherwise choose a moment among the first decode steps to
+        # walk everything the libraries hold (measured: one pause of 40 ms there).
+        gc.collect()
         if log:
             for g, grp in enumerate(self.cache.groups):
                 gb = grp.num_pages * page_size * grp.bytes_per_token() / 1e9

@@ -251,9 +251,8 @@ class StepRunner:
             return self.model.forward(ctx, self.cache.views)     # first times: run it, and let the workspace grow
         # Nothing may be destroyed on the device while a stream is being recorded: an object that the
         # cycle collector happened to free in the middle of it (another engine's graphs, say) ended the
-        # process.  What can be collected is collected before, and the collector rests meanwhile.
+        # process.  The collector rests meanwhile.
         graph = torch.cuda.CUDAGraph()
-        gc.collect()
         was_enabled = gc.isenabled()
         gc.disable()
         try:
