@@ -67,7 +67,20 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 // Lanes stride over k, four elements at a time, and each keeps one 32-bit sum per token and
 // row; the lanes' sums are added by a butterfly.  The order depends on K only.
 #define GEMV_MAX_M 8
-template <class T>
+// Four consecutive elements as 32-bit values: one 16-byte (float) or 8-byte (bfloat16) load.
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    float4 t = *(const float4*)p;
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    bf16x4_t t = *(const bf16x4_t*)p;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (float)t[j];
+}
+// VEC: K % 4 == 0 and every row starts on a multiple of four elements' size, so a lane's four
+// elements come in one load and none of them lies past K.  The sums are the same either way.
+template <class T, bool VEC>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W,
                                                         void* __restrict__ out, int ldc, int M, int N, int K, int epi) {
     int lane = threadIdx.x & 63;
@@ -79,21 +92,32 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A,
     float acc0[GEMV_MAX_M] = {}, acc1[GEMV_MAX_M] = {};
     for (int k = lane * 4; k < K; k += 256) {
         float a[4], b[4];
+        if constexpr (VEC) {
+            load4(w0 + k, a);
+            load4(w1 + k, b);
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            bool in = k + j < K;
-            a[j] = in ? to_f32(w0[k + j]) : 0.0f;
-            b[j] = in ? to_f32(w1[k + j]) : 0.0f;
+            for (int j = 0; j < 4; ++j) {
+                bool in = k + j < K;
+                a[j] = in ? to_f32(w0[k + j]) : 0.0f;
+                b[j] = in ? to_f32(w1[k + j]) : 0.0f;
+            }
         }
 #pragma unroll
         for (int m = 0; m < GEMV_MAX_M; ++m) {
             if (m >= M) break;
             const T* x = A + (size_t)m * lda + k;
+            float xv[4];
+            if constexpr (VEC) {
+                load4(x, xv);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xv[j] = k + j < K ? to_f32(x[j]) : 0.0f;
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                float xv = k + j < K ? to_f32(x[j]) : 0.0f;
-                acc0[m] = fmaf(a[j], xv, acc0[m]);
-                acc1[m] = fmaf(b[j], xv, acc1[m]);
+                acc0[m] = fmaf(a[j], xv[j], acc0[m]);
+                acc1[m] = fmaf(b[j], xv[j], acc1[m]);
             }
         }
     }
@@ -133,12 +157,13 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
     }
     if (M <= GEMV_MAX_M) {
         int blocks = ceil_div(N, 8);
-        if (dtype == LLMRS_F32)
-            gemm_rows_kernel<float><<<blocks, 256, 0, stream>>>((const float*)A, lda, (const float*)W, out, ldc, M, N, K, epi);
-        else if (dtype == LLMRS_BF16)
-            gemm_rows_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
-        else
-            return llmrs_fail("gemm: unknown dtype %d", dtype);
+        size_t elt = dtype == LLMRS_F32 ? sizeof(float) : sizeof(bf16);
+        bool vec = K % 4 == 0 && lda % 4 == 0 && (uintptr_t)A % (4 * elt) == 0 && (uintptr_t)W % (4 * elt) == 0;
+#define ROWS(T, V) gemm_rows_kernel<T, V><<<blocks, 256, 0, stream>>>((const T*)A, lda, (const T*)W, out, ldc, M, N, K, epi)
+        if (dtype == LLMRS_F32) { if (vec) ROWS(float, true); else ROWS(float, false); }
+        else if (dtype == LLMRS_BF16) { if (vec) ROWS(bf16, true); else ROWS(bf16, false); }
+        else return llmrs_fail("gemm: unknown dtype %d", dtype);
+#undef ROWS
         LLMRS_LAUNCH_CHECK("gemm");
         return 0;
     }
