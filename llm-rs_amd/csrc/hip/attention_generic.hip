@@ -8,33 +8,29 @@
 // bound.  This is the reference's paged_attention (shaders/ops.metal:636-758;
 // causal_len of :673-674 equals p + 1) with a tile of 64 keys, one per lane.
 // Tiles start at lo, so for a given query the order of every sum is fixed: it
-// does not depend on the batch or on how the prompt was cut.
+// does not depend on the batch or on how the prompt was cut.  A decoding request's
+// keys are shared out over waves in chunks aligned to absolute positions and the
+// chunks added in ascending order, which is another fixed order.
 #include "attention.h"
 #include "cache_layout.h"
 
 #define MAX_HEAD_DIM 512
 
-template <class T>
-__global__ __launch_bounds__(64) void attention_generic_kernel(
-    const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const int* __restrict__ block_table, const int* __restrict__ token_entry, const int* __restrict__ positions,
-    AttnArgs a) {
-    __shared__ float qs[MAX_HEAD_DIM];
-    int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    int hd = a.head_dim, ps = a.page_size;
-    int kvh = h / (a.n_heads / a.n_kv_heads);
-    int pos = positions[t];
-    const int* table = block_table + (size_t)token_entry[t] * a.table_width;
-    const T* qrow = q + (size_t)t * a.q_stride + (size_t)h * hd;
-    for (int d = lane; d < hd; d += 64) qs[d] = to_f32(qrow[d]);
-    __syncthreads();
+// Keys of a single-token entry that one wave of the split takes (aligned to absolute positions).
+#define GENERIC_CHUNK 128
 
-    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-    float m = -INFINITY, l = 0.0f;
-    float acc[MAX_HEAD_DIM / 64] = {};
-    for (int t0 = lo; t0 <= pos; t0 += 64) {
+// One wave walks the keys [begin, end) of its request for the query in `qs`, a tile of 64 keys at a
+// time (one key per lane), and folds them into the running maximum m, sum l and acc (lane's
+// features d = lane + 64 i, not yet divided by l).  VEC: head_dim % 4 == 0, a key's row is read four
+// elements at a load; the sums are the same either way.
+template <class T, bool VEC>
+__device__ __forceinline__ void walk_keys(const float* qs, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                          const int* __restrict__ table, const AttnArgs& a, int kvh, int begin, int end,
+                                          float& m, float& l, float (&acc)[MAX_HEAD_DIM / 64]) {
+    int lane = threadIdx.x, hd = a.head_dim, ps = a.page_size;
+    for (int t0 = begin; t0 < end; t0 += 64) {
         int j = t0 + lane;
-        bool valid = j <= pos;
+        bool valid = j < end;
         int page = 0, off = 0;
         float s = -INFINITY;
         if (valid) {
@@ -43,7 +39,16 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             off = j % ps;
             const T* kp = k_cache + k_cache_index(page, kvh, off, 0, a.n_kv_heads, ps, hd);
             float dot = 0.0f;
-            for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kp[d]), dot);
+            if constexpr (VEC) {
+                for (int d = 0; d < hd; d += 4) {
+                    float kv[4];
+                    load4(kp + d, kv);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) dot = fmaf(qs[d + i], kv[i], dot);
+                }
+            } else {
+                for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_f32(kp[d]), dot);
+            }
             s = dot * a.scale;
         }
         float m_new = fmaxf(m, wave_max(s));
@@ -53,7 +58,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         m = m_new;
 #pragma unroll
         for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) acc[i] *= rescale;
-        int n_valid = min(64, pos - t0 + 1);
+        int n_valid = min(64, end - t0);
         for (int jj = 0; jj < n_valid; ++jj) {
             float pj = __shfl(p, jj, 64);
             int pagej = __shfl(page, jj, 64), offj = __shfl(off, jj, 64);
@@ -65,12 +70,139 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             }
         }
     }
+}
+
+// skip_single: tokens of entries that bring one token are left to the split kernels below.
+template <class T, bool VEC>
+__global__ __launch_bounds__(64) void attention_generic_kernel(
+    const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ token_entry, const int* __restrict__ positions,
+    const int* __restrict__ q_starts, int skip_single, AttnArgs a) {
+    __shared__ float qs[MAX_HEAD_DIM];
+    int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    int hd = a.head_dim;
+    int kvh = h / (a.n_heads / a.n_kv_heads);
+    int e = token_entry[t];
+    if (skip_single && q_starts[e + 1] - q_starts[e] == 1) return;
+    int pos = positions[t];
+    const int* table = block_table + (size_t)e * a.table_width;
+    const T* qrow = q + (size_t)t * a.q_stride + (size_t)h * hd;
+    for (int d = lane; d < hd; d += 64) qs[d] = to_f32(qrow[d]);
+    __syncthreads();
+
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    float m = -INFINITY, l = 0.0f;
+    float acc[MAX_HEAD_DIM / 64] = {};
+    walk_keys<T, VEC>(qs, k_cache, v_cache, table, a, kvh, lo, pos + 1, m, l, acc);
     T* orow = out + (size_t)t * a.out_stride + (size_t)h * hd;
 #pragma unroll
     for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
         int d = lane + 64 * i;
         if (d < hd) orow[d] = from_f32<T>(acc[i] / l);
     }
+}
+
+// Entries with one token (decoding): a wave for each (entry, head, chunk of GENERIC_CHUNK keys), so
+// that a long context is read by many waves at once.  Chunks are aligned to absolute positions.
+// partial: [(entry * n_heads + head) * max_chunks + chunk][head_dim + 2] = m, l, acc (not divided).
+template <class T, bool VEC>
+__global__ __launch_bounds__(64) void attention_generic_split_kernel(
+    const T* __restrict__ q, float* __restrict__ partial, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ q_starts, const int* __restrict__ seq_lens,
+    int max_chunks, AttnArgs a) {
+    __shared__ float qs[MAX_HEAD_DIM];
+    int e = blockIdx.x, h = blockIdx.y, ch = blockIdx.z, lane = threadIdx.x;
+    int t = q_starts[e];
+    if (q_starts[e + 1] - t != 1) return;
+    int pos = seq_lens[e] - 1;                    // an entry with one token: its position is its length less one
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int first = lo / GENERIC_CHUNK;
+    if (ch > pos / GENERIC_CHUNK - first) return;
+    int begin = max(lo, (first + ch) * GENERIC_CHUNK), end = min(pos + 1, (first + ch + 1) * GENERIC_CHUNK);
+    int hd = a.head_dim;
+    int kvh = h / (a.n_heads / a.n_kv_heads);
+    const T* qrow = q + (size_t)t * a.q_stride + (size_t)h * hd;
+    for (int d = lane; d < hd; d += 64) qs[d] = to_f32(qrow[d]);
+    __syncthreads();
+    float m = -INFINITY, l = 0.0f;
+    float acc[MAX_HEAD_DIM / 64] = {};
+    walk_keys<T, VEC>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, begin, end, m, l, acc);
+    float* pp = partial + ((size_t)(e * a.n_heads + h) * max_chunks + ch) * (hd + 2);
+    if (lane == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+    for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
+        int d = lane + 64 * i;
+        if (d < hd) pp[2 + d] = acc[i];
+    }
+}
+
+// One wave for each (entry, head) adds the chunks up, in ascending order.
+template <class T>
+__global__ __launch_bounds__(64) void attention_generic_merge_kernel(
+    const float* __restrict__ partial, T* __restrict__ out, const int* __restrict__ q_starts,
+    const int* __restrict__ seq_lens, int max_chunks, AttnArgs a) {
+    int e = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, hd = a.head_dim;
+    int t = q_starts[e];
+    if (q_starts[e + 1] - t != 1) return;
+    int pos = seq_lens[e] - 1;
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int n_chunks = pos / GENERIC_CHUNK - lo / GENERIC_CHUNK + 1;
+    const float* pp = partial + (size_t)(e * a.n_heads + h) * max_chunks * (hd + 2);
+    int stride = hd + 2;
+    float M = -INFINITY;
+    for (int ch = 0; ch < n_chunks; ++ch) M = fmaxf(M, pp[(size_t)ch * stride]);
+    float L = 0.0f;
+    float o[MAX_HEAD_DIM / 64] = {};
+    for (int ch = 0; ch < n_chunks; ++ch) {
+        float w = expf(pp[(size_t)ch * stride] - M);
+        L = fmaf(pp[(size_t)ch * stride + 1], w, L);
+#pragma unroll
+        for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
+            int d = lane + 64 * i;
+            if (d < hd) o[i] = fmaf(pp[(size_t)ch * stride + 2 + d], w, o[i]);
+        }
+    }
+    T* orow = out + (size_t)t * a.out_stride + (size_t)h * hd;
+#pragma unroll
+    for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
+        int d = lane + 64 * i;
+        if (d < hd) orow[d] = from_f32<T>(o[i] / L);
+    }
+}
+
+template <class T>
+static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cache, const T* v_cache,
+                          const int* block_table, const int* token_entry, const int* positions, const int* q_starts,
+                          const int* seq_lens, int n_entries, float* scratch, size_t scratch_bytes, int max_seq_len,
+                          int n_single, const AttnArgs& a) {
+    bool vec = a.head_dim % 4 == 0 && (uintptr_t)k_cache % (4 * sizeof(T)) == 0;
+    // Single-token entries are split by key range when the caller gave room for the partial results.
+    int max_chunks = max_seq_len > 0 ? ceil_div(max_seq_len, GENERIC_CHUNK) : 0;
+    size_t need = (size_t)n_entries * a.n_heads * max_chunks * (a.head_dim + 2) * sizeof(float);
+    bool split = max_chunks > 0 && scratch != nullptr && q_starts != nullptr && seq_lens != nullptr &&
+                 scratch_bytes >= need && n_single != 0 && n_entries <= 65535 && max_chunks <= 65535;
+    bool only_single = split && a.n_tokens == n_entries;     // every entry brings one token
+    if (!only_single) {
+        dim3 grid(a.n_tokens, a.n_heads);
+        if (vec)
+            attention_generic_kernel<T, true><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
+                                                                    positions, q_starts, split, a);
+        else
+            attention_generic_kernel<T, false><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
+                                                                     positions, q_starts, split, a);
+    }
+    if (split) {
+        dim3 grid(n_entries, a.n_heads, max_chunks);
+        if (vec)
+            attention_generic_split_kernel<T, true><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
+                                                                          q_starts, seq_lens, max_chunks, a);
+        else
+            attention_generic_split_kernel<T, false><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
+                                                                           q_starts, seq_lens, max_chunks, a);
+        attention_generic_merge_kernel<T><<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, q_starts, seq_lens,
+                                                                                        max_chunks, a);
+    }
+    return 0;
 }
 
 // q: [n_tokens, q_stride] (head h at h*head_dim); out: [n_tokens, out_stride];
@@ -101,13 +233,14 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
                                              (float*)scratch, scratch_bytes, max_seq_len, n_single, a);
         if (took != 0) return took < 0 ? -1 : 0;
     }
-    dim3 grid(n_tokens, n_heads);
     if (dtype == LLMRS_F32)
-        attention_generic_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, (float*)out, (const float*)k_cache,
-                                                                 (const float*)v_cache, block_table, token_entry, positions, a);
+        launch_generic<float>(stream, (const float*)q, (float*)out, (const float*)k_cache, (const float*)v_cache, block_table,
+                              token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
+                              max_seq_len, n_single, a);
     else if (dtype == LLMRS_BF16)
-        attention_generic_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)q, (bf16*)out, (const bf16*)k_cache,
-                                                                (const bf16*)v_cache, block_table, token_entry, positions, a);
+        launch_generic<bf16>(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
+                             token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
+                             max_seq_len, n_single, a);
     else
         return llmrs_fail("attention: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("attention");

@@ -33,6 +33,18 @@ __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 template <class T>
 __device__ __forceinline__ T from_f32(float x) { return (T)x; }
 
+// Four consecutive elements as 32-bit values: one 16-byte (float) or 8-byte (bfloat16) load.
+__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    float4 t = *(const float4*)p;
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    bf16x4_t t = *(const bf16x4_t*)p;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = (float)t[j];
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

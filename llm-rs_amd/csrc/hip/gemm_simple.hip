@@ -67,17 +67,6 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 // Lanes stride over k, four elements at a time, and each keeps one 32-bit sum per token and
 // row; the lanes' sums are added by a butterfly.  The order depends on K only.
 #define GEMV_MAX_M 8
-// Four consecutive elements as 32-bit values: one 16-byte (float) or 8-byte (bfloat16) load.
-__device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
-    float4 t = *(const float4*)p;
-    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
-}
-__device__ __forceinline__ void load4(const bf16* p, float (&v)[4]) {
-    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
-    bf16x4_t t = *(const bf16x4_t*)p;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = (float)t[j];
-}
 // VEC: K % 4 == 0 and every row starts on a multiple of four elements' size, so a lane's four
 // elements come in one load and none of them lies past K.  The sums are the same either way.
 template <class T, bool VEC>

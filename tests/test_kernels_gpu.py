@@ -329,6 +329,41 @@ def test_attention_many_decoding_requests(n_req, window):
         assert (got[r].float() - want).abs().max() < 0.07, f"request {r} of length {lens[r]}, key {fars[r]}"
 
 
+@pytest.mark.parametrize("window", [0, 200])
+@pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.float32, 4, 2, 64, 16), (torch.float32, 3, 1, 20, 4),
+                                                     (torch.bfloat16, 6, 3, 48, 8), (torch.bfloat16, 5, 5, 80, 16),
+                                                     (torch.float32, 2, 2, 18, 4)])
+def test_attention_plain_kernel_splits_decoding_requests(dtype, n_heads, n_kv, hd, ps, window):
+    """Head and page sizes (and the 32-bit type) that the matrix-core kernels do not take: decoding
+    requests are shared out over waves in chunks of 128 keys and merged; a prompt portion rides in
+    the same call.  Each decoding query matches one key strongly, at the edges of chunks and of the
+    window: the output must be that key's value, and agree with the plain implementation."""
+    g = torch.Generator().manual_seed(hd + window)
+    lens = [1, 127, 128, 129, 256, 257, 700, 90]
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=hd)
+    edges = [0, 63, 64, 127, 128, 255, 256, 383, 384, 511, 512, 639, 640]
+    qs, pos, fars = [], [], []
+    for r, n in enumerate(lens[:-1]):
+        lo = max(0, n - window) if window else 0
+        seen = [e for e in edges + [lo, lo + 1, n - 1] if lo <= e < n]
+        far = seen[(3 * r + 1) % len(seen)]
+        fars.append(far)
+        qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 6.0).unsqueeze(0).to(dtype))
+        pos.append([n - 1])
+    qs.append(torch.randn((30, n_heads, hd), generator=g).to(dtype))       # a prompt portion of the last request
+    pos.append(list(range(60, 90)))
+    got = case.run(qs, pos, window=window)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    for r in range(len(lens) - 1):
+        ref = case.reference(r, qs[r], pos[r], window=window)[0].float()
+        assert (got[r].float() - ref).abs().max() <= tol, f"request of length {lens[r]}, key {fars[r]}"
+        if lens[r] > 1 and hd >= 48:        # (short heads cannot make one key stand out among hundreds)
+            want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
+            assert (ref - want).abs().max() < 0.1, "the case itself"
+    ref = case.reference(len(lens) - 1, qs[-1], pos[-1], window=window).float()
+    assert (got[len(lens) - 1:].float() - ref).abs().max() <= tol
+
+
 @pytest.mark.parametrize("hd", [64, 96, 128, 256])
 def test_attention_prompt_portion_finds_far_keys(hd):
     """A portion of a prompt far into a long sequence (page numbers are fetched 64 at a time, tiles
