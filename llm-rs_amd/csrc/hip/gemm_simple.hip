@@ -68,28 +68,28 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 // row; the lanes' sums are added by a butterfly.  The order depends on K only.
 #define GEMV_MAX_M 8
 // VEC: K % 4 == 0 and every row starts on a multiple of four elements' size, so a lane's four
-// elements come in one load and none of them lies past K.  The sums are the same either way.
-template <class T, bool VEC>
+// elements come in one load and none of them lies past K.  RW weight rows per wave (even): the
+// tokens' rows are read once for all of them.  The sums are the same whatever VEC and RW are.
+template <class T, bool VEC, int RW>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A, int lda, const T* __restrict__ W,
                                                         void* __restrict__ out, int ldc, int M, int N, int K, int epi) {
     int lane = threadIdx.x & 63;
-    int n = 2 * (blockIdx.x * 4 + (threadIdx.x >> 6));
+    int n = RW * (blockIdx.x * 4 + (threadIdx.x >> 6));
     if (n >= N) return;
-    bool two = n + 1 < N;
-    const T* w0 = W + (size_t)n * K;
-    const T* w1 = W + (size_t)(two ? n + 1 : n) * K;
-    float acc0[GEMV_MAX_M] = {}, acc1[GEMV_MAX_M] = {};
-    for (int k = lane * 4; k < K; k += 256) {
-        float a[4], b[4];
-        if constexpr (VEC) {
-            load4(w0 + k, a);
-            load4(w1 + k, b);
-        } else {
+    const T* w[RW];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                bool in = k + j < K;
-                a[j] = in ? to_f32(w0[k + j]) : 0.0f;
-                b[j] = in ? to_f32(w1[k + j]) : 0.0f;
+    for (int r = 0; r < RW; ++r) w[r] = W + (size_t)min(n + r, N - 1) * K;
+    float acc[RW][GEMV_MAX_M] = {};
+#pragma unroll 2
+    for (int k = lane * 4; k < K; k += 256) {
+        float a[RW][4];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            if constexpr (VEC) {
+                load4(w[r] + k, a[r]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) a[r][j] = k + j < K ? to_f32(w[r][k + j]) : 0.0f;
             }
         }
 #pragma unroll
@@ -104,22 +104,26 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A,
                 for (int j = 0; j < 4; ++j) xv[j] = k + j < K ? to_f32(x[j]) : 0.0f;
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                acc0[m] = fmaf(a[j], xv[j], acc0[m]);
-                acc1[m] = fmaf(b[j], xv[j], acc1[m]);
-            }
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < RW; ++r) acc[r][m] = fmaf(a[r][j], xv[j], acc[r][m]);
         }
     }
 #pragma unroll
     for (int m = 0; m < GEMV_MAX_M; ++m) {
         if (m >= M) break;
-        float v0 = wave_sum(acc0[m]), v1 = wave_sum(acc1[m]);
+        float v[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) v[r] = wave_sum(acc[r][m]);
         if (lane != 0) continue;
-        if (epi == LLMRS_EPI_SWIGLU) {
-            if (two) ((T*)out)[(size_t)m * ldc + n / 2] = from_f32<T>(silu_f32(v0) * v1);
-        } else {
-            epilogue_store<T>(epi, out, ldc, m, n, v0);
-            if (two) epilogue_store<T>(epi, out, ldc, m, n + 1, v1);
+#pragma unroll
+        for (int r = 0; r < RW; r += 2) {
+            if (epi == LLMRS_EPI_SWIGLU) {
+                if (n + r + 1 < N) ((T*)out)[(size_t)m * ldc + (n + r) / 2] = from_f32<T>(silu_f32(v[r]) * v[r + 1]);
+            } else {
+                if (n + r < N) epilogue_store<T>(epi, out, ldc, m, n + r, v[r]);
+                if (n + r + 1 < N) epilogue_store<T>(epi, out, ldc, m, n + r + 1, v[r + 1]);
+            }
         }
     }
 }
@@ -145,10 +149,15 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
         if (took != 0) return took < 0 ? -1 : 0;
     }
     if (M <= GEMV_MAX_M) {
-        int blocks = ceil_div(N, 8);
         size_t elt = dtype == LLMRS_F32 ? sizeof(float) : sizeof(bf16);
         bool vec = K % 4 == 0 && lda % 4 == 0 && (uintptr_t)A % (4 * elt) == 0 && (uintptr_t)W % (4 * elt) == 0;
-#define ROWS(T, V) gemm_rows_kernel<T, V><<<blocks, 256, 0, stream>>>((const T*)A, lda, (const T*)W, out, ldc, M, N, K, epi)
+        // four weight rows per wave once several tokens share them, if that leaves six waves or more
+        // for each compute unit (measured in 32-bit at 8 tokens: 28672 x 4096 130 -> 100 us; 4096 rows are
+        // better off with two, 49 against 56 us)
+        bool four = M > 2 && N >= 24 * llmrs_compute_units();
+        int blocks = ceil_div(N, four ? 16 : 8);
+#define ROWS(T, V) do { if (four) gemm_rows_kernel<T, V, 4><<<blocks, 256, 0, stream>>>((const T*)A, lda, (const T*)W, out, ldc, M, N, K, epi); \
+                        else gemm_rows_kernel<T, V, 2><<<blocks, 256, 0, stream>>>((const T*)A, lda, (const T*)W, out, ldc, M, N, K, epi); } while (0)
         if (dtype == LLMRS_F32) { if (vec) ROWS(float, true); else ROWS(float, false); }
         else if (dtype == LLMRS_BF16) { if (vec) ROWS(bf16, true); else ROWS(bf16, false); }
         else return llmrs_fail("gemm: unknown dtype %d", dtype);
