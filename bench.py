@@ -143,11 +143,12 @@ def main() -> int:
     cache_bytes = args.batch * (args.context + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
     achieved = (weight_bytes + cache_bytes) / step_s
     value = args.batch / step_s
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
     line = {
-        "metric": "decode tok/s at batch 8 (8B bf16); prefill tok/s at 2048 tokens and batch 1/64 alongside",
+        "metric": f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens and batch {'/'.join(str(p) for p in points)} alongside",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, uniform random token ids)",
+        "dtype": short, "data": "synthetic (random weights, uniform random token ids)",
         "config": {"model": "Llama-3.1-8B shape", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single GPU", "layers_run": L, "layers_of_config": full_layers,
                    "hidden_size": D, "num_attention_heads": config.num_attention_heads,
