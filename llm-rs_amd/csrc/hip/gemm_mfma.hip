@@ -623,8 +623,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         // the next tile must have landed before anybody reads it; later tiles may still be on their way
+        // (a bare barrier: __syncthreads() would wait for every load in flight, the later tiles' too)
         if (kt + STAGES - 1 < nk) wait_vmcnt<(STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
-        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0xc07f);                     // lgkmcnt(0): this wave has read what it needs of the tile
+        __builtin_amdgcn_s_barrier();
     }
 
     tile_epilogue<BM, BN, WGM, WGN, STAGES * STAGE_BYTES>(acc, dma_smem, out, ldc, M, N, epi, partial, m0, n0);
