@@ -815,14 +815,30 @@ static int skinny_splits(int N, int K) {
     while (blocks <= 64 && blocks * splits < 256 && splits < 16 && nkb / (splits * 2) >= 8) splits *= 2;
     return splits;
 }
-// Above (128 x 128 tiles, two to a compute unit): until the tiles fill the 512 places, each part at
-// least 8 k-tiles long.
+// Up to 256 rows whose 128 x 128 tiles are no more than the compute units: one block of eight waves per
+// unit with four k-tiles in LDS (three on their way) instead of two blocks of four waves with two
+// k-tiles each.  A tile's loads into LDS take longer than its MFMAs, and with few blocks per unit
+// the deeper pipeline is what keeps them coming (measured, 128 rows at the 8B shapes: qkv 21.9 -> 19.7 us,
+// o 21.3 -> 18.6, gate/up 76.6 -> 64.8, down 43.7 -> 36.6; 256 rows: o 25.8 -> 21.9, down 56.4 -> 50.9;
+// with more tiles than units, or more rows, the two blocks win).
+static bool deep_tiles(int M, int N, int K) {
+    return K % 64 == 0 && M <= 256 && (long)ceil_div(M, 128) * ceil_div(N, 128) <= llmrs_compute_units();
+}
+// Above (128 x 128 tiles): until the tiles fill the places (two to a compute unit, or one where the
+// deep pipeline runs), each part at least 8 k-tiles long.
 static int tiled_splits(int M, int N, int K) {
     if (K % 64) return 1;
     long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128);
+    long places = (long)llmrs_compute_units() * (deep_tiles(M, N, K) ? 1 : 2);
     int nk = K / 64, splits = 1;
-    while (tiles * splits * 2 <= 512 && splits < 16 && nk / (splits * 2) >= 8) splits *= 2;
+    while (tiles * splits * 2 <= places && splits < 16 && nk / (splits * 2) >= 8) splits *= 2;
     return splits;
+}
+// The 128 x 128 tiles of a product, in whichever of the two forms its shape asks for.
+static int launch_tiles_128(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
+                            int M, int N, int K, int epi, int splits, float* partial) {
+    if (deep_tiles(M, N, K)) return launch_dma<128, 128, 2, 4, 4>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial);
+    return launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial);
 }
 // 17..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
 // get blocks of many feature tiles): the 128 x 128 tiles with k split over blocks read the tokens'
@@ -865,7 +881,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         tiles_for_few = workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float);
     }
     if (tiles_for_few) {
-        rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, tiled_splits(M, N, K), (float*)workspace);
+        rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, tiled_splits(M, N, K), (float*)workspace);
     } else if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
         // waves in turn and their sums are added in wave order, so for a given weight an
@@ -952,9 +968,9 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         } else if (K % 64 == 0) {
             int splits = tiled_splits(M, N, K);
             if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
-                rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
+                rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
             else
-                rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi);
+                rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, 1, nullptr);
         }
         else rc = launch_tiled<128, 128, 64, 1>(stream, A, lda, W, out, ldc, M, N, K, epi);
     }
