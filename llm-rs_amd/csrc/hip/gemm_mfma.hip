@@ -366,7 +366,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
             }
             if (kt + 1 < nk) store_tile(cur ^ 1, (p + 1) % P);
-            __syncthreads();
+            // (a bare barrier: __syncthreads() would wait for the later tiles' loads as well)
+            __builtin_amdgcn_s_waitcnt(0xc07f);         // lgkmcnt(0): this wave's LDS reads and writes are done
+            __builtin_amdgcn_s_barrier();
         }
     }
 
