@@ -674,7 +674,7 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
 // (Measured on MI355X, 2048 x 4096 times 24576 features: 20 % faster than the loop above when
 // the product runs back to back with itself, 1 % inside a prompt step of the 8B shape.)
 // ---------------------------------------------------------------------------
-template <int BM, int BN, int WGM, int WGN>
+template <int BM, int BN, int WGM, int WGN, bool BUF = false>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_pingpong_kernel(const bf16* __restrict__ A, int lda,
                                                             const bf16* __restrict__ W, void* __restrict__ out,
                                                             int ldc, int M, int N, int K, int epi) {
@@ -701,19 +701,43 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_pingpong_kernel(const bf1
         gw[i] = W + (size_t)min(n0 + row, N - 1) * K + ((lslot ^ ((row >> 1) & 7)) * 8);
     }
     const int nk = K / 64;
+    // BUF: the loads go through buffer descriptors (a scalar base and a 32-bit offset per lane)
+    // instead of a 64-bit address per lane; the caller sees to it that both operands are under 4 GB.
+    // (The descriptor type and builtins exist for the device only.)
+#if defined(__HIP_DEVICE_COMPILE__)
+    __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)min((size_t)M * lda * 2, (size_t)0xffffffffu), 0x00020000);
+    __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)min((size_t)N * K * 2, (size_t)0xffffffffu), 0x00020000);
+#endif
+    unsigned oa[A_GROUPS], ow[W_GROUPS];
+#pragma unroll
+    for (int i = 0; i < A_GROUPS; ++i) oa[i] = (unsigned)((const char*)ga[i] - (const char*)A);
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) ow[i] = (unsigned)((const char*)gw[i] - (const char*)W);
     auto issue = [&](int kt) {
         if (kt >= nk) return;
         int stage = kt & 1;
         unsigned base = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + wave * A_GROUPS * 1024);
 #pragma unroll
-        for (int i = 0; i < A_GROUPS; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ga[i] + kt * 64),
-                                             (__attribute__((address_space(3))) void*)(pp_smem + base + i * 1024), 16, 0, 0);
+        for (int i = 0; i < A_GROUPS; ++i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (BUF)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (__attribute__((address_space(3))) void*)(pp_smem + base + i * 1024), 16, oa[i], kt * 128, 0, 0);
+            else
+#endif
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ga[i] + kt * 64),
+                                                 (__attribute__((address_space(3))) void*)(pp_smem + base + i * 1024), 16, 0, 0);
+        }
         unsigned wbase = __builtin_amdgcn_readfirstlane(stage * STAGE_BYTES + BM * 128 + wave * W_GROUPS * 1024);
 #pragma unroll
-        for (int i = 0; i < W_GROUPS; ++i)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gw[i] + kt * 64),
-                                             (__attribute__((address_space(3))) void*)(pp_smem + wbase + i * 1024), 16, 0, 0);
+        for (int i = 0; i < W_GROUPS; ++i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            if constexpr (BUF)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)(pp_smem + wbase + i * 1024), 16, ow[i], kt * 128, 0, 0);
+            else
+#endif
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gw[i] + kt * 64),
+                                                 (__attribute__((address_space(3))) void*)(pp_smem + wbase + i * 1024), 16, 0, 0);
+        }
     };
     f32x16 acc[FM][FN];
 #pragma unroll
@@ -790,20 +814,20 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_pingpong_kernel(const bf1
     tile_epilogue<BM, BN, WGM, WGN, 2 * STAGE_BYTES>(acc, pp_smem, out, ldc, M, N, epi, nullptr, m0, n0);
 }
 
-template <int BM, int BN, int WGM, int WGN>
+template <int BM, int BN, int WGM, int WGN, bool BUF = false>
 static int launch_pingpong(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                            int M, int N, int K, int epi) {
     static bool configured = false;
     size_t bytes = (size_t)2 * (BM + BN) * 128;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_pingpong_kernel<BM, BN, WGM, WGN>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_pingpong_kernel<BM, BN, WGM, WGN, BUF>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
         configured = true;
     }
     dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
-    gemm_pingpong_kernel<BM, BN, WGM, WGN><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+    gemm_pingpong_kernel<BM, BN, WGM, WGN, BUF><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
     return 0;
 }
 
@@ -956,16 +980,20 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                                         ldc, over, N, K, epi, workspace, workspace_bytes, qkv);
         }
         if (K % 64 == 0 && big_tiles >= 160) {
+            // operands under 4 GB are read through buffer descriptors (32-bit offsets), 1-4 % faster
+            const bool small = (size_t)M * lda * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32);
             long whole = big_tiles / cus * cus, rest = big_tiles - whole;
             int n_split = (int)(whole / m_tiles) * 256;        // features of the whole rounds
             if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4) {
                 size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
                 void* out_rest = (char*)out + (size_t)(epi == LLMRS_EPI_SWIGLU ? n_split / 2 : n_split) * elt;
-                rc = launch_pingpong<256, 256, 2, 4>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
+                rc = small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
+                           : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
                 if (rc == 0)
                     rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
             } else {
-                rc = launch_pingpong<256, 256, 2, 4>(stream, A, lda, W, out, ldc, M, N, K, epi);
+                rc = small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, N, K, epi)
+                           : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, N, K, epi);
             }
         } else if (K % 64 == 0) {
             int splits = tiled_splits(M, N, K);
