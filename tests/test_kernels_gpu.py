@@ -62,6 +62,8 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (513, 25600, 64),
                # few tiles and a long k: the k range is split over blocks and the parts are added by a second kernel
                (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048),
+               # up to 256 rows and no more tiles than compute units: one block of eight waves per unit, four k-tiles in LDS
+               (96, 6144, 2048), (256, 4096, 4096), (128, 28672, 1024), (192, 4100, 512),
                # a few rows beyond whole large tiles: those rows go to the kernel for few rows
                (1040, 10240, 128), (1080, 10500, 192), (2600, 4096, 1024),
                # long rows: narrow weights walk along k from staggered places too, with two feature tiles to a block
