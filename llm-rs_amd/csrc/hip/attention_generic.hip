@@ -136,6 +136,112 @@ __global__ __launch_bounds__(64) void attention_generic_split_kernel(
     }
 }
 
+// The same with a wave for each (entry, kv head, chunk) that serves all G heads of its kv head, so
+// that a key or a value is read once for them; each head's sums are formed exactly as walk_keys
+// forms them.  For 2, 4 or 8 heads per kv head and head sizes up to GROUP_MAX_HEAD_DIM.
+#define MAX_GROUP 8
+#define GROUP_MAX_HEAD_DIM 256
+template <class T, bool VEC, int G>
+__global__ __launch_bounds__(64) void attention_generic_group_kernel(
+    const T* __restrict__ q, float* __restrict__ partial, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ q_starts, const int* __restrict__ seq_lens,
+    int max_chunks, AttnArgs a) {
+    __shared__ float qs[G * GROUP_MAX_HEAD_DIM];
+    constexpr int NACC = GROUP_MAX_HEAD_DIM / 64;
+    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z, lane = threadIdx.x;
+    int t = q_starts[e];
+    if (q_starts[e + 1] - t != 1) return;
+    int pos = seq_lens[e] - 1;                    // an entry with one token: its position is its length less one
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int first = lo / GENERIC_CHUNK;
+    if (ch > pos / GENERIC_CHUNK - first) return;
+    int begin = max(lo, (first + ch) * GENERIC_CHUNK), end = min(pos + 1, (first + ch + 1) * GENERIC_CHUNK);
+    int hd = a.head_dim, ps = a.page_size;
+    const T* qrow = q + (size_t)t * a.q_stride + (size_t)kvh * G * hd;      // the kv head's G heads lie side by side
+    for (int d = lane; d < G * hd; d += 64) qs[d] = to_f32(qrow[d]);
+    __syncthreads();
+    const int* table = block_table + (size_t)e * a.table_width;
+    float m[G], l[G], acc[G][NACC];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY; l[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
+    }
+    for (int t0 = begin; t0 < end; t0 += 64) {
+        int j = t0 + lane;
+        bool valid = j < end;
+        int page = 0, off = 0;
+        float s[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) s[g] = -INFINITY;
+        if (valid) {
+            page = table[min(j / ps, a.table_width - 1)];
+            page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // stay inside the cache
+            off = j % ps;
+            const T* kp = k_cache + k_cache_index(page, kvh, off, 0, a.n_kv_heads, ps, hd);
+            float dot[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) dot[g] = 0.0f;
+            if constexpr (VEC) {
+                for (int d = 0; d < hd; d += 4) {
+                    float kv[4];
+                    load4(kp + d, kv);
+#pragma unroll
+                    for (int g = 0; g < G; ++g)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) dot[g] = fmaf(qs[g * hd + d + i], kv[i], dot[g]);
+                }
+            } else {
+                for (int d = 0; d < hd; ++d) {
+                    float kv = to_f32(kp[d]);
+#pragma unroll
+                    for (int g = 0; g < G; ++g) dot[g] = fmaf(qs[g * hd + d], kv, dot[g]);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) s[g] = dot[g] * a.scale;
+        }
+        float p[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float m_new = fmaxf(m[g], wave_max(s[g]));
+            p[g] = valid ? expf(s[g] - m_new) : 0.0f;
+            float rescale = expf(m[g] - m_new);
+            l[g] = l[g] * rescale + wave_sum(p[g]);
+            m[g] = m_new;
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) acc[g][i] *= rescale;
+        }
+        int n_valid = min(64, end - t0);
+        for (int jj = 0; jj < n_valid; ++jj) {
+            int pagej = __shfl(page, jj, 64), offj = __shfl(off, jj, 64);
+            float pj[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) pj[g] = __shfl(p[g], jj, 64);
+#pragma unroll
+            for (int i = 0; i < NACC; ++i) {
+                int d = lane + 64 * i;
+                if (d < hd) {
+                    float v = to_f32(v_cache[v_cache_index(pagej, kvh, offj, d, a.n_kv_heads, ps, hd)]);
+#pragma unroll
+                    for (int g = 0; g < G; ++g) acc[g][i] = fmaf(pj[g], v, acc[g][i]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float* pp = partial + ((size_t)(e * a.n_heads + kvh * G + g) * max_chunks + ch) * (hd + 2);
+        if (lane == 0) { pp[0] = m[g]; pp[1] = l[g]; }
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) {
+            int d = lane + 64 * i;
+            if (d < hd) pp[2 + d] = acc[g][i];
+        }
+    }
+}
+
 // One wave for each (entry, head) adds the chunks up, in ascending order.
 template <class T>
 __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
@@ -192,13 +298,26 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
                                                                      positions, q_starts, split, a);
     }
     if (split) {
-        dim3 grid(n_entries, a.n_heads, max_chunks);
-        if (vec)
-            attention_generic_split_kernel<T, true><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
-                                                                          q_starts, seq_lens, max_chunks, a);
-        else
-            attention_generic_split_kernel<T, false><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
-                                                                           q_starts, seq_lens, max_chunks, a);
+        int G = a.n_heads / a.n_kv_heads;
+        // a wave for all heads of a kv head when that still leaves two waves or more for each compute unit
+        // (measured in 32-bit at the 8B shape, 2048 keys: 8 requests 174 -> 88 us; one request alone is faster with a wave per head)
+        long group_waves = (long)(n_single > 0 ? n_single : n_entries) * a.n_kv_heads * max_chunks;
+        if (a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8) && group_waves >= 2L * llmrs_compute_units()) {
+            dim3 grid(n_entries, a.n_kv_heads, max_chunks);
+#define GROUP(V, GG) attention_generic_group_kernel<T, V, GG><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table, q_starts, seq_lens, max_chunks, a)
+            if (G == 8) { if (vec) GROUP(true, 8); else GROUP(false, 8); }
+            else if (G == 4) { if (vec) GROUP(true, 4); else GROUP(false, 4); }
+            else { if (vec) GROUP(true, 2); else GROUP(false, 2); }
+#undef GROUP
+        } else {
+            dim3 grid(n_entries, a.n_heads, max_chunks);
+            if (vec)
+                attention_generic_split_kernel<T, true><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
+                                                                              q_starts, seq_lens, max_chunks, a);
+            else
+                attention_generic_split_kernel<T, false><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table,
+                                                                               q_starts, seq_lens, max_chunks, a);
+        }
         attention_generic_merge_kernel<T><<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, q_starts, seq_lens,
                                                                                         max_chunks, a);
     }

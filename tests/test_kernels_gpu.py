@@ -334,7 +334,8 @@ def test_attention_many_decoding_requests(n_req, window):
 @pytest.mark.parametrize("window", [0, 200])
 @pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.float32, 4, 2, 64, 16), (torch.float32, 3, 1, 20, 4),
                                                      (torch.bfloat16, 6, 3, 48, 8), (torch.bfloat16, 5, 5, 80, 16),
-                                                     (torch.float32, 2, 2, 18, 4)])
+                                                     (torch.float32, 2, 2, 18, 4), (torch.float32, 8, 2, 32, 16),
+                                                     (torch.bfloat16, 8, 1, 48, 8)])
 def test_attention_plain_kernel_splits_decoding_requests(dtype, n_heads, n_kv, hd, ps, window):
     """Head and page sizes (and the 32-bit type) that the matrix-core kernels do not take: decoding
     requests are shared out over waves in chunks of 128 keys and merged; a prompt portion rides in
