@@ -367,6 +367,24 @@ def test_attention_plain_kernel_splits_decoding_requests(dtype, n_heads, n_kv, h
     assert (got[len(lens) - 1:].float() - ref).abs().max() <= tol
 
 
+@pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.float32, 8, 2, 32, 16), (torch.float32, 4, 2, 64, 16),
+                                                     (torch.bfloat16, 16, 2, 48, 8)])
+def test_attention_plain_kernel_many_decoding_requests(dtype, n_heads, n_kv, hd, ps):
+    """With enough decoding requests the plain kernel's waves each serve all heads of a kv head
+    (4, 2 and 8 here): every request against the plain implementation, a window on."""
+    n_req, window = 56, 300
+    g = torch.Generator().manual_seed(hd)
+    lens = [int(x) for x in torch.randint(1, 700, (n_req,), generator=g)]
+    lens[0], lens[1], lens[2] = 699, 128, 129
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=3)
+    qs = [torch.randn((1, n_heads, hd), generator=g).to(dtype) for _ in lens]
+    got = case.run(qs, [[n - 1] for n in lens], window=window)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    for r in range(n_req):
+        ref = case.reference(r, qs[r], [lens[r] - 1], window=window)[0].float()
+        assert (got[r].float() - ref).abs().max() <= tol, f"request {r} of length {lens[r]}"
+
+
 @pytest.mark.parametrize("hd", [64, 96, 128, 256])
 def test_attention_prompt_portion_finds_far_keys(hd):
     """A portion of a prompt far into a long sequence (page numbers are fetched 64 at a time, tiles
