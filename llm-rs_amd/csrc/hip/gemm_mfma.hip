@@ -671,7 +671,7 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
 // four phases later.  Every wave passes the same number of barriers.  Same LDS layout
 // as above (two tiles, rows of 128 bytes, chunks swizzled), same order of sums: the
 // results are bitwise those of the loop above.  A wave multiplies at raised priority.
-// (Measured on MI355X, 2048 x 4096 times 24576 features: 20 % faster than the loop above when
+// (Measured on MI355X, 2048 x 4096 times 24576 features: 2-5 % faster than the loop above when
 // the product runs back to back with itself, 1 % inside a prompt step of the 8B shape.)
 // ---------------------------------------------------------------------------
 template <int BM, int BN, int WGM, int WGN, bool BUF = false>
