@@ -136,38 +136,16 @@ __global__ __launch_bounds__(64) void attention_generic_split_kernel(
     }
 }
 
-// The same with a wave for each (entry, kv head, chunk) that serves all G heads of its kv head, so
-// that a key or a value is read once for them; each head's sums are formed exactly as walk_keys
-// forms them.  For 2, 4 or 8 heads per kv head and head sizes up to GROUP_MAX_HEAD_DIM.
-#define MAX_GROUP 8
+// A wave that serves all G heads of a kv head reads a key or a value once for them; each head's sums
+// are formed exactly as walk_keys forms them.  For 2, 4 or 8 heads per kv head and head sizes up
+// to GROUP_MAX_HEAD_DIM.  qs: the G heads' queries side by side, [G][head_dim].
 #define GROUP_MAX_HEAD_DIM 256
 template <class T, bool VEC, int G>
-__global__ __launch_bounds__(64) void attention_generic_group_kernel(
-    const T* __restrict__ q, float* __restrict__ partial, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const int* __restrict__ block_table, const int* __restrict__ q_starts, const int* __restrict__ seq_lens,
-    int max_chunks, AttnArgs a) {
-    __shared__ float qs[G * GROUP_MAX_HEAD_DIM];
+__device__ __forceinline__ void walk_keys_group(const float* qs, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                                const int* __restrict__ table, const AttnArgs& a, int kvh, int begin, int end,
+                                                float (&m)[G], float (&l)[G], float (&acc)[G][GROUP_MAX_HEAD_DIM / 64]) {
     constexpr int NACC = GROUP_MAX_HEAD_DIM / 64;
-    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z, lane = threadIdx.x;
-    int t = q_starts[e];
-    if (q_starts[e + 1] - t != 1) return;
-    int pos = seq_lens[e] - 1;                    // an entry with one token: its position is its length less one
-    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-    int first = lo / GENERIC_CHUNK;
-    if (ch > pos / GENERIC_CHUNK - first) return;
-    int begin = max(lo, (first + ch) * GENERIC_CHUNK), end = min(pos + 1, (first + ch + 1) * GENERIC_CHUNK);
-    int hd = a.head_dim, ps = a.page_size;
-    const T* qrow = q + (size_t)t * a.q_stride + (size_t)kvh * G * hd;      // the kv head's G heads lie side by side
-    for (int d = lane; d < G * hd; d += 64) qs[d] = to_f32(qrow[d]);
-    __syncthreads();
-    const int* table = block_table + (size_t)e * a.table_width;
-    float m[G], l[G], acc[G][NACC];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-        m[g] = -INFINITY; l[g] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
-    }
+    int lane = threadIdx.x, hd = a.head_dim, ps = a.page_size;
     for (int t0 = begin; t0 < end; t0 += 64) {
         int j = t0 + lane;
         bool valid = j < end;
@@ -230,6 +208,71 @@ __global__ __launch_bounds__(64) void attention_generic_group_kernel(
             }
         }
     }
+}
+
+// attention_generic_kernel with a wave for each (token, kv head).
+template <class T, bool VEC, int G>
+__global__ __launch_bounds__(64) void attention_generic_group_tokens_kernel(
+    const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ token_entry, const int* __restrict__ positions,
+    const int* __restrict__ q_starts, int skip_single, AttnArgs a) {
+    __shared__ float qs[G * GROUP_MAX_HEAD_DIM];
+    constexpr int NACC = GROUP_MAX_HEAD_DIM / 64;
+    int t = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x, hd = a.head_dim;
+    int e = token_entry[t];
+    if (skip_single && q_starts[e + 1] - q_starts[e] == 1) return;
+    int pos = positions[t];
+    const T* qrow = q + (size_t)t * a.q_stride + (size_t)kvh * G * hd;      // the kv head's G heads lie side by side
+    for (int d = lane; d < G * hd; d += 64) qs[d] = to_f32(qrow[d]);
+    __syncthreads();
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    float m[G], l[G], acc[G][NACC];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY; l[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
+    }
+    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, lo, pos + 1, m, l, acc);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        T* orow = out + (size_t)t * a.out_stride + (size_t)(kvh * G + g) * hd;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) {
+            int d = lane + 64 * i;
+            if (d < hd) orow[d] = from_f32<T>(acc[g][i] / l[g]);
+        }
+    }
+}
+
+// attention_generic_split_kernel with a wave for each (entry, kv head, chunk).
+template <class T, bool VEC, int G>
+__global__ __launch_bounds__(64) void attention_generic_group_kernel(
+    const T* __restrict__ q, float* __restrict__ partial, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const int* __restrict__ block_table, const int* __restrict__ q_starts, const int* __restrict__ seq_lens,
+    int max_chunks, AttnArgs a) {
+    __shared__ float qs[G * GROUP_MAX_HEAD_DIM];
+    constexpr int NACC = GROUP_MAX_HEAD_DIM / 64;
+    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z, lane = threadIdx.x;
+    int t = q_starts[e];
+    if (q_starts[e + 1] - t != 1) return;
+    int pos = seq_lens[e] - 1;                    // an entry with one token: its position is its length less one
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int first = lo / GENERIC_CHUNK;
+    if (ch > pos / GENERIC_CHUNK - first) return;
+    int begin = max(lo, (first + ch) * GENERIC_CHUNK), end = min(pos + 1, (first + ch + 1) * GENERIC_CHUNK);
+    int hd = a.head_dim;
+    const T* qrow = q + (size_t)t * a.q_stride + (size_t)kvh * G * hd;
+    for (int d = lane; d < G * hd; d += 64) qs[d] = to_f32(qrow[d]);
+    __syncthreads();
+    float m[G], l[G], acc[G][NACC];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY; l[g] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) acc[g][i] = 0.0f;
+    }
+    walk_keys_group<T, VEC, G>(qs, k_cache, v_cache, block_table + (size_t)e * a.table_width, a, kvh, begin, end, m, l, acc);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         float* pp = partial + ((size_t)(e * a.n_heads + kvh * G + g) * max_chunks + ch) * (hd + 2);
@@ -288,21 +331,32 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
     bool split = max_chunks > 0 && scratch != nullptr && q_starts != nullptr && seq_lens != nullptr &&
                  scratch_bytes >= need && n_single != 0 && n_entries <= 65535 && max_chunks <= 65535;
     bool only_single = split && a.n_tokens == n_entries;     // every entry brings one token
+    const int G = a.n_heads / a.n_kv_heads;
+    const bool groupable = a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8);
     if (!only_single) {
-        dim3 grid(a.n_tokens, a.n_heads);
-        if (vec)
-            attention_generic_kernel<T, true><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
-                                                                    positions, q_starts, split, a);
-        else
-            attention_generic_kernel<T, false><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
-                                                                     positions, q_starts, split, a);
+        // a wave for all heads of a kv head when that still leaves two waves or more for each compute unit
+        if (groupable && (long)a.n_tokens * a.n_kv_heads >= 2L * llmrs_compute_units()) {
+            dim3 grid(a.n_tokens, a.n_kv_heads);
+#define TOKENS(V, GG) attention_generic_group_tokens_kernel<T, V, GG><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, split, a)
+            if (G == 8) { if (vec) TOKENS(true, 8); else TOKENS(false, 8); }
+            else if (G == 4) { if (vec) TOKENS(true, 4); else TOKENS(false, 4); }
+            else { if (vec) TOKENS(true, 2); else TOKENS(false, 2); }
+#undef TOKENS
+        } else {
+            dim3 grid(a.n_tokens, a.n_heads);
+            if (vec)
+                attention_generic_kernel<T, true><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
+                                                                        positions, q_starts, split, a);
+            else
+                attention_generic_kernel<T, false><<<grid, 64, 0, stream>>>(q, out, k_cache, v_cache, block_table, token_entry,
+                                                                         positions, q_starts, split, a);
+        }
     }
     if (split) {
-        int G = a.n_heads / a.n_kv_heads;
         // a wave for all heads of a kv head when that still leaves two waves or more for each compute unit
         // (measured in 32-bit at the 8B shape, 2048 keys: 8 requests 174 -> 88 us; one request alone is faster with a wave per head)
         long group_waves = (long)(n_single > 0 ? n_single : n_entries) * a.n_kv_heads * max_chunks;
-        if (a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8) && group_waves >= 2L * llmrs_compute_units()) {
+        if (groupable && group_waves >= 2L * llmrs_compute_units()) {
             dim3 grid(n_entries, a.n_kv_heads, max_chunks);
 #define GROUP(V, GG) attention_generic_group_kernel<T, V, GG><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table, q_starts, seq_lens, max_chunks, a)
             if (G == 8) { if (vec) GROUP(true, 8); else GROUP(false, 8); }

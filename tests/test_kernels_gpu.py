@@ -385,6 +385,26 @@ def test_attention_plain_kernel_many_decoding_requests(dtype, n_heads, n_kv, hd,
         assert (got[r].float() - ref).abs().max() <= tol, f"request {r} of length {lens[r]}"
 
 
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.float32, 8, 2, 32, 16), (torch.float32, 4, 2, 64, 4),
+                                                     (torch.bfloat16, 16, 2, 48, 8)])
+def test_attention_plain_kernel_long_prompt_portion(dtype, n_heads, n_kv, hd, ps, window):
+    """A prompt portion long enough that the plain kernel's waves each serve all heads of a kv head
+    (4, 2 and 8 here), a whole short prompt and a decoding request beside it."""
+    g = torch.Generator().manual_seed(hd + window)
+    lens = [400, 9, 200]
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=5)
+    pos = [list(range(80, 400)), list(range(0, 9)), [199]]
+    qs = [torch.randn((len(p), n_heads, hd), generator=g).to(dtype) for p in pos]
+    got = case.run(qs, pos, window=window)
+    tol = 2e-4 if dtype == torch.float32 else 3e-2
+    at = 0
+    for r, p in enumerate(pos):
+        ref = case.reference(r, qs[r], p, window=window).float()
+        assert (got[at:at + len(p)].float() - ref).abs().max() <= tol, f"request {r}"
+        at += len(p)
+
+
 @pytest.mark.parametrize("hd", [64, 96, 128, 256])
 def test_attention_prompt_portion_finds_far_keys(hd):
     """A portion of a prompt far into a long sequence (page numbers are fetched 64 at a time, tiles
