@@ -1,8 +1,10 @@
 // The plain product: 64x64 tiles through LDS, 32-bit FMA, k in ascending order.
-// It is the whole 32-bit path (no matrix-core mode rounds its inputs) and the
-// bfloat16 fallback for shapes the MFMA kernels refuse.  The order of the sum for
-// an output depends on K only, so a row's result does not depend on M, on the
-// row's place in the batch or on its tile.
+// With the 32-bit matrix-core tiles and the few-row kernel below it is the whole
+// 32-bit path (nothing here rounds its inputs) and the bfloat16 fallback for shapes
+// the bfloat16 MFMA kernels refuse.  Within each of the three kernels the order of
+// the sum for an output depends on K only, so a row's result does not depend on the
+// row's place in the batch or on its tile; which kernel runs depends on M (up to 8
+// rows, up to 16, more), so across those ranges results differ by rounding.
 // Reference: gemm_f32 accumulates in 32-bit the same way (shaders/ops.metal:1053-1079).
 #include "gemm.h"
 
@@ -61,6 +63,112 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
             }
         }
     }
+}
+
+// 32-bit products on the matrix cores: v_mfma_f32_32x32x2_f32 multiplies and adds in 32-bit (no
+// reduced-precision mode), k in ascending order, so an output's sum depends on K only here too.
+// 128 x 128 tiles of four waves (64 x 64 each), k in steps of 16 through two LDS buffers; the next
+// step's rows are on their way to registers while this step is multiplied.  Any M, N, K: rows and
+// k beyond the edges are read as zeros.
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+#define F32_BK 16
+#define F32_LD (F32_BK + 1)      // LDS row stride in floats: lanes of an operand read (32 rows, one k each) hit distinct banks
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ A, int lda,
+                                                            const float* __restrict__ W, void* __restrict__ out, int ldc,
+                                                            int M, int N, int K, int epi) {
+    __shared__ float As[2][128 * F32_LD];
+    __shared__ float Ws[2][128 * F32_LD];
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int wm = wave >> 1, wn = wave & 1;
+    int m0 = blockIdx.y * 128, n0 = blockIdx.x * 128;
+    // staging: thread t brings 4 consecutive k of rows (t / 4) and (t / 4 + 64) of each tile
+    int srow = tid >> 2, sk = (tid & 3) * 4;
+    const bool vec = K % 4 == 0 && lda % 4 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0;
+    float ra[2][4], rw[2][4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int am = m0 + srow + 64 * h, wn_ = n0 + srow + 64 * h, k = k0 + sk;
+            const float* ap = A + (size_t)min(am, M - 1) * lda + k;
+            const float* wp = W + (size_t)min(wn_, N - 1) * K + k;
+            if (vec && k + 3 < K) {
+                load4(ap, ra[h]);
+                load4(wp, rw[h]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    ra[h][j] = k + j < K ? ap[j] : 0.0f;
+                    rw[h][j] = k + j < K ? wp[j] : 0.0f;
+                }
+            }
+            if (am >= M)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ra[h][j] = 0.0f;
+            if (wn_ >= N)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) rw[h][j] = 0.0f;
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                As[buf][(srow + 64 * h) * F32_LD + sk + j] = ra[h][j];
+                Ws[buf][(srow + 64 * h) * F32_LD + sk + j] = rw[h][j];
+            }
+    };
+    f32x16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    int nk = (K + F32_BK - 1) / F32_BK;
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    int frow = lane & 31, fk = lane >> 5;
+    for (int kt = 0; kt < nk; ++kt) {
+        int buf = kt & 1;
+        if (kt + 1 < nk) fetch((kt + 1) * F32_BK);
+        const float* as = As[buf] + (wm * 64 + frow) * F32_LD + fk;
+        const float* ws = Ws[buf] + (wn * 64 + frow) * F32_LD + fk;
+#pragma unroll
+        for (int ks = 0; ks < F32_BK / 2; ++ks) {
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = as[i * 32 * F32_LD + ks * 2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = ws[j * 32 * F32_LD + ks * 2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) stage(buf ^ 1);        // the other buffer's readers finished before the last barrier
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            int n = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                float v = acc[i][j][r];
+                if (epi == LLMRS_EPI_SWIGLU) {
+                    float other = __shfl_xor(v, 1, 64);   // even lane: gate here, up next door
+                    if (!(lane & 1) && m < M && n + 1 < N)
+                        ((float*)out)[(size_t)m * ldc + n / 2] = silu_f32(v) * other;
+                } else if (m < M && n < N) {
+                    epilogue_store<float>(epi, out, ldc, m, n, v);
+                }
+            }
+        }
 }
 
 // A few tokens (decoding): a wave for each pair of weight rows, every weight read once.
@@ -167,7 +275,11 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
     }
     dim3 grid(ceil_div(N, TILE), ceil_div(M, TILE));
     LLMRS_REQUIRE(grid.y <= 65535, "gemm: M=%d is too large for one launch", M);
-    if (dtype == LLMRS_F32)
+    if (dtype == LLMRS_F32 && allow_mfma && M > 16) {
+        dim3 g128(ceil_div(N, 128), ceil_div(M, 128));
+        LLMRS_REQUIRE(g128.y <= 65535, "gemm: M=%d is too large for one launch", M);
+        gemm_f32_mfma_kernel<<<g128, 256, 0, stream>>>((const float*)A, lda, (const float*)W, out, ldc, M, N, K, epi);
+    } else if (dtype == LLMRS_F32)
         gemm_simple_kernel<float><<<grid, 256, 0, stream>>>((const float*)A, lda, (const float*)W, out, ldc, M, N, K, epi);
     else if (dtype == LLMRS_BF16)
         gemm_simple_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi);
