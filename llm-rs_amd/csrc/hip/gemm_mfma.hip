@@ -42,6 +42,12 @@ __device__ __forceinline__ bf16x8 zero8() {
     return z;
 }
 
+// The tile loops' barrier: this wave's LDS reads and writes are done, then every wave of the block
+// has arrived.  Unlike __syncthreads() it does not wait for loads from memory that are still in
+// flight (the later tiles of a pipeline); the "memory" clobber keeps the compiler from moving
+// memory accesses across it.
+__device__ __forceinline__ void block_sync_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // ---------------------------------------------------------------------------
 // skinny: C^T[n, m] = sum_k W[n, k] X[m, k]
 //   A operand = W rows: lane l holds row n0 + l%16 (+16 per feature tile), 8 consecutive k
@@ -367,8 +373,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
             }
             if (kt + 1 < nk) store_tile(cur ^ 1, (p + 1) % P);
             // (a bare barrier: __syncthreads() would wait for the later tiles' loads as well)
-            __builtin_amdgcn_s_waitcnt(0xc07f);         // lgkmcnt(0): this wave's LDS reads and writes are done
-            __builtin_amdgcn_s_barrier();
+            block_sync_lds();
         }
     }
 
@@ -627,8 +632,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
         // the next tile must have landed before anybody reads it; later tiles may still be on their way
         // (a bare barrier: __syncthreads() would wait for every load in flight, the later tiles' too)
         if (kt + STAGES - 1 < nk) wait_vmcnt<(STAGES - 2) * LOADS>(); else wait_vmcnt<0>();
-        __builtin_amdgcn_s_waitcnt(0xc07f);                     // lgkmcnt(0): this wave has read what it needs of the tile
-        __builtin_amdgcn_s_barrier();
+        block_sync_lds();
     }
 
     tile_epilogue<BM, BN, WGM, WGN, STAGES * STAGE_BYTES>(acc, dma_smem, out, ldc, M, N, epi, partial, m0, n0);
@@ -749,7 +753,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_pingpong_kernel(const bf1
 
     auto barrier = [] {
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_barrier();
+        block_sync_lds();
         __builtin_amdgcn_sched_barrier(0);
     };
     auto lds_done = [] { __builtin_amdgcn_s_waitcnt(0xc07f); };     // lgkmcnt(0)
