@@ -983,7 +983,9 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             return llmrs_gemm_bf16_mfma(stream, A + (size_t)whole_rows * lda, lda, W, (char*)out + (size_t)whole_rows * ldc * elt,
                                         ldc, over, N, K, epi, workspace, workspace_bytes, qkv);
         }
-        if (K % 64 == 0 && big_tiles >= 160 && M > 128) {      // (up to 128 rows a 256-row tile would be half empty)
+        // (up to 128 rows a 256-row tile would be half empty; 257-384 rows are still faster on two rows of
+        // large tiles than on three of small ones: the lm head at 300 rows 640 against 750 us)
+        if (K % 64 == 0 && big_tiles >= 160 && M > 128) {
             // operands under 4 GB are read through buffer descriptors (32-bit offsets), 1-4 % faster
             const bool small = (size_t)M * lda * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32);
             long whole = big_tiles / cus * cus, rest = big_tiles - whole;
