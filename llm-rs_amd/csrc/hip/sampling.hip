@@ -1,5 +1,8 @@
 // Next-token choice on the device: only token ids go back to the host.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 // Greedy: the index of the largest logit; of equal ones the lowest index wins.
 // (The reference's kernel, shaders/ops.metal:803-835, leaves ties to the scan's
@@ -67,6 +70,60 @@ extern "C" int llmrs_argmax_rows(hipStream_t stream, const float* logits, int ld
         argmax_rows_kernel<<<dim3(n_rows, 1), 1024, 0, stream>>>(logits, ld, V, nullptr, nullptr, nullptr, out);
     }
     LLMRS_LAUNCH_CHECK("argmax_rows");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The same two stages for callers that cannot allocate (no_alloc.h): the partial
+// results live in a file-scope array of device memory instead of a buffer the
+// caller brings.  In host code the array's name only stands for the symbol; its
+// address on a device is asked for once per device, with that device current,
+// and kept.  Each GPU has its own copy of the array at its own address.
+static __device__ __align__(256) unsigned char scratch[LLMRS_ARGMAX_STATIC_BYTES];
+static_assert(LLMRS_ARGMAX_STATIC_BYTES == LLMRS_ARGMAX_STATIC_MAX_ROWS * ARGMAX_PARTS * 8, "a (value, index) pair per row and part");
+
+#define LLMRS_MAX_DEVICES 64
+static void* g_scratch_of_device[LLMRS_MAX_DEVICES];
+static std::mutex g_scratch_mutex;
+
+static int argmax_static_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    LLMRS_REQUIRE(e == hipSuccess, "argmax_rows_static: no current device: %s", hipGetErrorString(e));
+    LLMRS_REQUIRE(dev >= 0 && dev < LLMRS_MAX_DEVICES, "argmax_rows_static: device %d is beyond the %d this library keeps addresses for",
+                  dev, LLMRS_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_of_device[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        LLMRS_REQUIRE(e == hipSuccess && p != nullptr, "argmax_rows_static: cannot find the scratch array on device %d: %s", dev,
+                      hipGetErrorString(e));
+        g_scratch_of_device[dev] = p;
+    }
+    *ptr = g_scratch_of_device[dev];
+    return 0;
+}
+
+// A call with n_rows = 0 only looks the array's address up: a caller that is about to
+// record a graph makes one such call on each device first.
+extern "C" int llmrs_argmax_rows_static(hipStream_t stream, const float* logits, int ld, int n_rows, int V, int* out) {
+    LLMRS_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax_rows_static: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
+    LLMRS_REQUIRE(n_rows <= LLMRS_ARGMAX_STATIC_MAX_ROWS, "argmax_rows_static: %d rows, the scratch array holds the partial results of %d",
+                  n_rows, LLMRS_ARGMAX_STATIC_MAX_ROWS);
+    void* ptr = nullptr;
+    if (argmax_static_scratch(&ptr) != 0) return -1;
+    if (n_rows == 0) return 0;
+    LLMRS_REQUIRE(logits != nullptr && out != nullptr, "argmax_rows_static: null logits or out");
+    if (V >= 8192) {
+        // Stage 1 writes every (row, part) pair that stage 2 reads, so what an earlier call left is never seen.
+        float* pv = (float*)ptr;
+        int* pi = (int*)(pv + (size_t)n_rows * ARGMAX_PARTS);
+        argmax_rows_kernel<<<dim3(n_rows, ARGMAX_PARTS), 1024, 0, stream>>>(logits, ld, V, nullptr, nullptr, pv, pi);
+        argmax_rows_kernel<<<dim3(n_rows, 1), 64, 0, stream>>>(nullptr, 0, ARGMAX_PARTS, pv, pi, nullptr, out);
+    } else {
+        argmax_rows_kernel<<<dim3(n_rows, 1), 1024, 0, stream>>>(logits, ld, V, nullptr, nullptr, nullptr, out);
+    }
+    LLMRS_LAUNCH_CHECK("argmax_rows_static");
     return 0;
 }
 
