@@ -37,6 +37,10 @@ class OutOfPages(RuntimeError):
     pass
 
 
+class _GrewWhileRecording(Exception):
+    """A buffer would have had to grow in the middle of a recording."""
+
+
 @dataclass
 class StepEntry:
     slot: int
@@ -86,12 +90,19 @@ class StepRunner:
         self._dev_words = torch.zeros(words_capacity, dtype=torch.int32, device=self.device)
         self.ctx = StepContext(self)
         # HIP graphs of decode steps: key -> (graph, logits); a key is recorded when it has been seen a few times
-        self.use_graphs = (self._pinned and os.environ.get("LLMRS_GRAPHS", "1") != "0" and not cache.state_tensors
+        # (fixed-size state does not stand in the way: it is reset before a step runs, outside any recording,
+        # and a mixer that says it is graph_safe finds its rows through the slots on the device)
+        self.use_graphs = (self._pinned and os.environ.get("LLMRS_GRAPHS", "1") != "0" and not os.environ.get("LLM_PERF")
                            and bool(getattr(model, "graph_safe", lambda: False)()))
+        # With this on, an event is recorded right before a step's first kernel, for whoever wants the
+        # device's share of the time (the engine pairs it with one after sampling).
+        self.time_device = False
+        self.started: Optional["torch.cuda.Event"] = None
         self.max_graph_batch = 512
         self.max_graphs = 256            # recorded graphs kept (the least recently replayed goes first)
         self._graphs: "OrderedDict[tuple, tuple]" = OrderedDict()
         self._seen: Dict[tuple, int] = {}
+        self._recording = False          # between the start and the end of a stream capture
         self.graph_replays = 0
 
     def _new_host(self, n: int) -> torch.Tensor:
@@ -104,13 +115,23 @@ class StepRunner:
         nbytes = n * dtype.itemsize
         buf = self._buffers.get(name)
         if buf is None or buf.numel() < nbytes:
+            if self._recording:
+                # Neither allocating nor dropping the recorded graphs (they hold the old addresses) may
+                # happen while a stream is being captured: give the recording up; the step then runs
+                # eagerly, where this buffer grows in the ordinary way.
+                raise _GrewWhileRecording(name)
             # grow with head room so that a slowly growing step does not reallocate each time
             cap = max(nbytes, 256) if buf is None else max(nbytes, 2 * buf.numel())
             buf = torch.empty(cap, dtype=torch.uint8, device=self.device)
             self._buffers[name] = buf
-            self._graphs.clear()        # recorded graphs hold the old addresses
-            self._seen.clear()
+            self._drop_graphs()         # recorded graphs hold the old addresses
         return buf[:nbytes].view(dtype).view(*shape)
+
+    def _drop_graphs(self) -> None:
+        """Forgets every recorded graph.  Destroying a graph frees device objects, so never during a recording."""
+        assert not self._recording, "recorded graphs must not be destroyed while a stream is being captured"
+        self._graphs.clear()
+        self._seen.clear()
 
     # -- staging -----------------------------------------------------------------
     def _staging(self, words_needed: int) -> np.ndarray:
@@ -127,8 +148,7 @@ class StepRunner:
         i = self._turn
         if self._dev_words.numel() < n_words:
             self._dev_words = torch.zeros(max(n_words, 2 * self._dev_words.numel()), dtype=torch.int32, device=self.device)
-            self._graphs.clear()
-            self._seen.clear()
+            self._drop_graphs()
         dev = self._dev_words[:n_words]
         dev.copy_(self._host[i][:n_words], non_blocking=True)
         if self._pinned:
@@ -232,6 +252,9 @@ class StepRunner:
     def _execute(self, ctx: StepContext, graph_widths=None) -> Optional[torch.Tensor]:
         fresh = [slot for slot, start, _ in ctx.entries if start == 0]
         self.cache.reset_state(fresh)
+        if self.time_device and self._pinned:
+            self.started = torch.cuda.Event(enable_timing=True)
+            self.started.record()
         if graph_widths is None:
             return self.model.forward(ctx, self.cache.views)
         # A decode step.  Everything the kernels take from the host must be the same for
@@ -255,13 +278,23 @@ class StepRunner:
         graph = torch.cuda.CUDAGraph()
         was_enabled = gc.isenabled()
         gc.disable()
+        gave_up = False
+        self._recording = True
         try:
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, self.cache.views)
+        except _GrewWhileRecording:
+            gave_up = True
         finally:
+            self._recording = False
             if was_enabled:
                 gc.enable()
-        if key not in self._seen:       # the workspace grew while recording: those addresses are gone
+        if gave_up:
+            # A part asked for more room than the eager runs of this shape did.  The capture has ended;
+            # what it recorded is dropped now, the step runs eagerly (its buffers grow there), and the
+            # shape is counted from the start again.
+            del graph
+            self._seen.pop(key, None)
             return self.model.forward(ctx, self.cache.views)
         while len(self._graphs) >= self.max_graphs:
             self._graphs.popitem(last=False)
