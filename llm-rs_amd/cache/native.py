@@ -39,6 +39,7 @@ def _lib():
             "llmrs_build_batch": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                   c_void_p, c_int, c_void_p],
             "llmrs_sched_add": [c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_float, c_uint64, c_void_p, c_int],
+            "llmrs_sched_check": [c_void_p, c_int, c_int],
             "llmrs_sched_idle": [c_void_p], "llmrs_sched_running": [c_void_p], "llmrs_sched_waiting": [c_void_p],
             "llmrs_sched_plan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
             "llmrs_sched_build": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
@@ -158,6 +159,10 @@ class HostCore:
         if rc == -2:
             return -1
         return self._check(rc)
+
+    def check_request(self, n_prompt: int, max_new: int) -> None:
+        """Raises what `add_request` would raise for a request that can never run."""
+        self._check(self._lib.llmrs_sched_check(self._h, int(n_prompt), int(max_new)))
 
     def idle(self) -> bool:
         return bool(self._lib.llmrs_sched_idle(self._h))

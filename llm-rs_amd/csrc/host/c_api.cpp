@@ -136,6 +136,14 @@ int llmrs_sched_add(void* h, const int32_t* prompt, int n_prompt, int max_new, f
         return slot < 0 ? -2 : slot;
     });
 }
+// 0 when a request of these lengths could run, -1 when llmrs_sched_add would refuse it for good (see error)
+int llmrs_sched_check(void* h, int n_prompt, int max_new) {
+    auto c = (Core*)h;
+    return guarded(c, [&] {
+        c->scheduler->check(n_prompt, max_new);
+        return 0;
+    });
+}
 int llmrs_sched_idle(void* h) { return ((Core*)h)->scheduler->idle() ? 1 : 0; }
 int llmrs_sched_running(void* h) { return ((Core*)h)->scheduler->num_running(); }
 int llmrs_sched_waiting(void* h) { return ((Core*)h)->scheduler->num_waiting(); }

@@ -13,29 +13,38 @@ Scheduler::Scheduler(CacheManager& cache, int token_budget, int max_chunk, int m
     if (token_budget <= 0) throw std::invalid_argument("token budget must be positive");
 }
 
-int Scheduler::add(const int32_t* prompt, int n_prompt, int max_new, const SamplingParams& sp,
-                   const int32_t* stop, int n_stop) {
+void Scheduler::check(int n_prompt, int max_new) const {
     if (n_prompt <= 0) throw std::invalid_argument("a request needs at least one prompt token");
     if (max_new <= 0) throw std::invalid_argument("max_new_tokens must be positive");
-    int total = n_prompt + max_new;
+    long long total = (long long)n_prompt + max_new;
     if (total > max_positions_)
         throw std::invalid_argument("request needs " + std::to_string(total) + " positions, the model has " +
                                     std::to_string(max_positions_));
-    // The last step of a request alone in the pool: all it has computed plus one
-    // portion.  If even that exceeds a pool, no schedule can ever finish it.
+    // The most pages a request alone in the pool has to hold at once.  If even
+    // that exceeds a pool, no schedule can ever finish it.  Without a window: all
+    // it computes (its last token is sampled, never run).  With a window w: the
+    // keys a portion's first query still sees and the portion itself, w + n - 1
+    // positions in a row for a portion of n; where a portion starts depends on
+    // what else shared the budget, so the bound is for the worst start, where
+    // that many positions touch one page more than they fill.
+    int computed = (int)total - 1;
     for (int g = 0; g < cache_.num_groups(); ++g) {
-        int worst = 0;
-        if (cache_.group(g).window == 0) {
-            worst = cache_.pages_needed(g, 0, total - 1);
-        } else {
-            int chunk = std::min(max_chunk_, budget_);
-            for (int start = 0; start < total - 1; start += chunk)
-                worst = std::max(worst, cache_.pages_needed(g, start, std::min(chunk, total - 1 - start)));
+        int ps = cache_.group(g).page_size, w = cache_.group(g).window;
+        int worst = cache_.pages_needed(g, 0, computed);
+        if (w > 0) {
+            int n = std::min({max_chunk_, budget_, computed});
+            long long span = std::min<long long>((long long)w + n - 1, computed);
+            worst = std::min<long long>(worst, span <= 1 ? 1 : (span - 1 + ps - 1) / ps + 1);
         }
         if (worst > cache_.pages_total(g))
             throw std::invalid_argument("request needs " + std::to_string(worst) + " pages of cache group " +
                                         std::to_string(g) + ", the pool has " + std::to_string(cache_.pages_total(g)));
     }
+}
+
+int Scheduler::add(const int32_t* prompt, int n_prompt, int max_new, const SamplingParams& sp,
+                   const int32_t* stop, int n_stop) {
+    check(n_prompt, max_new);
     int slot = cache_.acquire_slot();
     if (slot < 0) return -1;
     Request& r = requests_[slot];

@@ -64,6 +64,8 @@ public:
     // or needing more pages at once than a pool has.
     int add(const int32_t* prompt, int n_prompt, int max_new, const SamplingParams& sp,
             const int32_t* stop, int n_stop);
+    // Throws what add() would throw for a request of these lengths; changes nothing.
+    void check(int n_prompt, int max_new) const;
     bool idle() const { return running_.empty() && waiting_.empty(); }
 
     // The next step's entries; empty when idle.

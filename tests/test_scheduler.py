@@ -245,3 +245,34 @@ def test_abort_gives_everything_back():
         core.abort_request(a)
     c = core.add_request([1, 2, 3], 2)
     assert Driver(core).run()[c][0] == alone([1, 2, 3], 2)[0]
+
+
+def test_window_group_bound_holds_for_portions_that_start_anywhere():
+    """With a window, a request's pages at once are the keys its portion's first query still sees and
+    the portion itself.  Where a portion starts depends on what else shared the budget: page 16,
+    window 16, portions of 16 need 2 pages from an aligned start and 3 from position 17.  A request
+    is admitted only to a pool that holds the worst start."""
+    with pytest.raises(CoreError, match="3 pages"):
+        HostCore([(16, 2, 16)], max_requests=2, token_budget=16, max_chunk=16).add_request(list(range(40)), 8)
+    # a request shorter than window + portion needs no more than all its keys
+    small = HostCore([(16, 2, 16)], max_requests=2, token_budget=16, max_chunk=16)
+    small.check_request(20, 13)                 # 32 computed positions: 2 pages
+    # two requests share the budget, so portions start off the page grid; the pool is exactly the bound
+    core = HostCore([(16, 3, 16)], max_requests=2, token_budget=17, max_chunk=16)
+    a = core.add_request([1] * 3, 2)            # one token of the budget goes to this one while it decodes
+    b = core.add_request(list(range(60)), 6)
+    d = Driver(core)
+    done = d.run()
+    starts = [p[1] for plan in d.steps for p in plan if p[0] == b]
+    assert any(s % 16 for s in starts), "the case must cut portions off the page grid"
+    assert done[a][0] == alone([1] * 3, 2)[0] and done[b][0] == alone(list(range(60)), 6)[0]
+    assert done[b][1]["preemptions"] == 0
+    assert core.pages_free() == 3
+
+
+def test_check_request_changes_nothing():
+    core = HostCore([(4, 5, 0)], max_requests=4, token_budget=64, max_positions=64)
+    with pytest.raises(CoreError, match="pages"):
+        core.check_request(18, 4)
+    core.check_request(10, 4)
+    assert core.idle() and core.slots_in_use() == 0 and core.pages_free() == 5
