@@ -27,7 +27,7 @@ GPU_ARCH = "gfx950"
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={GPU_ARCH}",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
-HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-pthread", "-ffp-contract=off"]
 
 
 class BuildError(RuntimeError):
@@ -41,7 +41,7 @@ def _sources(sub: str, exts) -> List[str]:
 
 def _digest(sub: str) -> str:
     h = hashlib.sha256()
-    for path in _sources(sub, (".h", ".cpp", ".hip")):
+    for path in _sources(sub, (".h", ".cpp", ".hip")) + _sources("shared", (".h",)):   # both libraries include csrc/shared
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())

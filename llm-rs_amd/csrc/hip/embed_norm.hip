@@ -1,16 +1,17 @@
 // Token embedding into the 32-bit residual stream, and RMSNorm out of it.
 #include "common.h"
 
-// out[t, :] = float(table[tokens[t], :])   (reference: embed_batch_*, shaders/ops.metal:878-915)
+// out[t, :] = float(table[tokens[t], :]) * scale   (reference: embed_batch_*, shaders/ops.metal:878-915,
+// which has no scale: 1 there and for every architecture that does not ask for one)
 template <class T>
 __global__ void embed_rows_kernel(float* __restrict__ out, const T* __restrict__ table,
-                                  const int* __restrict__ tokens, int D, int V) {
+                                  const int* __restrict__ tokens, int D, int V, float scale) {
     int t = blockIdx.x;
     int row = tokens[t];
     row = row < 0 ? 0 : (row >= V ? V - 1 : row);  // the host has checked ids; never read outside the table
     const T* src = table + (size_t)row * D;
     float* dst = out + (size_t)t * D;
-    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = to_f32(src[d]);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = to_f32(src[d]) * scale;
 }
 
 // One block per row: ss = sum x^2 in 32-bit, inv = 1/sqrt(ss/D + eps),
@@ -93,13 +94,13 @@ __global__ void rmsnorm_rows_reg_kernel(T* __restrict__ out, const float* __rest
 }
 
 extern "C" int llmrs_embed_rows(hipStream_t stream, int dtype, float* out, const void* table, const int* tokens,
-                                int n_tokens, int D, int V) {
+                                int n_tokens, int D, int V, float scale) {
     LLMRS_REQUIRE(n_tokens >= 0 && D > 0 && V > 0, "embed_rows: bad sizes T=%d D=%d V=%d", n_tokens, D, V);
     if (n_tokens == 0) return 0;
     if (dtype == LLMRS_F32)
-        embed_rows_kernel<float><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, tokens, D, V);
+        embed_rows_kernel<float><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, tokens, D, V, scale);
     else if (dtype == LLMRS_BF16)
-        embed_rows_kernel<bf16><<<n_tokens, 256, 0, stream>>>(out, (const bf16*)table, tokens, D, V);
+        embed_rows_kernel<bf16><<<n_tokens, 256, 0, stream>>>(out, (const bf16*)table, tokens, D, V, scale);
     else
         return llmrs_fail("embed_rows: unknown dtype %d", dtype);
     LLMRS_LAUNCH_CHECK("embed_rows");

@@ -1,14 +1,18 @@
 """Weights by tensor name from a model folder, with one error that names every
 missing, unexpected and mis-shaped tensor.  The reference looks tensors up by
 name and panics on the first missing one, without a shape check
-(src/arch/mod.rs:52-61, src/arch/llama.rs:80-94)."""
+(src/arch/mod.rs:52-61, src/arch/llama.rs:80-94); like it, this loader leaves
+alone what an architecture says its files may carry without the model using it
+(a stored table of rotation frequencies, the output matrix of a tied model):
+such names are reported in a line on stderr, not as an error."""
 from __future__ import annotations
 
+import fnmatch
 import json
 import os
 import sys
 import time
-from typing import Dict, Iterable, Mapping, Tuple
+from typing import Dict, Iterable, List, Mapping, Sequence, Tuple
 
 import torch
 
@@ -30,22 +34,38 @@ class WeightError(ValueError):
         super().__init__("\n".join(lines))
 
 
-def stored_dtype(dtype: torch.dtype) -> torch.dtype:
+def stored_dtype(dtype: torch.dtype, compute: torch.dtype = torch.bfloat16) -> torch.dtype:
     """How a tensor is kept: bfloat16, except that integer tables become int32 and
-    what the file stores in 32-bit (or wider) floating point stays float32."""
+    what the file stores in 32-bit (or wider) floating point stays float32.  A
+    float16 file read for an engine that computes in float32 is widened, not
+    rounded to bfloat16's eight bits: the 32-bit path sees the file's own values
+    (the reference picks its kernel by the tensor's own dtype,
+    src/backend/metal/mod.rs:503-512)."""
     if dtype in (torch.float32, torch.float64):
+        return torch.float32
+    if dtype == torch.float16 and compute == torch.float32:
         return torch.float32
     if dtype.is_floating_point:
         return torch.bfloat16
     return torch.int32
 
 
-def check_tensors(have: Mapping[str, Tuple[int, ...]], want: Mapping[str, Tuple[int, ...]], where: str = "") -> None:
+def check_tensors(have: Mapping[str, Tuple[int, ...]], want: Mapping[str, Tuple[int, ...]], where: str = "",
+                  ignorable: Sequence[str] = ()) -> List[str]:
+    """Raises one WeightError for everything that does not fit.  Names in `have` that the model does
+    not use are unexpected, unless they match one of the `ignorable` patterns: those are returned
+    (and said on stderr), the model just does not read them."""
     missing = [n for n in want if n not in have]
-    unexpected = [n for n in have if n not in want]
+    extra = [n for n in have if n not in want]
+    ignored = sorted(n for n in extra if any(fnmatch.fnmatchcase(n, pat) for pat in ignorable))
+    unexpected = [n for n in extra if n not in ignored]
     wrong = [(n, tuple(want[n]), tuple(have[n])) for n in want if n in have and tuple(have[n]) != tuple(want[n])]
     if missing or unexpected or wrong:
         raise WeightError(sorted(missing), sorted(unexpected), wrong, where)
+    if ignored:
+        shown = ", ".join(ignored[:4]) + (f", ... ({len(ignored)} in all)" if len(ignored) > 4 else "")
+        print(f"Warning: tensors the model does not use are left unread{' (' + where + ')' if where else ''}: {shown}", file=sys.stderr)
+    return ignored
 
 
 def open_model_files(folder: str) -> Dict[str, SafetensorsFile]:
@@ -69,18 +89,20 @@ def open_model_files(folder: str) -> Dict[str, SafetensorsFile]:
     return {name: f for name in f.names()}
 
 
-def load_tensors(folder: str, want: Mapping[str, Tuple[int, ...]], device="cpu", log=True) -> Dict[str, torch.Tensor]:
+def load_tensors(folder: str, want: Mapping[str, Tuple[int, ...]], device="cpu", log=True,
+                 compute: torch.dtype = torch.bfloat16, ignorable: Sequence[str] = ()) -> Dict[str, torch.Tensor]:
     """Read the tensors `want` names (name -> shape) from `folder`, check them all
-    before the first copy, and bring them to `device` in their kept dtype."""
+    before the first copy, and bring them to `device` in their kept dtype (which
+    depends on the dtype the engine computes in, see `stored_dtype`)."""
     start = time.time()
     where = open_model_files(folder)
-    check_tensors({n: f.entries[n][1] for n, f in where.items()}, want, folder)
+    check_tensors({n: f.entries[n][1] for n, f in where.items()}, want, folder, ignorable)
     out: Dict[str, torch.Tensor] = {}
     nbytes = 0
     for name in want:
         t = where[name].tensor(name)
         nbytes += t.numel() * t.dtype.itemsize
-        out[name] = t.to(device=device, dtype=stored_dtype(t.dtype))
+        out[name] = t.to(device=device, dtype=stored_dtype(t.dtype, compute))
     if log:
         dt = max(time.time() - start, 1e-9)
         print(f"Loaded model weights: {nbytes / 2**30:.2f} GB in {dt:.3f}s ({nbytes / 2**30 / dt:.1f} GB/s)", file=sys.stderr)
