@@ -11,14 +11,14 @@ capabilities of Leikoe/llm-rs for the Llama dense decoder.
             print(e.request, e.token, e.finished)
 """
 from .cache import CacheManager, FixedState, PagedKV
-from .config import (ConfigError, LlamaConfig, ModelSpec, LayerSpec, PartSpec, RunSpec, load_config,
+from .config import (ConfigError, ExtraPart, LlamaConfig, ModelSpec, LayerSpec, PartSpec, RunSpec, load_config,
                      config_from_dict, register_architecture)
 from .engine import Emitted, Engine, Model, OutOfPages, StepEntry, StepRunner, random_model_tensors
 from .kernels import KernelError, kernels, use_kernels
 from .sampling import SamplingParams
 from .weights import WeightError, load_tensors, write_model_folder
 
-__all__ = ["CacheManager", "FixedState", "PagedKV", "ConfigError", "LlamaConfig", "ModelSpec", "LayerSpec",
+__all__ = ["CacheManager", "FixedState", "PagedKV", "ConfigError", "ExtraPart", "LlamaConfig", "ModelSpec", "LayerSpec",
            "PartSpec", "RunSpec", "load_config", "config_from_dict", "register_architecture", "Emitted", "Engine", "Model",
            "OutOfPages", "StepEntry", "StepRunner", "random_model_tensors", "KernelError", "kernels",
            "use_kernels", "SamplingParams", "WeightError", "load_tensors", "write_model_folder"]

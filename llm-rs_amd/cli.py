@@ -55,6 +55,16 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
+def describe_model(config) -> str:
+    """One line about the model from what its configuration says of itself: the architecture's
+    name and every size among its config.json keys (the reference's line, src/arch/llama.rs:74-78,
+    without knowing which architecture it is)."""
+    d = config.to_dict()
+    name = (d.get("architectures") or ["model"])[0]
+    sizes = ", ".join(f"{k}={v}" for k, v in d.items() if isinstance(v, int) and not isinstance(v, bool) and not k.endswith("_token_id"))
+    return f"{name}: {sizes}"
+
+
 def parse_ids(text: str) -> List[int]:
     parts = [p for p in re.split(r"[\s,]+", text.strip()) if p]
     try:
@@ -90,8 +100,8 @@ def main(argv=None) -> int:
         print(f"Error: {e}", file=sys.stderr)
         return 1
     cfg = engine.config
-    print(f"llama model: dim={cfg.hidden_size}, layers={cfg.num_hidden_layers}, heads={cfg.num_attention_heads}, "
-          f"kv_heads={cfg.num_key_value_heads}, vocab={cfg.vocab_size}", file=sys.stderr)
+    print(describe_model(cfg), file=sys.stderr)
+    engine.measure_device_time()
     prompt = parse_ids(args.prompt)
     stop = parse_ids(args.stop) if args.stop else list(getattr(cfg, "eos_token_id", ()))
     print(f"Prompt tokens: {len(prompt)}", file=sys.stderr)
@@ -104,7 +114,12 @@ def main(argv=None) -> int:
     print(f"Prefill: {len(prompt)} tokens in {first:.2f}s ({len(prompt) / first:.1f} tok/s)", file=sys.stderr)
     print(" ".join(str(t) for t in out))
     rest = max(wall - first, 1e-9)
-    print(f"Generated: {len(out)} tokens in {rest:.2f}s ({max(len(out) - 1, 0) / rest:.1f} tok/s)", file=sys.stderr)
+    gpu = max(st.device_seconds - st.first_token_device_seconds, 0.0)     # the device's share of the decoding time
+    print(f"Generated: {len(out)} tokens in {rest:.2f}s ({max(len(out) - 1, 0) / rest:.1f} tok/s)  "
+          f"[gpu={gpu:.2f}s overhead={rest - gpu:.2f}s = {(rest - gpu) / rest * 100:.1f}%]", file=sys.stderr)
+    from .kernels import kernels
+    if kernels().times is not None:       # LLM_PERF: the per-kernel table (src/backend/metal/mod.rs:337-400)
+        kernels().times.dump()
     return 0
 
 

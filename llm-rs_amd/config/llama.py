@@ -162,4 +162,6 @@ class LlamaConfig:
             layers=layers, schedule=[RunSpec(i) for i in range(self.num_hidden_layers)],
             final_norm=PartSpec("rmsnorm", "model.norm", {"size": self.hidden_size, "eps": self.rms_norm_eps}),
             embedding_name="model.embed_tokens.weight",
-            head_name=None if self.tie_word_embeddings else "lm_head.weight")
+            head_name=None if self.tie_word_embeddings else "lm_head.weight",
+            # older files store the rotation's frequency table; files of tied models may repeat the token table
+            ignorable_tensors=("*.rotary_emb.inv_freq",) + (("lm_head.weight",) if self.tie_word_embeddings else ()))

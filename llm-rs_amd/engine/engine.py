@@ -14,10 +14,10 @@ from typing import Dict, List, Mapping, Optional, Sequence, Union
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheManager, CoreError
 from ..config import load_config
 from ..sampling import Sampler, SamplingParams
-from ..weights import load_tensors, random_tensors
+from ..weights import RandomTensors, load_tensors, random_tensors
 from .model import Model
 from .step import StepEntry, StepRunner
 
@@ -33,6 +33,8 @@ class GenerationStats:
     seconds: float = 0.0
     preemptions: int = 0
     first_token_seconds: float = 0.0
+    device_seconds: float = 0.0          # device time of the steps, when the engine was asked to measure it
+    first_token_device_seconds: float = 0.0
 
 
 @dataclass
@@ -89,6 +91,7 @@ class Engine:
         self._request_of: Dict[int, int] = {}              # slot -> request, for those the scheduler holds
         self._samples_randomly: set = set()                 # of those, the slots that do not decode greedily
         self._steps = 0
+        self._step_events: List[tuple] = []                 # (before the first kernel, after sampling) of measured steps
         # A full collection now, while nothing waits for it: building the model has made so many
         # objects that the collector would otherwise choose a moment among the first decode steps to
         # walk everything the libraries hold (measured: one pause of 40 ms there).
@@ -103,30 +106,53 @@ class Engine:
     @classmethod
     def from_folder(cls, folder: str, **kw) -> "Engine":
         config = load_config(folder)
-        probe = Model(config.model_spec(), torch.bfloat16, "cpu")
+        dtype = kw.get("dtype", "bfloat16")
+        if dtype not in _DTYPES:
+            raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
+        if torch.device(kw.get("device", "cuda")).type == "cuda":
+            from ..kernels import kernels
+            kernels()    # no GPU or no kernel library: say so before the first tensor is read
+        spec = config.model_spec()
+        probe = Model(spec, torch.bfloat16, "cpu")
         want = {n: t.shape for n, t in probe.tensors().items()}
-        tensors = load_tensors(folder, want, device="cpu", log=kw.get("log", False))
+        tensors = load_tensors(folder, want, device="cpu", log=kw.get("log", False), compute=_DTYPES[dtype],
+                               ignorable=spec.ignorable_tensors)
         return cls(config, tensors, **kw)
 
     @classmethod
     def from_random(cls, config, seed: int, **kw) -> "Engine":
-        """Random weights made where the engine lives, without a folder in between."""
-        tensors = random_model_tensors(config, seed, device=kw.get("device", "cuda"))
+        """Random weights made where the engine lives, without a folder in between, each tensor when
+        the model takes it: the same values as `random_model_tensors(config, seed)` gives on the host."""
+        probe = Model(config.model_spec(), torch.bfloat16, "cpu")
+        specs = probe.tensors()
+        tensors = RandomTensors({n: s.shape for n, s in specs.items()}, {n: s.kind for n, s in specs.items()}, seed,
+                                dtype=torch.bfloat16, device=kw.get("device", "cuda"))
         return cls(config, tensors, **kw)
 
+    def weights(self) -> Dict[str, torch.Tensor]:
+        """The model's tensors on the host, by file name and in the file's layout (`Model.weights`)."""
+        return self.model.weights()
+
     def _pages_from_memory(self, needs, page_size, fraction, max_requests):
-        """Pages that fit `fraction` of the memory still free after the weights
-        (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
-        from ..cache.spec import PagedKV
+        """Pages that fit `fraction` of the memory still free after the weights and after the
+        fixed-size state every request slot gets (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
+        from ..cache.spec import FixedState, PagedKV
         groups: Dict[PagedKV, int] = {}
+        state_bytes = 0
         for need, cache_of in needs:
             if isinstance(need, PagedKV) and cache_of is None:
                 groups[need] = groups.get(need, 0) + 1
+            elif isinstance(need, FixedState):
+                n = need.dtype.itemsize
+                for s in need.shape:
+                    n *= int(s)
+                state_bytes += n * max_requests
         if not groups:
             return []
         if self.device.type != "cuda":
             raise ValueError("num_pages must be given when the engine is not on a GPU")
         free, _ = torch.cuda.mem_get_info(self.device)
+        free = max(free - state_bytes, 0)
         per_token = sum(2 * n * need.kv_heads * need.head_dim * self.dtype.itemsize for need, n in groups.items())
         tokens = int(free * fraction) // per_token
         tokens = min(tokens, max_requests * self.max_seq_len)
@@ -157,11 +183,33 @@ class Engine:
             raise ValueError(f"token ids must be in [0, {vocab})")
         if max_new_tokens <= 0:
             raise ValueError("max_new_tokens must be positive")
+        # A request that could never run (longer than the positions allow, more pages at once than a
+        # pool has) is refused here, not at some later advance(), where it would stand in the way
+        # of every request behind it.
+        try:
+            self.cache.core.check_request(len(prompt), int(max_new_tokens))
+        except CoreError as e:
+            raise ValueError(str(e)) from None
         request = self._next_request
         self._next_request += 1
         self._waiting[request] = _Submitted(list(prompt), int(max_new_tokens),
                                             SamplingParams(temperature, top_k, top_p, seed), list(stop_token_ids))
         return request
+
+    def measure_device_time(self, on: bool = True) -> None:
+        """From now on every step of `advance()` is bracketed by two events on the device, and
+        `device_seconds()` says how long the device worked (the reference's gpu= figure, src/main.rs:141-150)."""
+        self.runner.time_device = bool(on)
+        self._step_events = []
+
+    def device_seconds(self) -> float:
+        """Device time of the steps since the last call (waits for the device)."""
+        if not self._step_events:
+            return 0.0
+        torch.cuda.synchronize(self.device)
+        total = sum(a.elapsed_time(b) for a, b in self._step_events) * 1e-3
+        self._step_events = []
+        return total
 
     def has_unfinished(self) -> bool:
         return bool(self._waiting) or bool(self._request_of)
@@ -205,7 +253,13 @@ class Engine:
             raise RuntimeError("the scheduler planned nothing although requests are waiting")
         sampled = []
         if n_want:
-            sampled = self.sampler.sample(logits, self.runner.ctx.sampling, not self._samples_randomly).cpu().numpy()
+            sampled = self.sampler.sample(logits, self.runner.ctx.sampling, not self._samples_randomly)
+        if self.runner.time_device and self.runner.started is not None:
+            done = torch.cuda.Event(enable_timing=True)
+            done.record()
+            self._step_events.append((self.runner.started, done))
+        if n_want:
+            sampled = sampled.cpu().numpy()
         self._steps += 1
         sampling_slots = [p[0] for p in plan if p[3]]
         finished = set(core.commit(sampled))
@@ -262,6 +316,7 @@ class Engine:
                 for e in self.advance():
                     if stats.first_token_seconds == 0.0:
                         stats.first_token_seconds = time.perf_counter() - t0
+                        stats.first_token_device_seconds = self.device_seconds()
                     if e.token is not None:
                         tokens[e.request].append(e.token)
                     if e.finished:
@@ -273,6 +328,7 @@ class Engine:
         if self.device.type == "cuda":
             torch.cuda.synchronize(self.device)
         stats.seconds = time.perf_counter() - t0
+        stats.device_seconds = stats.first_token_device_seconds + self.device_seconds()
         stats.steps = self._steps - steps0
         stats.generated_tokens = sum(len(r.tokens) for r in results)
         stats.preemptions = self.cache.core.preemptions() - preempt0

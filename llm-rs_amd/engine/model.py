@@ -10,7 +10,7 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..kernels import EPI_STORE_F32, kernels
-from ..parts import TensorSpec, build_block, build_norm
+from ..parts import TensorSpec, build_block, build_norm, place
 from ..weights import check_tensors
 
 
@@ -41,28 +41,49 @@ class Model:
         """Takes every tensor `tensors()` names; anything missing, left over or
         of another shape is reported in one error."""
         want = {n: t.shape for n, t in self.tensors().items()}
-        check_tensors({n: tuple(t.shape) for n, t in tensors.items()}, want)
+        # (a mapping that makes or reads its tensors only when asked says their shapes without doing so)
+        have = tensors.shapes() if hasattr(tensors, "shapes") else {n: tuple(t.shape) for n, t in tensors.items()}
+        check_tensors(have, want, ignorable=self.spec.ignorable_tensors)
         s = self.spec
-        self.embedding = tensors[s.embedding_name].to(device=self.device, dtype=self.dtype).contiguous()
+        self.embedding = place(tensors[s.embedding_name], self.device, self.dtype)
         # tied: the output matrix is the token table (src/arch/llama.rs:81)
-        self.head = self.embedding if s.head_name is None else \
-            tensors[s.head_name].to(device=self.device, dtype=self.dtype).contiguous()
+        self.head = self.embedding if s.head_name is None else place(tensors[s.head_name], self.device, self.dtype)
         for block in self.blocks:
             for part in block.parts():
                 part.load(tensors, self.device)
         self.final_norm.load(tensors, self.device)
 
+    def weights(self) -> Dict[str, torch.Tensor]:
+        """Every tensor of the model on the host, under its file name and in the file's layout
+        (what parts fused or reordered at load is undone), in the dtype the engine keeps it in:
+        what `load` would take again, and what another implementation can be given to compare."""
+        s = self.spec
+        out = {s.embedding_name: self.embedding.cpu()}
+        if s.head_name is not None:
+            out[s.head_name] = self.head.cpu()
+        for block in self.blocks:
+            for part in block.parts():
+                out.update(part.export())
+        out.update(self.final_norm.export())
+        return out
+
     def weight_bytes_per_step(self) -> int:
-        """Bytes of weights one step reads when it uses each once (the table's rows aside)."""
-        total = 0
+        """Bytes of weights one step reads when it uses each once (the table's rows aside):
+        every tensor a part of the schedule's layers holds, the final norm's, and the output matrix."""
         seen = set()
-        for run in self.spec.schedule:
-            for part in self.blocks[run.layer].parts():
-                for v in vars(part).values():
-                    if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
-                        seen.add(v.data_ptr())
-                        total += v.numel() * v.element_size()
-        total += self.head.numel() * self.head.element_size() + self.final_norm.weight.numel() * 4
+
+        def held(part) -> int:
+            total = 0
+            for v in vars(part).values():
+                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                    seen.add(v.data_ptr())
+                    total += v.numel() * v.element_size()
+            return total
+
+        total = sum(held(part) for run in self.spec.schedule for part in self.blocks[run.layer].parts())
+        total += held(self.final_norm)
+        if self.head.data_ptr() not in seen:
+            total += self.head.numel() * self.head.element_size()
         return total
 
     def graph_safe(self) -> bool:
@@ -71,7 +92,7 @@ class Model:
 
     # -- cache ---------------------------------------------------------------
     def cache_needs(self) -> List[Tuple[object, Optional[int]]]:
-        return [(self.blocks[run.layer].mixer.cache_need(), run.cache_of) for run in self.spec.schedule]
+        return [(self.blocks[run.layer].cache_need(), run.cache_of) for run in self.spec.schedule]
 
     # -- one step --------------------------------------------------------------
     def forward(self, ctx, cache_views) -> Optional[torch.Tensor]:
@@ -80,7 +101,7 @@ class Model:
         k = kernels()
         T = ctx.n_tokens
         h = ctx.workspace("model.h", (T, self.spec.hidden_size), torch.float32)
-        k.embed_rows(h, self.embedding, ctx.tokens)
+        k.embed_rows(h, self.embedding, ctx.tokens, self.spec.embedding_scale)
         for i, run in enumerate(self.spec.schedule):
             ctx.run_index = i
             self.blocks[run.layer].forward(ctx, h, cache_views[i])
@@ -92,4 +113,6 @@ class Model:
         self.final_norm.forward(ctx, h, x, ctx.want_rows)
         logits = ctx.workspace("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
         k.gemm(x, self.head, logits, EPI_STORE_F32, ctx.gemm_workspace(x, self.head))
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
+            k.scale_softcap_rows(logits, self.spec.logit_scale, self.spec.logit_softcap)
         return logits

@@ -25,8 +25,18 @@ class TraceReplayer:
         if TRACE_ROUND_TO % page_size:
             raise ValueError(f"page_size {page_size} must divide {TRACE_ROUND_TO}")
         num_pages = max(-(-max_tokens // page_size), 1)
-        self.engine = Engine.from_folder(model_dir, dtype=dtype, device=device, page_size=page_size,
-                                         num_pages=num_pages, max_requests=max_requests)
+        self._bind(Engine.from_folder(model_dir, dtype=dtype, device=device, page_size=page_size,
+                                      num_pages=num_pages, max_requests=max_requests))
+
+    @classmethod
+    def for_engine(cls, engine: Engine) -> "TraceReplayer":
+        """Replays traces through an engine that exists already (one made from random weights, say)."""
+        self = cls.__new__(cls)
+        self._bind(engine)
+        return self
+
+    def _bind(self, engine: Engine) -> None:
+        self.engine = engine
         self.slot: Dict[str, int] = {}
         self.position: Dict[str, int] = {}
 

@@ -12,18 +12,77 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
+import os
+import sys
 from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
-from typing import Optional
+from typing import Dict, List, Optional
 
 import torch
 
 EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
+_EPI_NAMES = {EPI_STORE: "store", EPI_STORE_F32: "store32", EPI_ACCUM_F32: "add32", EPI_SWIGLU: "swiglu"}
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
 
+# MI355X, published: HBM3E 8 TB/s; dense matrix cores 2.5 PFLOP/s in bfloat16, 157.3 TFLOP/s in float32
+PEAK_HBM_BYTES = 8.0e12
+PEAK_FLOPS = {torch.bfloat16: 2.5e15, torch.float32: 157.3e12}
+
+
 class KernelError(RuntimeError):
     pass
+
+
+class KernelTimes:
+    """Per-kernel device time with the bytes each call has to move and the operations it has to
+    do, as the reference keeps when LLM_PERF is set (src/backend/metal/mod.rs:321-400): a pair of
+    events around every call, read when the table is asked for."""
+
+    def __init__(self):
+        self.calls: List[tuple] = []       # (label, bytes, flops, peak flops, start event, end event)
+
+    def add(self, label, nbytes, flops, peak, start, end):
+        self.calls.append((label, nbytes, flops, peak, start, end))
+
+    def rows(self) -> List[dict]:
+        """One row per label, most device time first; clears what was recorded."""
+        torch.cuda.synchronize()
+        acc: Dict[str, dict] = {}
+        for label, nbytes, flops, peak, start, end in self.calls:
+            r = acc.setdefault(label, {"kernel": label, "calls": 0, "seconds": 0.0, "bytes": 0, "flops": 0, "peak_flops": peak})
+            r["calls"] += 1
+            r["seconds"] += start.elapsed_time(end) * 1e-3
+            r["bytes"] += nbytes
+            r["flops"] += flops
+        self.calls = []
+        rows = sorted(acc.values(), key=lambda r: -r["seconds"])
+        for r in rows:
+            t = max(r["seconds"], 1e-12)
+            r["gb_per_s"] = r["bytes"] / t / 1e9
+            r["hbm_frac"] = r["bytes"] / t / PEAK_HBM_BYTES
+            r["tflops"] = r["flops"] / t / 1e12
+            r["flops_frac"] = r["flops"] / t / r["peak_flops"] if r["peak_flops"] else 0.0
+        return rows
+
+    def dump(self, file=None) -> List[dict]:
+        file = file or sys.stderr
+        rows = self.rows()
+        if not rows:
+            return rows
+        total = sum(r["seconds"] for r in rows)
+        print(f"  {'kernel':<34} {'calls':>6} {'GPU time':>10} {'% total':>8}  {'GB/s (% of 8 TB/s)':>20}  {'TFLOP/s (% of peak)':>20}", file=file)
+        print("  " + "-" * 106, file=file)
+        for r in rows:
+            t = f"{r['seconds'] * 1e3:.2f}ms" if r["seconds"] >= 1e-3 else f"{r['seconds'] * 1e6:.0f}us"
+            fl = f"{r['tflops']:.1f} ({r['flops_frac'] * 100:.1f}%)" if r["flops"] else "-"
+            print(f"  {r['kernel']:<34} {r['calls']:>6} {t:>10} {r['seconds'] / total * 100:>7.1f}%  "
+                  f"{r['gb_per_s']:>10.0f} ({r['hbm_frac'] * 100:>4.1f}%)  {fl:>20}", file=file)
+        all_bytes = sum(r["bytes"] for r in rows)
+        print("  " + "-" * 106, file=file)
+        print(f"  {'TOTAL':<34} {'':>6} {total * 1e3:>8.2f}ms {'100.0%':>8}  {all_bytes / total / 1e9:>10.0f} ({all_bytes / total / PEAK_HBM_BYTES * 100:>4.1f}%)",
+              file=file)
+        return rows
 
 
 def _code(dtype: torch.dtype) -> int:
@@ -48,7 +107,10 @@ class HipKernels:
         lib.llmrs_hip_error.restype = c_char_p
         V, I, F = c_void_p, c_int, c_float
         sigs = {
-            "llmrs_embed_rows": [V, I, V, V, V, I, I, I],
+            "llmrs_embed_rows": [V, I, V, V, V, I, I, I, F],
+            "llmrs_fill_normal": [V, I, V, c_size_t, ctypes.c_uint64, ctypes.c_uint64, F, F],
+            "llmrs_cast": [V, V, I, V, I, c_size_t],
+            "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
             "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
@@ -69,6 +131,9 @@ class HipKernels:
         if not self.arch.startswith("gfx950"):
             raise KernelError(f"the kernel library is built for gfx950, the device is {self.arch!r}")
         self.allow_mfma = True  # tests switch the matrix-core kernels off to compare paths
+        # LLM_PERF in the environment (the reference's switch): every call is timed on the device and
+        # steps are not recorded into graphs, so that each kernel can be seen by itself
+        self.times: Optional[KernelTimes] = KernelTimes() if os.environ.get("LLM_PERF") else None
         lib.llmrs_attention_chunk.restype = I
         lib.llmrs_gemm_workspace_floats.restype = ctypes.c_long
         lib.llmrs_gemm_workspace_floats.argtypes = [I, I, I]
@@ -86,16 +151,47 @@ class HipKernels:
         if rc != 0:
             raise KernelError(self.lib.llmrs_hip_error().decode())
 
+    def _run(self, label: str, nbytes: int, flops: int, dtype, fn, *args) -> None:
+        """Calls the library; with timing on, between two events, noting what the call has to move and to compute."""
+        if self.times is None:
+            return self._check(fn(*args))
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        self._check(fn(*args))
+        end.record()
+        self.times.add(label, int(nbytes), int(flops), PEAK_FLOPS.get(dtype, 0.0), start, end)
+
     @staticmethod
     def _stream() -> int:
         return torch.cuda.current_stream().cuda_stream
 
-    # out[t, :] = table[tokens[t], :] as float32
-    def embed_rows(self, out: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor) -> None:
+    # out[t, :] = table[tokens[t], :] * scale as float32
+    def embed_rows(self, out: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, scale: float = 1.0) -> None:
         assert out.dtype == torch.float32 and tokens.dtype == torch.int32 and table.is_contiguous() and out.is_contiguous()
         assert out.shape[0] == tokens.shape[0] and out.shape[1] == table.shape[1]
-        self._check(self.lib.llmrs_embed_rows(self._stream(), _code(table.dtype), _p(out), _p(table), _p(tokens),
-                                              tokens.shape[0], table.shape[1], table.shape[0]))
+        self._run("embed", out.numel() * (4 + table.element_size()), 0, None,
+                  self.lib.llmrs_embed_rows, self._stream(), _code(table.dtype), _p(out), _p(table), _p(tokens),
+                  tokens.shape[0], table.shape[1], table.shape[0], float(scale))
+
+    # out.flat[i] = mean + std * normal(seed, first + i): the same bits as the host library makes
+    def fill_normal(self, out: torch.Tensor, seed: int, mean: float, std: float, first: int = 0) -> None:
+        assert out.is_contiguous()
+        self._check(self.lib.llmrs_fill_normal(self._stream(), _code(out.dtype), _p(out), out.numel(), seed & (2**64 - 1),
+                                               int(first), float(mean), float(std)))
+
+    # dst = src in dst's dtype (float32, bfloat16; src may be float16 too), both on the device
+    def cast(self, dst: torch.Tensor, src: torch.Tensor) -> None:
+        codes = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+        assert dst.is_contiguous() and src.is_contiguous() and dst.numel() == src.numel()
+        if dst.dtype not in (torch.float32, torch.bfloat16) or src.dtype not in codes:
+            raise KernelError(f"no cast from {src.dtype} to {dst.dtype}")
+        self._check(self.lib.llmrs_cast(self._stream(), _p(dst), codes[dst.dtype], _p(src), codes[src.dtype], src.numel()))
+
+    # logits <- logits * scale, then cap * tanh(logits / cap) if cap > 0, in place
+    def scale_softcap_rows(self, logits: torch.Tensor, scale: float, cap: float) -> None:
+        assert logits.dtype == torch.float32 and logits.stride(1) == 1
+        self._check(self.lib.llmrs_scale_softcap_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
+                                                      logits.shape[1], float(scale), float(cap)))
 
     # out[i, :] = rmsnorm(x[rows[i] or i, :]) * weight
     def rmsnorm(self, out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
@@ -104,8 +200,9 @@ class HipKernels:
         n = out.shape[0]
         assert out.shape[1] == x.shape[1] == weight.shape[0]
         assert (rows is None and n == x.shape[0]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
-        self._check(self.lib.llmrs_rmsnorm(self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(rows),
-                                           n, x.shape[1], eps))
+        self._run("rmsnorm", n * x.shape[1] * (4 + out.element_size()) + x.shape[1] * 4, 5 * n * x.shape[1], None,
+                  self.lib.llmrs_rmsnorm, self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(rows),
+                  n, x.shape[1], eps)
 
     # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
     def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
@@ -115,10 +212,11 @@ class HipKernels:
         assert w.shape[1] == K and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1 and a.dtype == w.dtype
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
         assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
-        self._check(self.lib.llmrs_gemm(self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
-                                        M, N, K, epilogue, _p(workspace),
-                                        0 if workspace is None else workspace.numel() * workspace.element_size(),
-                                        int(self.allow_mfma)))
+        moved = (M * K + N * K) * a.element_size() + out.numel() * out.element_size() * (2 if epilogue == EPI_ACCUM_F32 else 1)
+        self._run(f"gemm {N}x{K} {_EPI_NAMES[epilogue]}", moved, 2 * M * N * K, a.dtype,
+                  self.lib.llmrs_gemm, self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
+                  M, N, K, epilogue, _p(workspace),
+                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma))
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:
@@ -128,10 +226,12 @@ class HipKernels:
             assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
             assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
             assert slot_map.dtype == torch.int32 and slot_map.shape[0] == qkv.shape[0]
-        self._check(self.lib.llmrs_rope_kv_write(
-            self._stream(), _code(qkv.dtype), _p(qkv), qkv.stride(0), _p(positions), _p(slot_map), _p(inv_freq),
-            rotary_dim, int(interleaved), _p(k_cache), _p(v_cache), qkv.shape[0], n_heads, n_kv_heads, head_dim,
-            page_size, num_pages, int(write_kv)))
+        T = qkv.shape[0]
+        self._run("rope_kv_write", T * (2 * n_heads + 4 * n_kv_heads) * head_dim * qkv.element_size(),
+                  5 * T * (n_heads + n_kv_heads) * rotary_dim, None, self.lib.llmrs_rope_kv_write,
+                  self._stream(), _code(qkv.dtype), _p(qkv), qkv.stride(0), _p(positions), _p(slot_map), _p(inv_freq),
+                  rotary_dim, int(interleaved), _p(k_cache), _p(v_cache), qkv.shape[0], n_heads, n_kv_heads, head_dim,
+                  page_size, num_pages, int(write_kv))
 
     def qkv_rope_cache(self, x, w, qkv, positions, slot_map, inv_freq, rotary_dim, k_cache, v_cache,
                        n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv, workspace=None) -> None:
@@ -143,11 +243,13 @@ class HipKernels:
         if write_kv:
             assert k_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
             assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
-        self._check(self.lib.llmrs_qkv_rope_cache(
-            self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(w), _p(qkv), qkv.stride(0), x.shape[0], x.shape[1],
-            _p(positions), _p(slot_map), _p(inv_freq), rotary_dim, _p(k_cache), _p(v_cache), n_heads, n_kv_heads,
-            head_dim, page_size, num_pages, int(write_kv), _p(workspace),
-            0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma)))
+        M, K, N = x.shape[0], x.shape[1], w.shape[0]
+        self._run(f"gemm {N}x{K} qkv+rope+cache", (M * K + N * K + M * N) * x.element_size(), 2 * M * N * K, x.dtype,
+                  self.lib.llmrs_qkv_rope_cache,
+                  self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(w), _p(qkv), qkv.stride(0), x.shape[0], x.shape[1],
+                  _p(positions), _p(slot_map), _p(inv_freq), rotary_dim, _p(k_cache), _p(v_cache), n_heads, n_kv_heads,
+                  head_dim, page_size, num_pages, int(write_kv), _p(workspace),
+                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma))
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1) -> None:
@@ -156,26 +258,34 @@ class HipKernels:
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
         T = q.shape[0]
         assert token_entry.shape[0] == T and positions.shape[0] == T and out.shape[0] == T
-        self._check(self.lib.llmrs_attention(
-            self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
-            _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
-            block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
-            _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-            int(n_single), int(self.allow_mfma)))
+        moved = flops = 0
+        if self.times is not None:      # what the call has to read depends on the step: ask the device (timing mode only)
+            keys = int(seq_lens.sum().item())
+            seen = int((positions + 1).sum().item()) if window <= 0 else int((positions + 1).clamp(max=window).sum().item())
+            moved = (2 * keys * n_kv_heads + 2 * T * n_heads) * head_dim * q.element_size()
+            flops = 4 * seen * n_heads * head_dim
+        self._run("attention decode" if n_single == block_table.shape[0] else "attention", moved, flops, q.dtype,
+                  self.lib.llmrs_attention,
+                  self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
+                  _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
+                  block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
+                  _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
+                  int(n_single), int(self.allow_mfma))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
         """`scratch`: 256 bytes per row let several blocks share a long row."""
         assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
-        self._check(self.lib.llmrs_argmax_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
-                                               logits.shape[1], _p(out), _p(scratch),
-                                               0 if scratch is None else scratch.numel() * scratch.element_size()))
+        self._run("argmax", logits.numel() * 4, 0, None,
+                  self.lib.llmrs_argmax_rows, self._stream(), _p(logits), logits.stride(0), logits.shape[0],
+                  logits.shape[1], _p(out), _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size())
 
     # words[i] = uniform (float bits), temperature (float bits), top_k, top_p (float bits) of row i
     def sample_rows(self, logits: torch.Tensor, words: torch.Tensor, out: torch.Tensor) -> None:
         assert logits.dtype == torch.float32 and logits.stride(1) == 1 and out.dtype == torch.int32
         assert words.dtype == torch.int32 and words.is_contiguous() and words.shape == (logits.shape[0], 4)
-        self._check(self.lib.llmrs_sample_rows(self._stream(), _p(logits), logits.stride(0), logits.shape[0],
-                                               logits.shape[1], _p(words), _p(out)))
+        self._run("sample", logits.numel() * 4, 0, None,
+                  self.lib.llmrs_sample_rows, self._stream(), _p(logits), logits.stride(0), logits.shape[0],
+                  logits.shape[1], _p(words), _p(out))
 
 
 _kernels = None

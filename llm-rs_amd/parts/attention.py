@@ -25,7 +25,7 @@ import torch
 
 from ..cache.spec import PagedKV
 from ..kernels import EPI_ACCUM_F32, EPI_STORE, kernels
-from .base import Mixer, TensorSpec, build_position, register_mixer
+from .base import Mixer, TensorSpec, build_position, place, register_mixer
 
 
 class Attention(Mixer):
@@ -60,25 +60,37 @@ class Attention(Mixer):
             t[self.name("v_proj.weight")] = TensorSpec((self.kv_size, self.hidden))
         return t
 
-    def _pair_neighbours(self, w: torch.Tensor, heads: int) -> torch.Tensor:
-        """Rows of a q or k weight reordered so that each rotation pair is (2i, 2i+1)."""
+    def _pair_neighbours(self, w: torch.Tensor, heads: int, undo: bool = False) -> torch.Tensor:
+        """Rows of a q or k weight reordered so that each rotation pair is (2i, 2i+1); `undo` puts them back."""
         rotary = self.position.rotary() if self.position is not None else None
         if rotary is None or rotary[2] or rotary[1] == 0:
             return w          # no rotation here, or the pairs are neighbours already
         rot = rotary[1]
         order = torch.stack([torch.arange(rot // 2), torch.arange(rot // 2) + rot // 2], dim=1).flatten()
-        order = torch.cat([order, torch.arange(rot, self.head_dim)]).to(w.device)
-        return w.view(heads, self.head_dim, -1)[:, order, :].reshape(w.shape)
+        order = torch.cat([order, torch.arange(rot, self.head_dim)])
+        if undo:
+            order = torch.argsort(order)
+        return w.view(heads, self.head_dim, -1)[:, order.to(w.device), :].reshape(w.shape)
 
     def load(self, tensors, device):
-        get = lambda n: tensors[self.name(n)].to(device=device, dtype=self.dtype)
+        get = lambda n: place(tensors[self.name(n)], device, self.dtype)
         parts = [self._pair_neighbours(get("q_proj.weight"), self.heads)]
         if self.kv_proj:
             parts += [self._pair_neighbours(get("k_proj.weight"), self.kv_heads), get("v_proj.weight")]
         self.w_qkv = torch.cat(parts, dim=0).contiguous()
-        self.w_o = tensors[self.name("o_proj.weight")].to(device=device, dtype=self.dtype).contiguous()
+        self.w_o = get("o_proj.weight")
         if self.position is not None:
             self.position.to(device)
+
+    def export(self):
+        w = self.w_qkv.cpu()
+        out = {self.name("q_proj.weight"): self._pair_neighbours(w[:self.q_size], self.heads, undo=True).contiguous(),
+               self.name("o_proj.weight"): self.w_o.cpu()}
+        if self.kv_proj:
+            k, v = w[self.q_size:self.q_size + self.kv_size], w[self.q_size + self.kv_size:]
+            out[self.name("k_proj.weight")] = self._pair_neighbours(k, self.kv_heads, undo=True).contiguous()
+            out[self.name("v_proj.weight")] = v.contiguous()
+        return out
 
     def cache_need(self):
         return PagedKV(self.kv_heads, self.head_dim, self.window)

@@ -22,6 +22,19 @@ import torch
 from ..config.spec import PartSpec
 
 
+def place(t: torch.Tensor, device, dtype: torch.dtype) -> torch.Tensor:
+    """`t` on `device` in `dtype`, contiguous.  The copy to the device is the library's; the
+    change of dtype there is this engine's cast kernel."""
+    device = torch.device(device)
+    if device.type != "cuda" or t.dtype == dtype:
+        return t.to(device=device, dtype=dtype).contiguous()
+    from ..kernels import kernels
+    src = t.to(device=device).contiguous()
+    dst = torch.empty(src.shape, dtype=dtype, device=device)
+    kernels().cast(dst, src)
+    return dst
+
+
 class TensorSpec(NamedTuple):
     shape: Tuple[int, ...]
     kind: str = "matrix"   # "matrix": N(0, 0.02) in random-weights mode; "norm": 1 + N(0, 0.1)
@@ -48,6 +61,13 @@ class Part:
 
     def load(self, tensors: Mapping[str, torch.Tensor], device) -> None:
         pass
+
+    def export(self) -> Dict[str, torch.Tensor]:
+        """The tensors `load` took, under their names and in the layout of the file they came
+        from (whatever `load` fused or reordered is undone), in the dtype the part keeps them in."""
+        if not self.tensors():
+            return {}
+        raise NotImplementedError(f"{type(self).__name__} cannot give its tensors back: it has no export()")
 
 
 class Norm(Part):
@@ -89,14 +109,29 @@ class FeedForward(Part):
 
 
 class Block:
-    """An arrangement of a mixer, a feed-forward and their norms around the residual stream."""
+    """An arrangement of parts around the residual stream.  It gets the layer's parts by the
+    names the `LayerSpec` gives them: "mixer", "feed_forward", "mixer_norm",
+    "feed_forward_norm" and whatever the spec lists under `extra`; `needs` names those an
+    arrangement cannot do without.  The layer's cache belongs to the part called "mixer"."""
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+    needs = ("mixer",)
+
+    def __init__(self, named: Mapping[str, Part]):
+        missing = [n for n in self.needs if named.get(n) is None]
+        if missing:
+            raise ValueError(f"block arrangement {type(self).__name__} needs the parts {', '.join(missing)}")
+        self.named: Dict[str, Part] = {n: p for n, p in named.items() if p is not None}
+        self.mixer: Optional[Mixer] = self.named.get("mixer")
+        self.feed_forward: Optional[FeedForward] = self.named.get("feed_forward")
+        self.mixer_norm: Optional[Norm] = self.named.get("mixer_norm")
+        self.feed_forward_norm: Optional[Norm] = self.named.get("feed_forward_norm")
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        return tuple(self.named.values())
+
+    def cache_need(self):
+        """What the layer asks of the cache manager: its mixer's need, or nothing."""
+        return None if self.mixer is None else self.mixer.cache_need()
 
     def forward(self, ctx, h: torch.Tensor, cache) -> None:
         raise NotImplementedError
@@ -147,7 +182,14 @@ def build_position(params: Optional[Mapping], dtype) -> Optional[PositionEncodin
     return _build(POSITIONS, "position encoding", params["kind"], params, dtype)
 
 
+_BUILDERS = {"mixer": build_mixer, "feed_forward": build_feed_forward, "norm": build_norm}
+
+
 def build_block(layer_spec, dtype) -> Block:
-    return _build(BLOCKS, "block arrangement", layer_spec.block,
-                  build_mixer(layer_spec.mixer, dtype), build_feed_forward(layer_spec.feed_forward, dtype),
-                  build_norm(layer_spec.mixer_norm, dtype), build_norm(layer_spec.feed_forward_norm, dtype))
+    opt = lambda build, spec: None if spec is None else build(spec, dtype)
+    named = {"mixer_norm": opt(build_norm, layer_spec.mixer_norm), "mixer": opt(build_mixer, layer_spec.mixer),
+             "feed_forward_norm": opt(build_norm, layer_spec.feed_forward_norm),
+             "feed_forward": opt(build_feed_forward, layer_spec.feed_forward)}
+    for extra in layer_spec.extra:
+        named[extra.name] = _BUILDERS[extra.family](extra.spec, dtype)
+    return _build(BLOCKS, "block arrangement", layer_spec.block, named)

@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import EPI_ACCUM_F32, EPI_SWIGLU, kernels
-from .base import FeedForward, TensorSpec, register_feed_forward
+from .base import FeedForward, TensorSpec, place, register_feed_forward
 
 
 class SwiGLU(FeedForward):
@@ -28,10 +28,15 @@ class SwiGLU(FeedForward):
                 self.name("down_proj.weight"): TensorSpec((self.hidden, self.inter))}
 
     def load(self, tensors, device):
-        gate = tensors[self.name("gate_proj.weight")].to(device=device, dtype=self.dtype)
-        up = tensors[self.name("up_proj.weight")].to(device=device, dtype=self.dtype)
+        gate = place(tensors[self.name("gate_proj.weight")], device, self.dtype)
+        up = place(tensors[self.name("up_proj.weight")], device, self.dtype)
         self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
-        self.w_down = tensors[self.name("down_proj.weight")].to(device=device, dtype=self.dtype).contiguous()
+        self.w_down = place(tensors[self.name("down_proj.weight")], device, self.dtype)
+
+    def export(self):
+        both = self.w_gate_up.cpu().view(self.inter, 2, self.hidden)
+        return {self.name("gate_proj.weight"): both[:, 0, :].contiguous(), self.name("up_proj.weight"): both[:, 1, :].contiguous(),
+                self.name("down_proj.weight"): self.w_down.cpu()}
 
     def forward(self, ctx, x, h):
         k = kernels()

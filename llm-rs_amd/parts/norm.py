@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import kernels
-from .base import Norm, TensorSpec, register_norm
+from .base import Norm, TensorSpec, place, register_norm
 
 
 class RMSNorm(Norm):
@@ -24,7 +24,10 @@ class RMSNorm(Norm):
     def load(self, tensors, device):
         # The reference wants norm weights in 32-bit (ops.metal:972); whatever the
         # file stores, the kernel multiplies by a float32 weight.
-        self.weight = tensors[self.name("weight")].to(device=device, dtype=torch.float32).contiguous()
+        self.weight = place(tensors[self.name("weight")], device, torch.float32)
+
+    def export(self):
+        return {self.name("weight"): self.weight.cpu()}
 
     def forward(self, ctx, h, out, rows=None):
         kernels().rmsnorm(out, h, self.weight, self.eps, rows)

@@ -18,8 +18,16 @@ class EmulatedKernels:
     def attention_scratch_floats(self, n_entries, n_heads, head_dim, max_seq_len):
         return 0
 
-    def embed_rows(self, out, table, tokens):
-        out.copy_(table[tokens.long()].float())
+    def embed_rows(self, out, table, tokens, scale=1.0):
+        out.copy_(table[tokens.long()].float() * scale)
+
+    def scale_softcap_rows(self, logits, scale, cap):
+        logits.mul_(scale)
+        if cap > 0:
+            logits.copy_(cap * torch.tanh(logits / cap))
+
+    def cast(self, dst, src):
+        dst.copy_(src.to(dst.dtype))
 
     def rmsnorm(self, out, x, weight, eps, rows=None):
         src = x if rows is None else x[rows.long()]

@@ -1,0 +1,99 @@
+"""The engine's host side with the emulated kernels in place of the device:
+requests that come and go through submit/advance, a request that can never run,
+export of the model's tensors, the seeded fill, and the order of checks at start."""
+import numpy as np
+import pytest
+import torch
+
+from emulated_kernels import EmulatedKernels
+from llm_rs_amd import Engine, KernelError, LlamaConfig, random_model_tensors, use_kernels, write_model_folder
+from llm_rs_amd.weights import fill_normal
+from plain_llama import plain_generate
+from tiny_configs import TINY_A, TINY_B
+
+
+@pytest.fixture
+def engine_a():
+    cfg = LlamaConfig.from_dict(TINY_A)
+    tensors = random_model_tensors(cfg, 4)
+    with use_kernels(EmulatedKernels()):
+        yield Engine(cfg, tensors, dtype="float32", device="cpu", page_size=4, num_pages=24, max_requests=3), tensors
+
+
+def test_a_request_that_can_never_run_is_refused_at_submit_and_blocks_nobody(engine_a):
+    eng, tensors = engine_a
+    prompts = [[5, 6, 7], [9, 1], [3, 3, 3, 3]]
+    got, ids = {}, []
+    ids.append(eng.submit(prompts[0], 5))
+    with pytest.raises(ValueError, match="positions"):
+        eng.submit(list(range(100)), 60)                    # 160 positions, the model has 128
+    with pytest.raises(ValueError, match="pages"):
+        eng.submit(list(range(90)), 20)                     # 28 pages at once, the pool has 24
+    ids += [eng.submit(p, 5) for p in prompts[1:]]
+    assert ids == [0, 1, 2], "a refused request takes no number and leaves nothing behind"
+    while eng.has_unfinished():
+        for e in eng.advance():
+            got.setdefault(e.request, []).append(e.token)
+    cfg = TINY_A
+    for r, p in zip(ids, prompts):
+        assert got[r] == plain_generate(cfg, tensors, p, 5)
+    core = eng.cache.core
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16")])
+def test_weights_gives_back_what_was_loaded(which, dtype):
+    cfg = LlamaConfig.from_dict({"A": TINY_A, "B": TINY_B}[which])
+    tensors = random_model_tensors(cfg, 11)
+    with use_kernels(EmulatedKernels()):
+        eng = Engine(cfg, tensors, dtype=dtype, device="cpu", page_size=4, num_pages=8, max_requests=2)
+    back = eng.weights()
+    assert sorted(back) == sorted(tensors)
+    for name, t in tensors.items():
+        want = t.float() if dtype == "float32" or name.endswith("norm.weight") else t
+        assert back[name].dtype == want.dtype and torch.equal(back[name], want), name
+    # and what comes back can be loaded again
+    with use_kernels(EmulatedKernels()):
+        again = Engine(cfg, back, dtype=dtype, device="cpu", page_size=4, num_pages=8, max_requests=2)
+        assert again.generate([[1, 2, 3]], max_new_tokens=4) == eng.generate([[1, 2, 3]], max_new_tokens=4)
+
+
+def test_seeded_fill_is_a_function_of_key_and_index():
+    a = fill_normal(torch.empty(100003), 77, 0.0, 1.0)
+    b = fill_normal(torch.empty(100003), 77, 0.0, 1.0)
+    c = fill_normal(torch.empty(100003), 78, 0.0, 1.0)
+    assert torch.equal(a, b) and not torch.equal(a, c)
+    # a longer tensor of the same key starts with the same values: element i depends on (key, i) alone,
+    # however the range was shared out over threads
+    long = fill_normal(torch.empty(400000), 77, 0.0, 1.0)
+    assert torch.equal(long[:100003], a)
+    # bfloat16 is the float32 value rounded once, to nearest even
+    h = fill_normal(torch.empty(100003, dtype=torch.bfloat16), 77, 0.0, 1.0)
+    assert torch.equal(h, a.bfloat16())
+    shifted = fill_normal(torch.empty(1000), 77, 1.0, 0.1)
+    assert float((shifted - (1.0 + 0.1 * a[:1000])).abs().max()) < 2e-7      # one fused multiply-add
+
+
+def test_seeded_fill_is_normal():
+    z = fill_normal(torch.empty(4_000_000), 2024, 0.0, 1.0).double()
+    assert abs(float(z.mean())) < 2e-3 and abs(float(z.var()) - 1.0) < 4e-3
+    assert abs(float((z ** 3).mean())) < 1e-2 and abs(float((z ** 4).mean()) - 3.0) < 3e-2
+    for bound, mass in ((1.0, 0.317311), (2.0, 0.045500), (3.0, 0.002700)):
+        assert abs(float((z.abs() > bound).double().mean()) - mass) < 0.02 * mass + 1e-4
+    assert abs(float((z[1:] * z[:-1]).mean())) < 2e-3, "neighbours are uncorrelated"
+    assert float(z.abs().max()) < 5.8                      # u1 >= 2^-24: sqrt(48 ln 2) = 5.77
+
+
+def test_no_gpu_is_said_before_any_weight_is_read(tmp_path, monkeypatch):
+    """Without a GPU (or a kernel library) the engine says so first: a folder of many gigabytes is
+    not read only to find that out."""
+    if torch.cuda.is_available():
+        pytest.skip("this machine has a GPU")
+    cfg = LlamaConfig.from_dict(TINY_A)
+    write_model_folder(str(tmp_path), cfg, random_model_tensors(cfg, 0))
+    import llm_rs_amd.engine.engine as engine_module
+    read = []
+    monkeypatch.setattr(engine_module, "load_tensors", lambda *a, **k: read.append(1))
+    with pytest.raises(Exception, match="GPU|gfx950|kernel"):
+        Engine.from_folder(str(tmp_path))
+    assert read == []

@@ -611,3 +611,55 @@ def test_qkv_rope_cache(dtype, M, n_heads, n_kv, hd, rot, K):
             size = torch.cat([pair, size[..., rot:]], dim=-1)
         assert (err <= size * rel + floor).all(), f"{name}: max err {float(err.max())}"
     assert (qkv[:, N:] == 0).all(), "padding touched"
+
+
+# ---- utilities ----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n,key,mean,std", [(1, 5, 0.0, 0.02), (100003, 2**63 + 11, 1.0, 0.1), (3_000_001, 99, 0.0, 1.0)])
+def test_seeded_fill_is_the_same_on_host_and_device(dtype, n, key, mean, std):
+    """Random-weights mode makes a tensor where the engine lives; the plain implementation gets the
+    host's.  They are the same function of (key, index), so they must agree in every bit."""
+    from llm_rs_amd.weights import fill_normal
+    host = fill_normal(torch.empty(n, dtype=dtype), key, mean, std)
+    dev = fill_normal(torch.empty(n, dtype=dtype, device=DEV), key, mean, std)
+    assert torch.equal(dev.cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                       host.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+def test_random_model_is_the_same_on_host_and_device():
+    from llm_rs_amd import LlamaConfig, random_model_tensors
+    from tiny_configs import TINY_B
+    cfg = LlamaConfig.from_dict(TINY_B)
+    host, dev = random_model_tensors(cfg, 3), random_model_tensors(cfg, 3, device=DEV)
+    assert sorted(host) == sorted(dev)
+    for name in host:
+        assert torch.equal(host[name], dev[name].cpu()), name
+
+
+@pytest.mark.parametrize("src,dst", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+                                     (torch.float16, torch.bfloat16), (torch.float32, torch.float32)])
+def test_cast(src, dst):
+    x = rnd((7, 1001), torch.float32, 3, 5.0).to(src)
+    out = torch.empty((7, 1001), dtype=dst, device=DEV)
+    kernels().cast(out, x)
+    assert torch.equal(out, x.to(dst))
+
+
+def test_embed_rows_scaled():
+    table = rnd((50, 72), torch.bfloat16, 0)
+    tokens = torch.tensor([3, 49, 0], dtype=torch.int32, device=DEV)
+    out = torch.empty((3, 72), dtype=torch.float32, device=DEV)
+    kernels().embed_rows(out, table, tokens, 8.485281)
+    assert torch.equal(out, table[tokens.long()].float() * torch.tensor(8.485281, dtype=torch.float32))
+
+
+@pytest.mark.parametrize("scale,cap", [(0.25, 0.0), (1.0, 30.0), (0.5, 2.0)])
+def test_scale_softcap_rows(scale, cap):
+    x = rnd((5, 1003), torch.float32, 4, 20.0)
+    big = x.clone()[:, :1000]                     # a view with a row stride, as logits of a padded buffer would be
+    ref = big.double().cpu() * scale
+    if cap > 0:
+        ref = cap * torch.tanh(ref / cap)
+    kernels().scale_softcap_rows(big, scale, cap)
+    assert float((big.double().cpu() - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))

@@ -10,11 +10,11 @@ from types import SimpleNamespace
 import pytest
 import torch
 
-from llm_rs_amd import (Engine, FixedState, LayerSpec, ModelSpec, PartSpec, RunSpec, StepEntry, StepRunner,
+from llm_rs_amd import (Engine, ExtraPart, FixedState, LayerSpec, ModelSpec, PartSpec, RunSpec, StepEntry, StepRunner,
                         register_architecture)
 from llm_rs_amd.cache import CacheManager, PagedKV
-from llm_rs_amd.parts import (FeedForward, Mixer, PositionEncoding, TensorSpec, build_block, build_feed_forward,
-                              build_mixer, build_norm, build_position, register_feed_forward, register_mixer,
+from llm_rs_amd.parts import (Block, FeedForward, Mixer, PositionEncoding, TensorSpec, build_block, build_feed_forward,
+                              build_mixer, build_norm, build_position, register_block, register_feed_forward, register_mixer,
                               register_position)
 from plain_llama import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope, plain_swiglu
 
@@ -220,7 +220,7 @@ class ToyConfig:
         rope = {"kind": "rope", "head_dim": 32, "rotary_dim": 32, "theta": 1e4, "layout": "split_half"}
         att = lambda p, kvp: PartSpec("attention", p, {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 32,
                                                        "window": None, "position": rope, "kv_proj": kvp})
-        layers = [LayerSpec("prenorm", PartSpec("test_decay", "l0.mix", {"hidden_size": H, "decay": 0.9}), ffn("l0.mlp"), norm("l0.n1"), norm("l0.n2")),
+        layers = [LayerSpec("prenorm", PartSpec(self.d.get("decay_kind", "test_decay"), "l0.mix", {"hidden_size": H, "decay": 0.9}), ffn("l0.mlp"), norm("l0.n1"), norm("l0.n2")),
                   LayerSpec("prenorm", att("l1.att", True), ffn("l1.mlp"), norm("l1.n1"), norm("l1.n2")),
                   LayerSpec("prenorm", att("l2.att", False), ffn("l2.mlp"), norm("l2.n1"), norm("l2.n2"))]
         return ModelSpec(H, V, 256, layers, [RunSpec(0), RunSpec(1), RunSpec(0), RunSpec(2, cache_of=1)],
@@ -416,4 +416,166 @@ def test_toy_architecture_with_routing_and_another_position_encoding(dtype):
             # a token whose two best router logits are close may go to another expert in 16-bit: leave those rows out
             xs = (got - ref).abs().max(dim=1).values <= tol * max(float(ref.abs().max()), 1.0)
             assert int((~xs).sum()) <= 3, (cuts, int((~xs).sum()))
+        eng.close_request(slot)
+
+
+# ---- a stateful mixer whose decode steps may be recorded ----------------------------------------
+
+class RecordableDecayMixer(DecayMixer):
+    """The same mixer, with a decode step that launches only device work whose arguments do not
+    change between steps of one shape (the rows of the state are found through the slots on the
+    device): it says so, and the step function may then record and replay such steps."""
+    graph_safe = True
+
+    def forward(self, ctx, x, h, cache):
+        if ctx.n_single != ctx.n_entries:
+            return super().forward(ctx, x, h, cache)
+        slots = ctx.slots.long()
+        s = cache.state[slots] * self.decay + x.float()
+        cache.state.index_copy_(0, slots, s)
+        h += s @ self.w.T
+
+
+def test_decode_steps_of_a_stateful_mixer_are_recorded_and_replayed():
+    register_mixer("test_decay", DecayMixer)
+    register_mixer("test_decay_recordable", RecordableDecayMixer)
+    register_architecture("TestToyForCausalLM", ToyConfig)
+    H, V = 40, 90
+    from llm_rs_amd.engine import Model
+    cfg = ToyConfig({"architectures": ["TestToyForCausalLM"], "hidden_size": H, "vocab_size": V, "decay_kind": "test_decay_recordable"})
+    names = Model(cfg.model_spec(), torch.float32, "cpu").tensors()
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.2)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    eng = Engine(cfg, ws, dtype="float32", page_size=16, num_pages=32, max_requests=4)
+    assert eng.runner.use_graphs, "fixed-size state does not keep a model whose parts are all graph_safe from being recorded"
+    plain = Engine(ToyConfig({**cfg.d, "decay_kind": "test_decay"}), ws, dtype="float32", page_size=16, num_pages=32, max_requests=4)
+    assert not plain.runner.use_graphs, "a part that does not say graph_safe keeps the whole model eager"
+    seqs = {0: torch.randint(0, V, (40,), generator=torch.Generator().manual_seed(1)).tolist(),
+            1: torch.randint(0, V, (40,), generator=torch.Generator().manual_seed(2)).tolist()}
+    refs = {i: toy_reference(ws, t, H) for i, t in seqs.items()}
+    for round_ in range(2):                              # the second round reuses the slots: their state starts from zero again
+        slots = {i: eng.open_request() for i in seqs}
+        rows = {0: [], 1: []}
+        out = eng.step([StepEntry(slots[i], 0, seqs[i][:6], [5]) for i in seqs]).double().cpu()   # a prompt portion first
+        for i in seqs:
+            rows[i].append(out[i])
+        for p in range(6, 40):
+            out = eng.step([StepEntry(slots[i], p, [seqs[i][p]], [0]) for i in seqs]).double().cpu()
+            for i in seqs:
+                rows[i].append(out[i])
+        for i in seqs:
+            got, ref = torch.stack(rows[i]), refs[i][5:]
+            assert float((got - ref).abs().max()) <= 3e-5 * max(float(ref.abs().max()), 1.0), (round_, i)
+            eng.close_request(slots[i])
+    assert eng.runner.graph_replays >= 60, eng.runner.graph_replays
+
+
+# ---- other arrangements of a layer, a scaled embedding and bent logits ---------------------------
+
+class ParallelBlock(Block):
+    """One norm feeds both halves: x = norm(h); h += mixer(x); h += feed_forward(x)."""
+    needs = ("mixer", "feed_forward", "mixer_norm")
+
+    def forward(self, ctx, h, cache):
+        x = ctx.workspace("block.x", tuple(h.shape), self.mixer.dtype)
+        self.mixer_norm.forward(ctx, h, x)
+        self.mixer.forward(ctx, x, h, cache)
+        self.feed_forward.forward(ctx, x, h)
+
+
+class SandwichBlock(Block):
+    """A norm before and a norm after each half: h += post(mixer(pre(h))); the same for the feed-forward.
+    The two norms after come as the layer spec's extra parts."""
+    needs = ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm", "post_mixer_norm", "post_feed_forward_norm")
+
+    def _half(self, ctx, h, pre, part, post, *cache):
+        x = ctx.workspace("block.x", tuple(h.shape), self.mixer.dtype)
+        pre.forward(ctx, h, x)
+        t = ctx.workspace("sandwich.t", tuple(h.shape), torch.float32)
+        t.zero_()
+        part.forward(ctx, x, t, *cache)                  # parts add into the stream they are given
+        post.forward(ctx, t, x)
+        h += x.float()
+
+    def forward(self, ctx, h, cache):
+        self._half(ctx, h, self.mixer_norm, self.mixer, self.named["post_mixer_norm"], cache)
+        self._half(ctx, h, self.feed_forward_norm, self.feed_forward, self.named["post_feed_forward_norm"])
+
+
+class ToyShapesConfig:
+    def __init__(self, d):
+        self.d = d
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        H, V = self.d["hidden_size"], self.d["vocab_size"]
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": H, "eps": 1e-5})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": H, "intermediate_size": 2 * H})
+        rope = {"kind": "rope", "head_dim": 16, "rotary_dim": 16, "theta": 1e4, "layout": "split_half"}
+        att = lambda p: PartSpec("attention", p, {"hidden_size": H, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                                  "window": None, "position": rope})
+        layers = [LayerSpec("test_parallel", mixer=att("l0.att"), feed_forward=ffn("l0.mlp"), mixer_norm=norm("l0.n")),
+                  LayerSpec("test_sandwich", att("l1.att"), ffn("l1.mlp"), norm("l1.n1"), norm("l1.n2"),
+                            extra=(ExtraPart("post_mixer_norm", "norm", norm("l1.n1post")),
+                                   ExtraPart("post_feed_forward_norm", "norm", norm("l1.n2post"))))]
+        return ModelSpec(H, V, 256, layers, [RunSpec(0), RunSpec(1)], norm("final"), "embed", None,
+                         embedding_scale=math.sqrt(H), logit_scale=0.5, logit_softcap=4.0)
+
+
+def toy_shapes_reference(ws, tokens, H):
+    w = {k: v.double() for k, v in ws.items()}
+    T = len(tokens)
+    pos = torch.arange(T)
+    inv = plain_inv_freq(16, 1e4, None)
+    x = w["embed"][torch.tensor(tokens)] * float(torch.tensor(math.sqrt(H), dtype=torch.float32))
+
+    def att(xn, p):
+        q = plain_rope((xn @ w[f"{p}.q_proj.weight"].T).view(T, 4, 16), pos, inv)
+        k = plain_rope((xn @ w[f"{p}.k_proj.weight"].T).view(T, 2, 16), pos, inv)
+        v = (xn @ w[f"{p}.v_proj.weight"].T).view(T, 2, 16)
+        return plain_attention(q, k, v).reshape(T, 64) @ w[f"{p}.o_proj.weight"].T
+
+    mlp = lambda xn, p: plain_swiglu(xn, w[f"{p}.gate_proj.weight"], w[f"{p}.up_proj.weight"], w[f"{p}.down_proj.weight"])
+    n = lambda x, name: plain_rmsnorm(x, w[f"{name}.weight"], 1e-5)
+    xn = n(x, "l0.n")
+    x = x + att(xn, "l0.att") + mlp(xn, "l0.mlp")
+    x = x + n(att(n(x, "l1.n1"), "l1.att"), "l1.n1post")
+    x = x + n(mlp(n(x, "l1.n2"), "l1.mlp"), "l1.n2post")
+    logits = n(x, "final") @ w["embed"].T * 0.5
+    return 4.0 * torch.tanh(logits / 4.0)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_other_block_arrangements_scaled_embedding_and_bent_logits(dtype):
+    register_block("test_parallel", ParallelBlock)
+    register_block("test_sandwich", SandwichBlock)
+    register_architecture("TestToyShapesForCausalLM", ToyShapesConfig)
+    H, V = 64, 101
+    cfg = ToyShapesConfig({"architectures": ["TestToyShapesForCausalLM"], "hidden_size": H, "vocab_size": V})
+    from llm_rs_amd.engine import Model
+    probe = Model(cfg.model_spec(), torch.float32, "cpu")
+    names = probe.tensors()
+    assert {"l0.n.weight", "l1.n1post.weight", "l1.n2post.weight"} <= set(names) and "l0.n2.weight" not in names
+    with pytest.raises(ValueError, match="needs the parts"):
+        build_block(LayerSpec("test_sandwich", cfg.model_spec().layers[1].mixer), torch.float32)
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.2)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    eng = Engine(cfg, ws, dtype=dtype, page_size=16, num_pages=24, max_requests=4)
+    assert eng.model.weight_bytes_per_step() == sum(t.numel() * (4 if dtype == "float32" or n.endswith(".weight") and t.dim() == 1 else 2)
+                                                    for n, t in ws.items())
+    back = eng.weights()
+    assert all(torch.equal(back[n].float(), t.float()) for n, t in ws.items()), "every part gives its tensors back"
+    seq = torch.randint(0, V, (50,), generator=torch.Generator().manual_seed(8)).tolist()
+    ref = toy_shapes_reference(ws, seq, H)
+    assert float(ref.abs().max()) < 4.0 and float(ref.abs().max()) > 1.0, "the cap must bite for the test to see it"
+    tol = 3e-5 if dtype == "float32" else 2e-2
+    for cuts in ([50], [9, 2, 20, 1, 1, 17]):
+        slot, pos, rows = eng.open_request(), 0, []
+        for n in cuts:
+            rows.append(eng.step([StepEntry(slot, pos, seq[pos:pos + n], list(range(n)))]).double().cpu())
+            pos += n
+        got = torch.cat(rows)
+        assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), cuts
         eng.close_request(slot)

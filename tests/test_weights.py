@@ -34,6 +34,9 @@ def test_kept_dtypes():
     assert stored_dtype(torch.bfloat16) == torch.bfloat16 and stored_dtype(torch.float16) == torch.bfloat16
     assert stored_dtype(torch.float32) == torch.float32          # what is stored in 32-bit stays so
     assert stored_dtype(torch.int64) == torch.int32 and stored_dtype(torch.uint8) == torch.int32
+    # a float16 file keeps its own values when the engine computes in 32-bit
+    assert stored_dtype(torch.float16, torch.float32) == torch.float32
+    assert stored_dtype(torch.bfloat16, torch.float32) == torch.bfloat16
 
 
 def test_load_keeps_32_bit_and_makes_int32(tmp_path):
@@ -49,18 +52,61 @@ def test_one_error_lists_everything(tmp_path):
     del tensors["model.layers.0.mlp.up_proj.weight"]
     del tensors["model.norm.weight"]
     tensors["model.layers.1.self_attn.q_proj.weight"] = torch.zeros(64, 63).bfloat16()
-    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
-    tensors["lm_head.weight"] = torch.zeros(256, 64).bfloat16()      # the config ties the embeddings
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)   # left unread, not an error
+    tensors["model.layers.0.mlp.gate_proj.bias"] = torch.zeros(192)
+    tensors["model.layers.9.input_layernorm.weight"] = torch.zeros(64)
     write_model_folder(str(tmp_path), cfg, tensors)
     with pytest.raises(WeightError) as e:
         Engine.from_folder(str(tmp_path), device="cpu", num_pages=4)
     err = e.value
     assert err.missing == ["model.layers.0.mlp.up_proj.weight", "model.norm.weight"]
-    assert err.unexpected == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert err.unexpected == ["model.layers.0.mlp.gate_proj.bias", "model.layers.9.input_layernorm.weight"]
     assert err.wrong_shape == [("model.layers.1.self_attn.q_proj.weight", (64, 64), (64, 63))]
     text = str(err)
     for piece in ("missing (2)", "unexpected (2)", "expected [64, 64] got [64, 63]", "model.norm.weight"):
         assert piece in text
+
+
+def test_tensors_an_architecture_may_carry_unused_are_left_unread(tmp_path, capsys):
+    """Older Llama files store the rotation's frequencies, files of tied models may repeat the token
+    table as lm_head.weight: the folder loads, and a line says what was not read."""
+    cfg = LlamaConfig.from_dict(TINY_A)                 # tied
+    tensors = random_model_tensors(cfg, 0)
+    for i in range(2):
+        tensors[f"model.layers.{i}.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    write_model_folder(str(tmp_path / "a"), cfg, tensors)
+    from emulated_kernels import EmulatedKernels
+    from llm_rs_amd import use_kernels
+    with use_kernels(EmulatedKernels()):
+        eng = Engine.from_folder(str(tmp_path / "a"), device="cpu", dtype="float32", num_pages=8, page_size=4)
+        assert eng.generate([[1, 2, 3]], max_new_tokens=2)
+    said = capsys.readouterr().err
+    assert "left unread" in said and "rotary_emb.inv_freq" in said and "lm_head.weight" in said
+    # an untied model's files have no business holding a second head under another name
+    cfg_b = LlamaConfig.from_dict(TINY_B)
+    tensors = random_model_tensors(cfg_b, 0)
+    tensors["output.weight"] = torch.zeros(2)
+    with pytest.raises(WeightError, match="unexpected"):
+        Model(cfg_b.model_spec(), torch.float32, "cpu").load(tensors)
+
+
+def test_float16_file_is_exact_under_a_float32_engine(tmp_path):
+    cfg = LlamaConfig.from_dict(TINY_A)
+    g = torch.Generator().manual_seed(0)
+    tensors = {n: (t.float() + 1e-3 * torch.randn(t.shape, generator=g)).half() for n, t in random_model_tensors(cfg, 0).items()}
+    write_model_folder(str(tmp_path), cfg, tensors)
+    want = {n: tuple(t.shape) for n, t in tensors.items()}
+    exact = load_tensors(str(tmp_path), want, log=False, compute=torch.float32)
+    rounded = load_tensors(str(tmp_path), want, log=False, compute=torch.bfloat16)
+    name = "model.layers.0.mlp.down_proj.weight"
+    assert exact[name].dtype == torch.float32 and torch.equal(exact[name], tensors[name].float())
+    assert rounded[name].dtype == torch.bfloat16 and not torch.equal(rounded[name].float(), tensors[name].float())
+    from emulated_kernels import EmulatedKernels
+    from llm_rs_amd import use_kernels
+    with use_kernels(EmulatedKernels()):
+        eng = Engine.from_folder(str(tmp_path), device="cpu", dtype="float32", num_pages=8, page_size=4)
+    assert torch.equal(eng.model.blocks[0].feed_forward.w_down, tensors[name].float())
 
 
 def test_untied_model_needs_its_head():
