@@ -1,15 +1,27 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes]
 
-The default run is the Llama-3.1-8B shape with random bfloat16 weights: 8
+The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context already in the cache, decode K steps
 (one token per request per step, sampled greedily on the device, ids read back),
 and report decoded tokens a second.  The same line carries a 2,048-token prefill,
-the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+the decode step's share of the HBM roofline, decode at batch 1 and 64, and the
+host's share of a step (wall time minus the device's, from events around the step).
 A "step" is one decode step.  Counterpart of the reference's timing lines
 (src/main.rs:108-112, :141-150) and examples/bench_throughput.rs, in-process.
+
+The other workloads print one line of the same form each:
+  serve1b   Llama-3.2-1B shape, 256 requests at once through submit()/advance(), prompts
+            uniform in 128..4096 tokens, 256 new tokens each (continuous batching with
+            chunked prefill); value = generated tokens a second; a step is a scheduler step.
+  mixed70b  Llama-3.1-70B shape, all 80 layers: 16 requests decoding at context 4096 beside
+            one 2,048-token prompt portion, as one step; value = tokens a second of that step.
+  sizes     the 8B shape at further sizes: decode at context 8192 (batch 1/8/64) and at batch
+            128/256 (context 2048), each with its share of the HBM roofline.
+With LLM_PERF set in the environment every kernel call is timed by itself and a table
+by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
 import argparse
 import json
@@ -24,143 +36,326 @@ sys.path.insert(0, ROOT)
 PEAK_HBM = 8.0e12
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-LLAMA_8B = dict(
-    architectures=["LlamaForCausalLM"], num_hidden_layers=32, hidden_size=4096, num_attention_heads=32,
-    num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256, rope_theta=500000.0,
-    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
-                      original_max_position_embeddings=8192),
-    max_position_embeddings=8192, rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act="silu")
+
+def _llama(layers, hidden, heads, kv_heads, head_dim, inter, factor, tied):
+    return dict(
+        architectures=["LlamaForCausalLM"], num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads,
+        num_key_value_heads=kv_heads, head_dim=head_dim, intermediate_size=inter, vocab_size=128256, rope_theta=500000.0,
+        rope_scaling=dict(rope_type="llama3", factor=factor, low_freq_factor=1.0, high_freq_factor=4.0,
+                          original_max_position_embeddings=8192),
+        max_position_embeddings=8192, rms_norm_eps=1e-5, tie_word_embeddings=tied, hidden_act="silu")
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=2048, help="tokens each request has in the cache when decoding starts")
-    ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
-    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report")
-    ap.add_argument("--only", default="", choices=["", "prefill", "decode"], help="for profiling: time one phase only")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
-        return 2
+LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
+LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
+LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
+SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes")
 
-    import torch
-    from llm_rs_amd import Engine, LlamaConfig, StepEntry
 
-    full_layers = LLAMA_8B["num_hidden_layers"]
-    cfg_dict = dict(LLAMA_8B)
-    if args.layers:
-        cfg_dict["num_hidden_layers"] = args.layers
-    config = LlamaConfig.from_dict(cfg_dict)
-    points = [int(p) for p in args.points.split(",") if p]
-    max_batch = max([args.batch] + points)
-    page_size = 16
-    ctx_pages = -(-(args.context + args.steps + args.warmup + 8) // page_size)
-    num_pages = max_batch * ctx_pages + 8
-    t0 = time.time()
-    engine = Engine.from_random(config, seed=0, dtype=args.dtype, device="cuda:0", page_size=page_size,
-                                num_pages=num_pages, max_requests=max(max_batch, 8),
-                                max_batch_tokens=max(args.prefill_tokens, 2048))
-    torch.cuda.synchronize()
-    print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
-    vocab = config.vocab_size
-    gen = torch.Generator().manual_seed(0)
+def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
+    """The `config` of a line: every size of the shape by name, flat, at most 20 keys."""
+    d = SHAPES[model]
+    out = {"model": model, "global_batch": global_batch, "seq_len": seq_len, "parallelism": "single GPU",
+           "layers_run": layers_run, "layers_of_config": d["num_hidden_layers"], "hidden_size": d["hidden_size"],
+           "num_attention_heads": d["num_attention_heads"], "num_key_value_heads": d["num_key_value_heads"],
+           "head_dim": d["head_dim"], "intermediate_size": d["intermediate_size"], "vocab_size": d["vocab_size"],
+           "max_context": d["max_position_embeddings"], "page_size": page_size}
+    out.update(more)
+    assert len(out) <= 20 and all(not isinstance(v, (dict, list)) for v in out.values())
+    return out
 
-    def prompt(n):
-        return torch.randint(0, vocab, (n,), generator=gen).tolist()
 
-    def timed(fn, reps):
+def base_line(metric: str, value: float, steps: int, warmup: int, step_s: float, dtype: str, config: dict) -> dict:
+    return {"metric": metric, "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if dtype == "bfloat16" else "fp32",
+            "data": "synthetic (random weights, uniform random token ids)", "config": config}
+
+
+def roofline(bytes_per_step: float, step_s: float) -> dict:
+    achieved = bytes_per_step / step_s
+    return {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM, 4)}
+
+
+def host_share(wall_s: float, device_s: float) -> dict:
+    """Wall time of a step against the device's time for it (events before its first kernel and after
+    sampling): what is left is the host's (src/main.rs:141-150 prints the same three figures)."""
+    return {"wall_ms_per_step": round(wall_s * 1e3, 4), "device_ms_per_step": round(device_s * 1e3, 4),
+            "overhead_frac": round(max(wall_s - device_s, 0.0) / wall_s, 4)}
+
+
+def prefill_flops(d: dict, layers: int, T: int, start: int = 0) -> int:
+    """Operations of a portion of T tokens from position `start`: the products of every layer, QK^T and PV
+    over the keys each token sees, and the output matrix for one row."""
+    D, F, V = d["hidden_size"], d["intermediate_size"], d["vocab_size"]
+    Hq, Hkv = d["num_attention_heads"] * d["head_dim"], d["num_key_value_heads"] * d["head_dim"]
+    linear = 2 * T * layers * (D * (Hq + 2 * Hkv) + Hq * D + 3 * D * F) + 2 * V * D
+    keys_seen = T * start + T * (T + 1) // 2
+    return linear + layers * 2 * 2 * Hq * keys_seen
+
+
+def decode_line(args, layers, step_s, weight_bytes, cache_bytes_per_token, prefill_s, points, host) -> dict:
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    T = args.prefill_tokens
+    line = base_line(
+        f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens and batch "
+        f"{'/'.join(p.split('_b')[1] for p in points)} alongside",
+        args.batch / step_s, args.steps, args.warmup, step_s, args.dtype,
+        flat_config("Llama-3.1-8B shape", layers, args.batch, args.context, 16, prefill_tokens=T))
+    line["prefill"] = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
+                       "frac": round(prefill_flops(LLAMA_8B, layers, T) / prefill_s / PEAK_FLOPS[args.dtype], 4)}
+    cache_bytes = args.batch * (args.context + args.warmup + args.steps // 2) * cache_bytes_per_token
+    line["roofline"] = roofline(weight_bytes + cache_bytes, step_s)
+    line["points"] = points
+    line["host"] = host
+    return line
+
+
+def serve_line(args, layers, n_requests, prompt_tokens, generated, seconds, steps, device_s, preemptions, budget) -> dict:
+    line = base_line(
+        f"generated tok/s, {n_requests} requests at once, prompts uniform in 128..4096, {args.new_tokens} new tokens each "
+        f"(1B bf16, continuous batching with chunked prefill)",
+        generated / seconds, steps, 0, seconds / max(steps, 1), args.dtype,
+        flat_config("Llama-3.2-1B shape", layers, n_requests, 4096 + args.new_tokens, 16,
+                    max_batch_tokens=budget, new_tokens=args.new_tokens))
+    line["total_tokens_per_s"] = round((prompt_tokens + generated) / seconds, 1)
+    line["prompt_tokens"] = prompt_tokens
+    line["generated_tokens"] = generated
+    line["seconds"] = round(seconds, 3)
+    line["preemptions"] = preemptions
+    line["host"] = host_share(seconds / max(steps, 1), device_s / max(steps, 1))
+    return line
+
+
+def mixed_line(args, layers, step_s, weight_bytes, cache_bytes, host) -> dict:
+    n_dec, chunk, ctx = 16, 2048, 4096
+    tokens = n_dec + chunk
+    line = base_line(
+        f"tokens/s of one step: {n_dec} requests decoding at context {ctx} beside a {chunk}-token prompt portion (70B bf16)",
+        tokens / step_s, args.steps, args.warmup, step_s, args.dtype,
+        flat_config("Llama-3.1-70B shape", layers, n_dec + 1, ctx, 16, decodes=n_dec, prefill_chunk=chunk))
+    flops = prefill_flops(LLAMA_70B, layers, chunk, start=ctx - chunk) + \
+        n_dec * (prefill_flops(LLAMA_70B, layers, 1, start=ctx - 1) - 2 * 128256 * 8192) + n_dec * 2 * 128256 * 8192
+    line["compute"] = {"bound": "mfma", "achieved": round(flops / step_s / 1e12, 1), "peak": PEAK_FLOPS[args.dtype] / 1e12,
+                       "unit": "TFLOP/s", "frac": round(flops / step_s / PEAK_FLOPS[args.dtype], 4)}
+    line["roofline"] = roofline(weight_bytes + cache_bytes, step_s)
+    line["host"] = host
+    return line
+
+
+def sizes_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
+    """`value` and `ms_per_step` are the first point's; the others stand under `points`."""
+    first = next(iter(points))
+    line = base_line("decode tok/s of the 8B shape at further sizes (context 8192; batch 128 and 256), each with its share of the HBM roofline",
+                     points[first], args.steps, args.warmup, first_step_s, args.dtype,
+                     flat_config("Llama-3.1-8B shape", layers, 0, 8192, 16))
+    line["points"] = points
+    line["roofline_frac"] = fractions
+    return line
+
+
+# ---- measurements (need the GPU) -------------------------------------------------------------------------------
+
+class Bench:
+    def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int):
+        import torch
+        from llm_rs_amd import Engine, LlamaConfig
+        self.torch = torch
+        d = dict(shape)
+        if args.layers:
+            d["num_hidden_layers"] = args.layers
+        self.config = LlamaConfig.from_dict(d)
+        t0 = time.time()
+        self.engine = Engine.from_random(self.config, seed=0, dtype=args.dtype, device="cuda:0", page_size=16,
+                                         num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens)
         torch.cuda.synchronize()
+        print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+        self.gen = torch.Generator().manual_seed(0)
+
+    def prompt(self, n):
+        return self.torch.randint(0, self.config.vocab_size, (n,), generator=self.gen).tolist()
+
+    def timed(self, fn, reps):
+        self.torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(reps):
             fn()
-        torch.cuda.synchronize()
+        self.torch.cuda.synchronize()
         return (time.perf_counter() - t) / reps
 
-    # ---- prefill: one request, its whole prompt in one step, the last logits wanted
-    def prefill_once():
-        slot = engine.open_request()
-        engine.step([StepEntry(slot, 0, toks, [len(toks) - 1])])
-        engine.close_request(slot)
+    def fill(self, slot, tokens, chunk=2048):
+        from llm_rs_amd import StepEntry
+        at = 0
+        while at < len(tokens):
+            n = min(chunk, len(tokens) - at)
+            self.engine.step([StepEntry(slot, at, tokens[at:at + n], [])])
+            at += n
 
-    toks = prompt(args.prefill_tokens)
-    prefill_once()
-    prefill_s = timed(prefill_once, 3 if args.only != "decode" else 1)
-    spec = engine.model.spec
-    D, F, V, L = config.hidden_size, config.intermediate_size, vocab, config.num_hidden_layers
-    Hq, Hkv = config.num_attention_heads * config.head_dim, config.num_key_value_heads * config.head_dim
-    T = args.prefill_tokens
-    linear = 2 * T * L * (D * (Hq + 2 * Hkv) + Hq * D + 3 * D * F) + 2 * V * D
-    attention = L * 2 * 2 * Hq * T * (T + 1) // 2      # QK^T and PV over the causal half
-    prefill_flops = linear + attention
-    print(f"[bench] prefill {T} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
+    def device_seconds(self, fn, reps):
+        """Device time of `fn` (a step and its sampling), from an event before the step's first kernel to one after."""
+        torch, runner = self.torch, self.engine.runner
+        runner.time_device = True
+        pairs = []
+        for _ in range(reps):
+            fn()
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            pairs.append((runner.started, end))
+        runner.time_device = False
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / reps
 
-    # ---- decode
-    def decode_run(batch, steps, warmup):
+    def decode_run(self, batch, context, steps, warmup, with_device_time=False):
+        from llm_rs_amd import StepEntry
+        engine = self.engine
         slots = [engine.open_request() for _ in range(batch)]
         for s in slots:                         # fill each request's cache with `context` tokens
-            p, at = prompt(args.context), 0
-            while at < len(p):
-                n = min(2048, len(p) - at)
-                engine.step([StepEntry(s, at, p[at:at + n], [])])
-                at += n
-        pos = [args.context] * batch
-        last = [1] * batch
-        state = {"last": last}
+            self.fill(s, self.prompt(context))
+        pos = [context] * batch
+        state = {"last": [1] * batch}
 
         def one_step():
             entries = [StepEntry(s, pos[i], [state["last"][i]], [0]) for i, s in enumerate(slots)]
             logits = engine.step(entries)
-            ids = engine.sampler.sample(logits, engine.runner.ctx.sampling, True).cpu().tolist()
-            state["last"] = ids
+            ids = engine.sampler.sample(logits, engine.runner.ctx.sampling, True)
+            one_step.after = ids            # (the device-time event is recorded between the launch and the read-back)
+            state["last"] = ids.cpu().tolist()
             for i in range(batch):
                 pos[i] += 1
 
         for _ in range(warmup):
             one_step()
-        sec = timed(one_step, steps)
+        sec = self.timed(one_step, steps)
+        dev = self.device_seconds(one_step, min(steps, 16)) if with_device_time else None
         for s in slots:
             engine.close_request(s)
-        return sec
+        return sec, dev
 
+
+def run_decode8b(args) -> dict:
+    from llm_rs_amd import StepEntry
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    ctx_pages = -(-(args.context + args.steps + args.warmup + 24) // 16)
+    b = Bench(args, LLAMA_8B, max_batch * ctx_pages + 8, max(max_batch, 8), max(args.prefill_tokens, 2048))
+    engine = b.engine
+    toks = b.prompt(args.prefill_tokens)
+
+    def prefill_once():     # one request, its whole prompt in one step, the last logits wanted
+        slot = engine.open_request()
+        engine.step([StepEntry(slot, 0, toks, [len(toks) - 1])])
+        engine.close_request(slot)
+
+    prefill_once()
+    prefill_s = b.timed(prefill_once, 3 if args.only != "decode" else 1)
+    print(f"[bench] prefill {args.prefill_tokens} tokens: {prefill_s * 1e3:.1f} ms", file=sys.stderr, flush=True)
     if args.only == "prefill":
-        print(json.dumps({"prefill_ms": round(prefill_s * 1e3, 3), "tokens": T}))
-        return 0
-    step_s = decode_run(args.batch, args.steps, args.warmup)
-    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+        return {"prefill_ms": round(prefill_s * 1e3, 3), "tokens": args.prefill_tokens}
+    step_s, dev_s = b.decode_run(args.batch, args.context, args.steps, args.warmup, with_device_time=True)
+    print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step (device {dev_s * 1e3:.3f})", file=sys.stderr, flush=True)
     point_values = {}
-    for b in points:
-        s = decode_run(b, max(args.steps // 2, 8), max(args.warmup // 2, 2))
-        point_values[f"decode_b{b}"] = round(b / s, 1)
-        print(f"[bench] decode batch {b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    for p in points:
+        s, _ = b.decode_run(p, args.context, max(args.steps // 2, 8), max(args.warmup // 2, 2))
+        point_values[f"decode_b{p}"] = round(p / s, 1)
+        print(f"[bench] decode batch {p}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    return decode_line(args, b.config.num_hidden_layers, step_s, engine.model.weight_bytes_per_step(),
+                       engine.cache.bytes_per_token(), prefill_s, point_values, host_share(step_s, dev_s))
 
-    weight_bytes = engine.model.weight_bytes_per_step()
-    cache_bytes = args.batch * (args.context + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
-    achieved = (weight_bytes + cache_bytes) / step_s
-    value = args.batch / step_s
-    short = "bf16" if args.dtype == "bfloat16" else "fp32"
-    line = {
-        "metric": f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens and batch {'/'.join(str(p) for p in points)} alongside",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": short, "data": "synthetic (random weights, uniform random token ids)",
-        "config": {"model": "Llama-3.1-8B shape", "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single GPU", "layers_run": L, "layers_of_config": full_layers,
-                   "hidden_size": D, "num_attention_heads": config.num_attention_heads,
-                   "num_key_value_heads": config.num_key_value_heads, "head_dim": config.head_dim,
-                   "intermediate_size": F, "vocab_size": V, "max_context": config.max_position_embeddings,
-                   "page_size": page_size, "prefill_tokens": T},
-        "prefill": {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(prefill_flops / prefill_s / PEAK_FLOPS[args.dtype], 4)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM, 4)},
-        "points": point_values,
-    }
+
+def run_sizes(args) -> dict:
+    steps, warmup = max(args.steps // 2, 8), max(args.warmup // 2, 2)
+    cases = [(1, 8192), (8, 8192), (64, 8192), (128, 2048), (256, 2048)]
+    pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
+    b = Bench(args, LLAMA_8B, pages, 256, 2048)
+    weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
+    points, fractions, first_s = {}, {}, None
+    for batch, ctx in cases:
+        s, _ = b.decode_run(batch, ctx, steps, warmup)
+        first_s = s if first_s is None else first_s
+        key = f"decode_b{batch}_ctx{ctx}"
+        points[key] = round(batch / s, 1)
+        fractions[key] = round((weight_bytes + batch * (ctx + warmup + steps // 2) * per_token) / s / PEAK_HBM, 4)
+        print(f"[bench] {key}: {s * 1e3:.3f} ms/step, {fractions[key] * 100:.1f}% of the HBM roofline", file=sys.stderr, flush=True)
+    return sizes_line(args, b.config.num_hidden_layers, points, fractions, first_s)
+
+
+def run_serve1b(args) -> dict:
+    n, new = args.requests, args.new_tokens
+    b = Bench(args, LLAMA_1B, (n * (4096 + new)) // 16 + 64, n, args.max_batch_tokens)
+    engine, torch = b.engine, b.torch
+    lens = torch.randint(128, 4097, (n,), generator=b.gen).tolist()
+    prompts = [b.prompt(k) for k in lens]
+    engine.generate([prompts[0][:300], prompts[1][:40]], max_new_tokens=4)       # buffers grow, nothing is timed yet
+    engine.measure_device_time()
+    t0 = time.perf_counter()
+    out = engine.generate(prompts, max_new_tokens=new)
+    seconds = time.perf_counter() - t0
+    st = engine.last_stats
+    generated = sum(len(o) for o in out)
+    assert all(len(o) == new for o in out)
+    print(f"[bench] {n} requests: {st.prompt_tokens} prompt + {generated} generated tokens in {seconds:.2f}s, {st.steps} steps, "
+          f"graph replays {engine.runner.graph_replays}", file=sys.stderr, flush=True)
+    from llm_rs_amd.kernels import kernels
+    if kernels().times is not None:
+        kernels().times.dump()
+    return serve_line(args, b.config.num_hidden_layers, n, st.prompt_tokens, generated, seconds, st.steps, st.device_seconds,
+                      st.preemptions, args.max_batch_tokens)
+
+
+def run_mixed70b(args) -> dict:
+    from llm_rs_amd import StepEntry
+    n_dec, chunk, ctx = 16, 2048, 4096
+    b = Bench(args, LLAMA_70B, (n_dec + 1) * (ctx // 16 + 2) + 8, 24, 4096)
+    engine = b.engine
+    dec = [engine.open_request() for _ in range(n_dec)]
+    for s in dec:
+        b.fill(s, b.prompt(ctx - 1))
+    pre = engine.open_request()
+    ptoks = b.prompt(ctx)
+    b.fill(pre, ptoks[:ctx - chunk])
+    last = b.prompt(n_dec)
+
+    def step():     # positions are not advanced: the same step again writes the same cache slots
+        logits = engine.step([StepEntry(s, ctx - 1, [last[i]], [0]) for i, s in enumerate(dec)] +
+                             [StepEntry(pre, ctx - chunk, ptoks[ctx - chunk:], [chunk - 1])])
+        engine.sampler.sample(logits, engine.runner.ctx.sampling, True).cpu()
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    step_s = b.timed(step, args.steps)
+    dev_s = b.device_seconds(step, min(args.steps, 4))
+    print(f"[bench] mixed step: {step_s * 1e3:.2f} ms (device {dev_s * 1e3:.2f})", file=sys.stderr, flush=True)
+    cache_bytes = (n_dec * ctx + ctx) * engine.cache.bytes_per_token()
+    return mixed_line(args, b.config.num_hidden_layers, step_s, engine.model.weight_bytes_per_step(), cache_bytes,
+                      host_share(step_s, dev_s))
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 64; 8 for mixed70b)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default 8; 2 for mixed70b)")
+    ap.add_argument("--workload", default="decode8b", choices=WORKLOADS)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048, help="tokens each request has in the cache when decoding starts")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report (decode8b)")
+    ap.add_argument("--only", default="", choices=["", "prefill", "decode"], help="for profiling: time one phase only (decode8b)")
+    ap.add_argument("--requests", type=int, default=256, help="serve1b: requests submitted at once")
+    ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")
+    ap.add_argument("--max-batch-tokens", type=int, default=2048, help="serve1b: tokens a scheduler step may run")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    heavy = args.workload == "mixed70b"
+    args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
+    args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
+    line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes}[args.workload](args)
     print(json.dumps(line))
     return 0
 
