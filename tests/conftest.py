@@ -21,3 +21,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The worst logit error the model-level comparisons saw, as a part of the largest logit: the
+    bfloat16 bound in replay_checks.py is set from this line."""
+    try:
+        from replay_checks import WORST
+    except Exception:
+        return
+    if WORST:
+        terminalreporter.write_line("worst logit error against the plain implementation, of the largest logit: " +
+                                    ", ".join(f"{k} {v:.3e}" for k, v in sorted(WORST.items())))

@@ -126,35 +126,59 @@ def plain_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_do
 
 # ---- the model -----------------------------------------------------------------
 
+def plain_layer(cfg: dict, W: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor, pos: torch.Tensor,
+                inv_freq: torch.Tensor, layout: str = "split_half") -> torch.Tensor:
+    """One layer on one whole sequence x [T, hidden]: x += attention(norm(x)); x += swiglu(norm(x))
+    (src/arch/llama.rs:151-170).  `W` holds the layer's tensors under `prefix` + their names."""
+    H, D = cfg["num_attention_heads"], cfg["hidden_size"]
+    KV = cfg.get("num_key_value_heads") or H
+    d = cfg.get("head_dim") or D // H
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    T = x.shape[0]
+    p = prefix
+    xn = plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps)
+    q = (xn @ W[p + "self_attn.q_proj.weight"].T).view(T, H, d)
+    k = (xn @ W[p + "self_attn.k_proj.weight"].T).view(T, KV, d)
+    v = (xn @ W[p + "self_attn.v_proj.weight"].T).view(T, KV, d)
+    q, k = plain_rope(q, pos, inv_freq, layout), plain_rope(k, pos, inv_freq, layout)
+    o = plain_attention(q, k, v).reshape(T, H * d)
+    x = x + o @ W[p + "self_attn.o_proj.weight"].T
+    xn = plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps)
+    return x + plain_swiglu(xn, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+
+
 def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
                   compute: torch.dtype = torch.float64, layout: str = "split_half",
                   position_offset: int = 0) -> torch.Tensor:
     """Logits [T, vocab] for one whole sequence from position 0 (or `position_offset`).  Layer loop of
     src/arch/llama.rs:150-171, final norm and output matrix of :135-139; tied
     embeddings reuse the token table (:81)."""
-    W = {n: t.to(compute) for n, t in weights.items()}
+    return plain_forward_streamed(cfg, lambda name: weights[name], [tokens], compute, layout, position_offset)[0]
+
+
+def plain_forward_streamed(cfg: dict, tensor_of, sequences: Sequence[Sequence[int]], compute: torch.dtype = torch.float64,
+                           layout: str = "split_half", position_offset: int = 0) -> List[torch.Tensor]:
+    """The same for several whole sequences, one after the other through each layer, with the
+    tensors asked for by name through `tensor_of(name)` when their layer is reached and dropped
+    after it: a model too large to hold in `compute` precision needs one layer's worth of room."""
     H, D = cfg["num_attention_heads"], cfg["hidden_size"]
-    KV = cfg.get("num_key_value_heads") or H
     d = cfg.get("head_dim") or D // H
-    eps = cfg.get("rms_norm_eps", 1e-5)
     inv_freq = plain_inv_freq(d, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
-    T = len(tokens)
-    pos = torch.arange(T) + position_offset
-    x = plain_embedding(W["model.embed_tokens.weight"], tokens)
+    table = tensor_of("model.embed_tokens.weight")
+    xs = [plain_embedding(table, tokens).to(compute) for tokens in sequences]
+    positions = [torch.arange(len(tokens)) + position_offset for tokens in sequences]
+    leaves = ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight",
+              "self_attn.o_proj.weight", "post_attention_layernorm.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight",
+              "mlp.down_proj.weight")
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        xn = plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps)
-        q = (xn @ W[p + "self_attn.q_proj.weight"].T).view(T, H, d)
-        k = (xn @ W[p + "self_attn.k_proj.weight"].T).view(T, KV, d)
-        v = (xn @ W[p + "self_attn.v_proj.weight"].T).view(T, KV, d)
-        q, k = plain_rope(q, pos, inv_freq, layout), plain_rope(k, pos, inv_freq, layout)
-        o = plain_attention(q, k, v).reshape(T, H * d)
-        x = x + o @ W[p + "self_attn.o_proj.weight"].T
-        xn = plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps)
-        x = x + plain_swiglu(xn, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
-    xn = plain_rmsnorm(x, W["model.norm.weight"], eps)
-    head = W["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else W["lm_head.weight"]
-    return xn @ head.T
+        W = {p + leaf: tensor_of(p + leaf).to(compute) for leaf in leaves}
+        xs = [plain_layer(cfg, W, p, x, pos, inv_freq, layout) for x, pos in zip(xs, positions)]
+        del W
+    norm = tensor_of("model.norm.weight").to(compute)
+    head = (table if cfg.get("tie_word_embeddings", False) else tensor_of("lm_head.weight")).to(compute)
+    eps = cfg.get("rms_norm_eps", 1e-5)
+    return [plain_rmsnorm(x, norm, eps) @ head.T for x in xs]
 
 
 # ---- sampling ------------------------------------------------------------------

@@ -8,7 +8,7 @@ import torch
 from llm_rs_amd import Engine, StepEntry
 from plain_llama import plain_forward, plain_generate, read_model_folder
 from replay_cases import random_tokens
-from replay_checks import TOLERANCE
+from replay_checks import TOLERANCE, logit_scale, note, tolerance_for
 from tiny_configs import CONFIGS, PAGE_SIZE, make_folder
 
 pytestmark = pytest.mark.gpu
@@ -30,11 +30,12 @@ def check_greedy_path(cfg, weights, prompt, out, dtype):
     """Every generated token is the plain implementation's choice given the same
     prefix, or (bfloat16) so close to it that rounding decides."""
     logits = plain_forward(cfg, weights, prompt + out)
-    scale = max(float(logits.abs().max()), 1.0)
+    scale = logit_scale(logits)
+    allowed = tolerance_for(dtype, cfg, weights, [prompt + out], [logits])
     for i, tok in enumerate(out):
         row = logits[len(prompt) - 1 + i]
         gap = float(row.max() - row[tok])
-        assert gap <= 2 * TOLERANCE[dtype] * scale, f"token {i}: engine chose {tok}, plain prefers {int(row.argmax())} by {gap}"
+        assert gap <= allowed * scale, f"token {i}: engine chose {tok}, plain prefers {int(row.argmax())} by {gap}"
 
 
 @pytest.mark.parametrize("which", ["A", "B"])
@@ -74,9 +75,10 @@ def test_long_decoding(folders, dtype):
         rows.append(eng.step([StepEntry(s, i, [toks[i]], [0])]).clone())
     eng.close_request(s)
     got = torch.cat(rows).double().cpu()
-    err = (got - ref).abs().max(dim=1).values / max(float(ref.abs().max()), 1.0)
-    bad = (err > TOLERANCE[dtype]).nonzero()
+    err = (got - ref).abs().max(dim=1).values / logit_scale(ref)
+    bad = (err > tolerance_for(dtype, cfg, weights, [toks], [ref])).nonzero()
     assert len(bad) == 0, f"first wrong position {int(bad[0])}: {float(err[int(bad[0])])}"
+    note(dtype, err.max())
     with pytest.raises(ValueError, match="beyond the model"):
         s = eng.open_request()
         eng.step([StepEntry(s, 0, toks + [1], [])])
@@ -90,12 +92,12 @@ def test_first_tokens(folders, dtype):
     eng = engine(folders[which], which, dtype)
     seqs = [random_tokens(cfg["vocab_size"], 3, seed=s) for s in range(4)]
     slots = [eng.open_request() for _ in seqs]
-    scale_tol = TOLERANCE[dtype]
+    scale_tol = tolerance_for(dtype, cfg, weights, seqs)
     for pos in range(3):
         out = eng.step([StepEntry(s, pos, [seq[pos]], [0]) for s, seq in zip(slots, seqs)]).double().cpu()
         for i, seq in enumerate(seqs):
             ref = plain_forward(cfg, weights, seq[:pos + 1])[-1]
-            assert float((out[i] - ref).abs().max()) <= scale_tol * max(float(ref.abs().max()), 1.0), (pos, i)
+            assert float((out[i] - ref).abs().max()) <= scale_tol * logit_scale(ref), (pos, i)
 
 
 def test_batching_and_seeds_do_not_change_outputs(folders):
@@ -198,7 +200,7 @@ def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
     """The tiny configurations never reach the kernels that wide layers get at 17 to 64 tokens (k ranges
     split over blocks, large tiles for few rows, a rotation kernel of its own after the qkv product).
     One layer of an 8B and of a 70B model's widths: the same decoded token alone, among 8, 24 and 48 requests and beside a prompt
-    portion, in bfloat16, against the float32 engine."""
+    portion, in float32 and bfloat16, against the plain implementation run on the tensors the engine gives back."""
     from llm_rs_amd import LlamaConfig
     cfg = LlamaConfig.from_dict(dict(
         architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=hidden, num_attention_heads=heads,
@@ -207,9 +209,11 @@ def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
     n_req, plen = 48, 24
     prompts = [random_tokens(2000, plen + 1, seed=300 + i) for i in range(n_req)]
     portion = random_tokens(2000, 150, seed=399)
-    rows = {}
+    rows, weights = {}, None
     for dtype in ("float32", "bfloat16"):
         eng = Engine.from_random(cfg, 5, dtype=dtype, page_size=16, num_pages=256, max_requests=64)
+        if weights is None:
+            weights = {n: t.double() for n, t in eng.weights().items()}     # made on the device, read back
         slots = [eng.open_request() for _ in range(n_req)]
         for s, p in zip(slots, prompts):
             eng.step([StepEntry(s, 0, p[:plen], [])])
@@ -218,17 +222,26 @@ def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
         got = {n: eng.step(decode(n)).float().cpu().clone() for n in (1, 8, 24, 48)}
         got["mixed"] = eng.step(decode(20) + [StepEntry(extra, 0, portion, [len(portion) - 1])]).float().cpu().clone()
         rows[dtype] = got
-    ref = rows["float32"][48]
-    scale = float(ref.abs().max())
-    for key, got in rows["float32"].items():                   # float32: any batch, the same to rounding
-        n = min(len(got), n_req) if key != "mixed" else 20
-        assert float((got[:n] - ref[:n]).abs().max()) <= TOLERANCE["float32"] * scale, key
-    for key, got in rows["bfloat16"].items():
-        n = len(got) if key != "mixed" else 20
-        err = float((got[:n] - ref[:n]).abs().max()) / scale
-        assert err <= TOLERANCE["bfloat16"], f"bfloat16 batch {key}: error {err:.3e} of the largest logit"
-    err = float((rows["bfloat16"]["mixed"][20] - rows["float32"]["mixed"][20]).abs().max()) / scale
-    assert err <= TOLERANCE["bfloat16"], f"prompt portion beside decoded tokens: {err:.3e}"
+        del eng
+    checked = [0, 7, 19, 23, 47]                                            # requests whose rows the plain implementation computes
+    plain = {i: plain_forward(cfg.to_dict(), weights, prompts[i])[-1] for i in checked}
+    plain_portion = plain_forward(cfg.to_dict(), weights, portion)[-1]
+    scale = max(logit_scale(r) for r in plain.values())
+    for dtype in ("float32", "bfloat16"):
+        allowed = tolerance_for(dtype, cfg.to_dict(), {n: t.bfloat16() if t.dim() > 1 else t.float() for n, t in weights.items()},
+                                [prompts[i] for i in checked[:3]] + [portion])
+        worst = 0.0
+        for key, got in rows[dtype].items():
+            n = min(len(got), n_req) if key != "mixed" else 20
+            for i in (i for i in checked if i < n):
+                err = float((got[i].double() - plain[i]).abs().max()) / scale
+                assert err <= allowed, f"{dtype} batch {key}, request {i}: error {err:.3e} of the largest logit, allowed {allowed:.3e}"
+                worst = max(worst, err)
+        err = float((rows[dtype]["mixed"][20].double() - plain_portion).abs().max()) / logit_scale(plain_portion)
+        assert err <= allowed, f"{dtype}: prompt portion beside decoded tokens: {err:.3e}, allowed {allowed:.3e}"
+        note(dtype, max(worst, err))
+        if dtype == "bfloat16":
+            note("bfloat16, of what is allowed", max(worst, err) / allowed)
 
 
 def test_requests_that_come_and_go(folders):
@@ -287,15 +300,22 @@ def test_bfloat16_under_preemption_follows_float32():
     assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
     del bf
     ref = Engine.from_random(cfg, 1, dtype="float32", page_size=16, num_pages=64, max_requests=2)
+    weights = {n: t.double() for n, t in ref.weights().items()}
+    shortest = sorted(range(len(prompts)), key=lambda i: len(prompts[i]) + len(out[i]))[:3]
+    allowed = tolerance_for("bfloat16", cfg.to_dict(), {n: t.bfloat16() if t.dim() > 1 else t.float() for n, t in weights.items()},
+                            [prompts[i] + out[i] for i in shortest])
     for i, (p, o) in enumerate(zip(prompts, out)):
         assert len(o) == limits[i]
         slot = ref.open_request()
         logits = ref.step([StepEntry(slot, 0, p + o, list(range(len(p) - 1, len(p) + len(o) - 1)))]).float()
         ref.close_request(slot)
-        scale = max(float(logits.abs().max()), 1.0)
+        if i in shortest:       # the float32 engine that judges here is itself judged by the plain implementation
+            plain = plain_forward(cfg.to_dict(), weights, p + o)[len(p) - 1:len(p) + len(o) - 1]
+            assert float((logits.double().cpu() - plain).abs().max()) <= TOLERANCE["float32"] * logit_scale(plain), i
+        scale = logit_scale(logits)
         chosen = logits[torch.arange(len(o)), torch.tensor(o, device=logits.device)]
         gap = float((logits.max(dim=1).values - chosen).max()) / scale
-        assert gap <= 2 * TOLERANCE["bfloat16"], f"request {i}: a chosen token lies {gap:.3e} of the logit scale below the float32 choice"
+        assert gap <= allowed, f"request {i}: a chosen token lies {gap:.3e} of the logit scale below the float32 choice (allowed {allowed:.3e})"
 
 
 def test_a_dropped_engine_is_freed_at_once(folders):

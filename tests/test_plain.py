@@ -70,6 +70,32 @@ def test_llama3_scaling_bands():
     assert ((mid > 1 / 8.0) & (mid < 1.0)).all() and (mid[:-1] >= mid[1:]).all(), "the band between blends monotonically"
 
 
+def test_llama3_scaling_blends_in_frequency_not_in_wavelength():
+    """Between the two band edges the new frequency is a straight line in L / wavelength (that is,
+    in the frequency itself) from freq / factor at the low edge to freq at the high edge.  A
+    frequency placed a quarter, a half and three quarters of the way between the edges must come out
+    scaled by (1 - s) / factor + s for s = 1/4, 1/2, 3/4 (0.344, 0.563, 0.781 with factor 8); blending along
+    the wavelength instead gives 0.160, 0.222, 0.364, and a line that runs the other way 0.781, 0.563, 0.344.
+    The same through the engine's own table (parts/rope.py), which the kernels multiply positions by."""
+    from llm_rs_amd.parts import rope_inv_freq
+    L, factor, low, high = 64.0, 8.0, 1.0, 4.0
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high, original_max_position_embeddings=int(L))
+    for s_want in (0.25, 0.5, 0.75):
+        turns = low + s_want * (high - low)             # L / wavelength of the frequency under test
+        freq = 2 * math.pi * turns / L
+        theta = freq ** -2.0                            # rotary_dim 4: pair 1 has frequency theta^(-1/2)
+        want = freq * ((1 - s_want) / factor + s_want)
+        got = float(plain_inv_freq(4, theta, sc)[1])
+        assert abs(got / want - 1) < 1e-6, (s_want, got / freq)
+        assert abs(float(rope_inv_freq(4, theta, sc)[1]) / want - 1) < 1e-6
+        in_wavelength = 1.0 / ((1 - s_want) * factor + s_want)      # what a blend along the wavelength would give
+        assert abs(got / freq - in_wavelength) > 0.05
+    # the edges themselves: kept at the high edge, divided by the factor at the low edge, no jump next to them
+    for turns, ratio in ((high * 1.0001, 1.0), (high * 0.9999, 1.0), (low * 1.0001, 1 / factor), (low * 0.9999, 1 / factor)):
+        freq = 2 * math.pi * turns / L
+        assert abs(float(plain_inv_freq(4, freq ** -2.0, sc)[1]) / freq - ratio) < 2e-4
+
+
 def test_attention_special_cases():
     T, H, d = 9, 4, 8
     q, k, v = (torch.randn(T, H, d, dtype=D) for _ in range(3))
