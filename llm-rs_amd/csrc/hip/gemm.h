@@ -24,6 +24,27 @@ struct QkvEpilogue {
     int page_size, num_pages, write_kv;
 };
 
+// RMSNorm without a kernel of its own, for steps of up to 16 tokens.  The product that adds into the
+// 32-bit stream (its last writer before a norm) also leaves, for the norm that follows,
+//   y[m, n]     = bfloat16(h[m, n] * weight[n])        the new row times the norm's weight, rounded once
+//   sumsq[m, p] = sum of h[m, n]^2 over the 16 features n of group p
+// (NextNorm); the product that follows takes y as its rows and multiplies each of its 32-bit sums by
+//   inv[m] = 1 / sqrt(sum_p sumsq[m, p] / K + eps)       (RowScale; the groups are added in a fixed order)
+// before its epilogue.  x W^T with x = h inv weight is the same number as inv (h weight) W^T; what
+// differs from the norm kernel's output is where the one rounding to bfloat16 falls (on h weight
+// instead of on h inv weight), not how many there are.
+struct NextNorm {
+    float* sumsq;          // [M, ceil(N / 16)]; null: nothing is left
+    bf16* y;               // [M, N], row stride ldy
+    int ldy;
+    const float* weight;   // [N]
+};
+struct RowScale {
+    const float* sumsq;    // [M, nparts]; null: no scale
+    int nparts;
+    float eps;
+};
+
 template <class T>
 __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int m, int n, float v) {
     if (epi == LLMRS_EPI_STORE) ((T*)out)[(size_t)m * ldc + n] = from_f32<T>(v);
@@ -35,6 +56,10 @@ __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int 
 // product, 0 when its shape or alignment is not theirs, -1 on error.
 // workspace: device memory for the partial sums of products that split K over blocks (may be null).
 // qkv: needed when epi is LLMRS_EPI_QKV; such a call is taken only by the kernels that fuse it.
+// scale, next: see RowScale and NextNorm; both only where llmrs_gemm_defers_norm(M, N, K) holds (next: with
+// LLMRS_EPI_ACCUM_F32 only).
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
-                         const QkvEpilogue* qkv = nullptr);
+                         const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr);
+// Whether the bfloat16 product of this shape goes to the kernel that can scale its rows' sums and leave a NextNorm.
+extern "C" int llmrs_gemm_defers_norm(int M, int N, int K);

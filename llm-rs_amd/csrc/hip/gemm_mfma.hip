@@ -71,7 +71,8 @@ template <int MT, int NT, int NW, int U>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
                                                               int ldc, int M, int N, int K, int epi,
-                                                              float* __restrict__ partial, QkvEpilogue qe, int rot_feats) {
+                                                              float* __restrict__ partial, QkvEpilogue qe, int rot_feats,
+                                                              RowScale rs, NextNorm nn) {
     extern __shared__ __attribute__((aligned(16))) unsigned char skinny_smem[];
     float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -105,13 +106,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     // out += sum: the old values of the tile this wave will finish are asked for now, so that
     // their trip to memory runs beside the weights' instead of after the sums are ready
     float old[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float next_w[4] = {0.0f, 0.0f, 0.0f, 0.0f};     // the next norm's weight for the same features, if something is left for it
     const bool old_ahead = epi == LLMRS_EPI_ACCUM_F32 && partial == nullptr && wave < MT * NT;
     if (old_ahead) {
         int m = (wave / NT) * 16 + row, n = n0 + (wave % NT) * 16 + 4 * g;
         if (m < M)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (n + r < N) old[r] = ((const float*)out)[(size_t)m * ldc + n + r];
+                if (n + r < N) {
+                    old[r] = ((const float*)out)[(size_t)m * ldc + n + r];
+                    if (nn.sumsq != nullptr) next_w[r] = nn.weight[n + r];
+                }
     }
     int j = wave;
     for (; j + (U - 1) * NW < cnt; j += U * NW) {
@@ -158,6 +163,33 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         }
         if (partial_turn) break;
     }
+    // A norm left to this product (RowScale, up to 16 rows, so MT = 1): the waves that will finish tiles find their
+    // row's scale now, so that the trip for the partial sums of squares runs beside the other waves' last rounds and
+    // the barrier.  The row's four lanes take every fourth group of four parts in ascending order and add their sums
+    // pairwise; every lane of a row, in every block, ends with the same bits.
+    float inv_row = 1.0f;
+    if (rs.sumsq != nullptr && wave < MT * NT) {
+        const float* sp = rs.sumsq + (size_t)min(row, M - 1) * rs.nparts;
+        float ss = 0.0f;
+        if (rs.nparts % 256 == 0 && ((uintptr_t)rs.sumsq & 15) == 0) {
+            // sixteen loads on their way at a time (the sums were written on other XCDs and come from memory)
+            for (int base = 4 * g; base < rs.nparts; base += 256) {
+                f32x4 p[16];
+#pragma unroll
+                for (int t = 0; t < 16; ++t) p[t] = *(const f32x4*)(sp + base + 16 * t);
+#pragma unroll
+                for (int t = 0; t < 16; ++t) { ss += p[t][0]; ss += p[t][1]; ss += p[t][2]; ss += p[t][3]; }
+            }
+        } else {
+            for (int i = 4 * g; i < rs.nparts; i += 16)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (i + q < rs.nparts) ss += sp[i + q];
+        }
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        inv_row = 1.0f / sqrtf(ss / (float)K + rs.eps);
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -174,7 +206,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
             float s = 0.0f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) s += red[(((w * MT + mt) * NT + nt) * 4 + r) * 64 + lane];
-            v[r] = s;
+            v[r] = s * inv_row;      // (1 without a norm left to this product; with one, MT = 1 and the lane's row is `row`)
         }
         int m = mt * 16 + row;
         int n = n0 + nt * 16 + 4 * g;
@@ -225,9 +257,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                 }
             }
         } else if (old_ahead && tile == wave) {
+            float ss = 0.0f;
+            bf16x4 y4;
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (n + r < N) ((float*)out)[(size_t)m * ldc + n + r] = old[r] + v[r];
+            for (int r = 0; r < 4; ++r) {
+                float nv = 0.0f;
+                if (n + r < N) {
+                    nv = old[r] + v[r];
+                    ((float*)out)[(size_t)m * ldc + n + r] = nv;
+                    ss = fmaf(nv, nv, ss);
+                    nv *= next_w[r];
+                }
+                y4[r] = (bf16)nv;
+            }
+            if (nn.sumsq != nullptr) {
+                // for the norm that follows (NextNorm).  The row's four lanes hold four features each of this tile's
+                // sixteen; they are all here: a row is in the batch for all of them or for none.
+                if (n + 3 < N) *(bf16x4*)(nn.y + (size_t)m * nn.ldy + n) = y4;
+                else
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < N) nn.y[(size_t)m * nn.ldy + n + r] = y4[r];
+                ss += __shfl_xor(ss, 16, 64);
+                ss += __shfl_xor(ss, 32, 64);
+                if (g == 0) nn.sumsq[(size_t)m * ((N + 15) / 16) + (n0 / 16 + nt)] = ss;
+            }
         } else {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -262,7 +315,8 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
 template <int MT, int NT, int NW, int U>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                           int M, int N, int K, int epi, const QkvEpilogue* qkv, int splits = 1,
-                          float* partial = nullptr, int rot_feats = 0) {
+                          float* partial = nullptr, int rot_feats = 0, const RowScale* scale = nullptr,
+                          const NextNorm* next = nullptr) {
     size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
     static bool configured = false;
     if (!configured) {
@@ -273,7 +327,8 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
     dim3 grid(ceil_div(N, NT * 16), splits);
     gemm_skinny_kernel<MT, NT, NW, U><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                           splits > 1 ? partial : nullptr,
-                                                                          qkv ? *qkv : QkvEpilogue{}, rot_feats);
+                                                                          qkv ? *qkv : QkvEpilogue{}, rot_feats,
+                                                                          scale ? *scale : RowScale{}, next ? *next : NextNorm{});
     if (splits > 1) {
         size_t pairs = (size_t)M * ((N + 1) / 2);
         gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
@@ -892,10 +947,24 @@ extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
     return 0;
 }
 
+// Up to 16 rows a bfloat16 product goes to the kernel for few rows with every tile of a block finished by a wave
+// of its own (not the widest weights, whose blocks take seven tiles): that kernel scales its rows' sums by a
+// norm left to it and leaves what the next norm needs.
+extern "C" int llmrs_gemm_defers_norm(int M, int N, int K) { return M >= 1 && M <= 16 && N >= 1 && K % 8 == 0; }
+
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
-                         const QkvEpilogue* qkv) {
-    if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return 0;
+                         const QkvEpilogue* qkv, const RowScale* scale, const NextNorm* next) {
+    if (K % 8 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) {
+        if (scale != nullptr || next != nullptr) { llmrs_fail("gemm: a deferred norm needs rows of a multiple of 8 values, 16-byte aligned"); return -1; }
+        return 0;
+    }
+    if (scale != nullptr || next != nullptr) {
+        bool ok = llmrs_gemm_defers_norm(M, N, K) && (scale == nullptr || (scale->sumsq != nullptr && scale->nparts >= 1 && scale->eps > 0.0f)) &&
+                  (next == nullptr || (epi == LLMRS_EPI_ACCUM_F32 && N < 16384 && next->sumsq != nullptr && next->y != nullptr &&
+                                       next->weight != nullptr && next->ldy >= N && next->ldy % 4 == 0 && ((uintptr_t)next->y & 7) == 0));
+        if (!ok) { llmrs_fail("gemm: a deferred norm is taken for up to 16 rows (what is left for the next one: with the += epilogue, under 16384 features), got M=%d N=%d K=%d epilogue %d", M, N, K, epi); return -1; }
+    }
     if (epi == LLMRS_EPI_QKV) {   // only the skinny kernel fuses it; its 8-byte stores need aligned rows
         if (M > 64 || qkv == nullptr || qkv->head_dim % 4 || ldc % 4 || ((uintptr_t)out & 7) ||
             ((uintptr_t)qkv->k_cache & 7) || qkv->rotary_dim % 4)
@@ -920,7 +989,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // Features per block (NT*16) grow with N and M: a block reads its tokens' rows
         // again for every 16*NT features, which costs L2 bandwidth once M is large, but
         // a weight with few rows needs small blocks to have enough of them.
-        // (Measured on MI355X at the 8B shapes; see profiles/.)
+        // (Measured on MI355X at the 8B shapes.)
         bool wide = N >= 16384;
         bool eight = !wide && K >= 2048;
         // A wide weight's blocks take 7 or 4 feature tiles: whichever number of blocks fills the
@@ -932,7 +1001,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // Other weights with long rows (measured at 8192 x 8192: 32.6 -> 28.6 us; nothing at K = 4096):
         // by groups of 64 features, which hold the features of any block that these weights get.
         int rot = wide ? 16 * wide_nt : (K >= 8192 ? 64 : 0);
-#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot)
+#define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, next)
         if (M <= 16) {
             if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else if (wide_nt == 7) SKINNY(1, 7, 4, 1); else SKINNY(1, 4, 4, 2); }
             else if (eight) { if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4); else SKINNY(1, 1, 8, 4); }   // 8192 x 28672: 90 -> 83 us

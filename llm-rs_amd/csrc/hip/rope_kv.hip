@@ -216,7 +216,9 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
 }
 
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
-                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma);
+                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma,
+                          const float* scale_sumsq, int scale_parts, float scale_eps, float* next_sumsq, void* next_y,
+                          int next_ldy, const float* next_weight);
 
 // qkv = x W^T for W = [q heads; k heads; v heads], then what llmrs_rope_kv_write does,
 // with pairs (2i, 2i+1): in one kernel when the product is one the rotation fuses into
@@ -226,7 +228,9 @@ extern "C" int llmrs_qkv_rope_cache(hipStream_t stream, int dtype, const void* x
                                     int row_stride, int M, int K, const int* positions, const int* slot_map,
                                     const float* inv_freq, int rotary_dim, void* k_cache, void* v_cache,
                                     int n_heads, int n_kv_heads, int head_dim, int page_size, int num_pages,
-                                    int write_kv, void* workspace, size_t workspace_bytes, int allow_mfma) {
+                                    int write_kv, void* workspace, size_t workspace_bytes, int allow_mfma,
+                                    const float* scale_sumsq, int scale_parts, float scale_eps) {
+    // scale_sumsq: a norm left to this product (RowScale in gemm.h); then only the fused kernel will do
     int N = (n_heads + 2 * n_kv_heads) * head_dim;
     LLMRS_REQUIRE(M >= 0 && K > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "qkv_rope_cache: bad sizes");
     LLMRS_REQUIRE(row_stride >= N && lda >= K, "qkv_rope_cache: row stride too short");
@@ -237,12 +241,14 @@ extern "C" int llmrs_qkv_rope_cache(hipStream_t stream, int dtype, const void* x
     if (dtype == LLMRS_BF16 && allow_mfma) {
         QkvEpilogue qe{positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, n_heads, n_kv_heads, head_dim,
                        rotary_dim, page_size, num_pages, write_kv};
+        RowScale rs{scale_sumsq, scale_parts, scale_eps};
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)x, lda, (const bf16*)w, qkv, row_stride, M, N, K,
-                                        LLMRS_EPI_QKV, nullptr, 0, &qe);
+                                        LLMRS_EPI_QKV, nullptr, 0, &qe, scale_sumsq ? &rs : nullptr);
         if (took != 0) return took < 0 ? -1 : 0;
     }
+    LLMRS_REQUIRE(scale_sumsq == nullptr, "qkv_rope_cache: a deferred norm needs the fused bfloat16 kernel (M=%d K=%d)", M, K);
     int rc = llmrs_gemm(stream, dtype, x, lda, w, qkv, row_stride, M, N, K, LLMRS_EPI_STORE, workspace, workspace_bytes,
-                        allow_mfma);
+                        allow_mfma, nullptr, 0, 0.0f, nullptr, nullptr, 0, nullptr);
     if (rc != 0) return rc;
     return llmrs_rope_kv_write(stream, dtype, qkv, row_stride, positions, slot_map, inv_freq, rotary_dim, 1, k_cache,
                                v_cache, M, n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv);

@@ -102,9 +102,18 @@ class Model:
         T = ctx.n_tokens
         h = ctx.workspace("model.h", (T, self.spec.hidden_size), torch.float32)
         k.embed_rows(h, self.embedding, ctx.tokens, self.spec.embedding_scale)
+        ctx.note_left(h, None)
         for i, run in enumerate(self.spec.schedule):
             ctx.run_index = i
-            self.blocks[run.layer].forward(ctx, h, cache_views[i])
+            block = self.blocks[run.layer]
+            # the norm that reads the stream after this block: the next block's first (the final norm reads
+            # gathered rows and runs as a kernel of its own)
+            later = self.spec.schedule[i + 1] if i + 1 < len(self.spec.schedule) else None
+            ctx.norm_after_block = self.blocks[later.layer].first_norm() if later is not None else None
+            block.forward(ctx, h, cache_views[i])
+            if not block.keeps_left_current:
+                ctx.note_left(h, None)
+        ctx.norm_after_block = ctx.upcoming_norm = None
         if ctx.n_want == 0:
             return None
         # Norm only the wanted rows, then the output matrix: the reference norms all

@@ -68,9 +68,41 @@ class StepContext:
         self.max_seq_len = 0                            # largest start + count among the entries
         self.n_single = 0                               # entries that bring one token
         self.device = runner.device
+        # A norm without a kernel of its own (steps of a few tokens): the part that adds into the stream last
+        # before a norm leaves what that norm needs (`room_for_next_norm`, `note_left`), and the norm hands it on
+        # to the product that follows (`left_for`).  `upcoming_norm` is the norm that will read the stream after
+        # the part that runs now (its block says so); `norm_after_block` the one after the block (the model says so).
+        self.upcoming_norm = None
+        self.norm_after_block = None
+        self._left = None               # kernels.NextNorm that describes the stream as it stands, or None
+        self._left_of = 0               # the stream it describes
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)
+
+    def room_for_next_norm(self, h: torch.Tensor, w: torch.Tensor):
+        """For a part about to add a product with weight `w` into the stream `h`: a `kernels.NextNorm` for that
+        product to fill (`kernels().gemm(..., leave=...)`; then `note_left(h, it)`), or None when the norm that
+        follows cannot be left to the next product (no such norm, other dtype, too many rows)."""
+        from ..kernels import NextNorm, kernels
+        k = kernels()
+        norm = self.upcoming_norm
+        weight = norm.deferred_weight() if norm is not None else None
+        defers = getattr(k, "gemm_defers_norm", None)
+        T, N = h.shape[0], w.shape[0]
+        if (weight is None or defers is None or w.dtype != torch.bfloat16 or N != h.shape[1] or weight.shape[0] != N
+                or N >= 16384 or not defers(T, N, w.shape[1])):
+            return None
+        return NextNorm(self.workspace("model.prenormed", (T, N), torch.bfloat16),
+                        self.workspace("model.sumsq", (T, -(-N // 16)), torch.float32), weight)
+
+    def note_left(self, h: torch.Tensor, left) -> None:
+        """`left` (a filled NextNorm, or None) is what describes `h` from now on."""
+        self._left, self._left_of = left, (h.data_ptr() if left is not None else 0)
+
+    def left_for(self, h: torch.Tensor):
+        """What the last product that added into `h` left for the norm that follows, or None."""
+        return self._left if self._left is not None and self._left_of == h.data_ptr() else None
 
     def gemm_workspace(self, a: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
         """Room for the partial sums of a @ w.T, when the kernel would split K over blocks."""

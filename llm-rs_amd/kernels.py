@@ -34,6 +34,26 @@ class KernelError(RuntimeError):
     pass
 
 
+class NormedRows:
+    """Rows whose norm is left to the product that takes them (steps of a few tokens; no norm kernel runs).
+    `y` [rows, K] holds the stream's rows times the norm's weight, rounded once to the activation type, and
+    `sumsq` [rows, parts] the sums of squares of each 16 consecutive features of the stream's rows: both left
+    by the product that added into the stream last.  The product multiplies each of its 32-bit sums by the row's
+    1 / sqrt(sum(sumsq) / K + eps): x W^T with x = h inv weight equals inv (h weight) W^T."""
+
+    def __init__(self, y: torch.Tensor, sumsq: torch.Tensor, eps: float):
+        self.y, self.sumsq, self.eps = y, sumsq, float(eps)
+        self.shape, self.dtype = y.shape, y.dtype
+
+
+class NextNorm:
+    """What a product that adds into the stream leaves for the norm that follows, see `NormedRows`:
+    `y` and `sumsq` to fill, `weight` the following norm's."""
+
+    def __init__(self, y: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor):
+        self.y, self.sumsq, self.weight = y, sumsq, weight
+
+
 class KernelTimes:
     """Per-kernel device time with the bytes each call has to move and the operations it has to
     do, as the reference keeps when LLM_PERF is set (src/backend/metal/mod.rs:321-400): a pair of
@@ -112,10 +132,11 @@ class HipKernels:
             "llmrs_cast": [V, V, I, V, I, c_size_t],
             "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
-            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V],
+            "llmrs_gemm_defers_norm": [I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
-            "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I],
+            "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I, V, I, F],
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
         }
@@ -142,6 +163,11 @@ class HipKernels:
     def gemm_workspace_floats(self, M: int, N: int, K: int) -> int:
         """Room that lets a product with too few blocks split K over blocks (the kernels' own rule)."""
         return int(self.lib.llmrs_gemm_workspace_floats(int(M), int(N), int(K)))
+
+    def gemm_defers_norm(self, M: int, N: int, K: int) -> bool:
+        """Whether the bfloat16 product of M rows with an [N, K] weight takes `NormedRows` as its rows and, adding
+        into the stream, leaves a `NextNorm` (that: for fewer than 16384 features)."""
+        return self.allow_mfma and bool(self.lib.llmrs_gemm_defers_norm(int(M), int(N), int(K)))
 
     def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int) -> int:
         """Room the split of single-token entries needs for its partial results."""
@@ -205,18 +231,34 @@ class HipKernels:
                   n, x.shape[1], eps)
 
     # out (epilogue) a @ w.T ; a: [M, K] rows may be strided, w: [N, K] dense
-    def gemm(self, a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
-             workspace: Optional[torch.Tensor] = None) -> None:
+    def gemm(self, a, w: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
+             workspace: Optional[torch.Tensor] = None, leave: Optional[NextNorm] = None) -> None:
+        """`a` may be `NormedRows`, and `leave` a `NextNorm` (with the += epilogue), where `gemm_defers_norm` holds."""
+        scale = None
+        if isinstance(a, NormedRows):
+            scale, a = a, a.y
+            assert scale.sumsq.dtype == torch.float32 and scale.sumsq.is_contiguous() and scale.sumsq.shape[0] == a.shape[0]
         M, K = a.shape
         N = w.shape[0]
         assert w.shape[1] == K and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1 and a.dtype == w.dtype
+        if leave is not None:
+            assert epilogue == EPI_ACCUM_F32 and N < 16384 and leave.sumsq.dtype == torch.float32 and leave.sumsq.is_contiguous()
+            assert tuple(leave.sumsq.shape) == (M, -(-N // 16)) and tuple(leave.y.shape) == (M, N) and leave.y.stride(1) == 1
+            assert leave.y.dtype == torch.bfloat16 and leave.weight.dtype == torch.float32 and leave.weight.shape[0] == N
+        if scale is not None or leave is not None:
+            assert a.dtype == torch.bfloat16 and self.gemm_defers_norm(M, N, K)
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
         assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
         moved = (M * K + N * K) * a.element_size() + out.numel() * out.element_size() * (2 if epilogue == EPI_ACCUM_F32 else 1)
-        self._run(f"gemm {N}x{K} {_EPI_NAMES[epilogue]}", moved, 2 * M * N * K, a.dtype,
+        label = f"gemm {N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{'+next' if leave is not None else ''}"
+        self._run(label, moved, 2 * M * N * K, a.dtype,
                   self.lib.llmrs_gemm, self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
                   M, N, K, epilogue, _p(workspace),
-                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma))
+                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma),
+                  None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
+                  0.0 if scale is None else scale.eps, None if leave is None else _p(leave.sumsq),
+                  None if leave is None else _p(leave.y), 0 if leave is None else leave.y.stride(0),
+                  None if leave is None else _p(leave.weight))
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:
@@ -237,19 +279,26 @@ class HipKernels:
                        n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv, workspace=None) -> None:
         """qkv = x @ w.T, q and k rotated by adjacent pairs (2i, 2i+1), k and v written to the cache: fused into
         one kernel where the product allows.  Afterwards only the q part of `qkv` is certain to be filled."""
-        assert x.stride(1) == 1 and qkv.stride(1) == 1 and w.is_contiguous() and x.dtype == w.dtype == qkv.dtype
         assert w.shape[0] == (n_heads + 2 * n_kv_heads) * head_dim and w.shape[1] == x.shape[1] and qkv.shape[0] == x.shape[0]
+        scale = None
+        if isinstance(x, NormedRows):
+            scale, x = x, x.y
+            assert scale.sumsq.dtype == torch.float32 and scale.sumsq.is_contiguous() and scale.sumsq.shape[0] == x.shape[0]
+            assert x.dtype == torch.bfloat16 and self.gemm_defers_norm(x.shape[0], w.shape[0], x.shape[1])
+        assert x.stride(1) == 1 and qkv.stride(1) == 1 and w.is_contiguous() and x.dtype == w.dtype == qkv.dtype
         assert rotary_dim == 0 or (inv_freq.dtype == torch.float32 and inv_freq.shape[0] == rotary_dim // 2)
         if write_kv:
             assert k_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
             assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
-        self._run(f"gemm {N}x{K} qkv+rope+cache", (M * K + N * K + M * N) * x.element_size(), 2 * M * N * K, x.dtype,
+        self._run(f"gemm {N}x{K} {'norm+' if scale is not None else ''}qkv+rope+cache", (M * K + N * K + M * N) * x.element_size(), 2 * M * N * K, x.dtype,
                   self.lib.llmrs_qkv_rope_cache,
                   self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(w), _p(qkv), qkv.stride(0), x.shape[0], x.shape[1],
                   _p(positions), _p(slot_map), _p(inv_freq), rotary_dim, _p(k_cache), _p(v_cache), n_heads, n_kv_heads,
-                  head_dim, page_size, num_pages, int(write_kv), _p(workspace),
-                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma))
+                        head_dim, page_size, num_pages, int(write_kv), _p(workspace),
+                  0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma),
+                  None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
+                  0.0 if scale is None else scale.eps)
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1) -> None:

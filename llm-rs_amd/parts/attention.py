@@ -95,6 +95,13 @@ class Attention(Mixer):
     def cache_need(self):
         return PagedKV(self.kv_heads, self.head_dim, self.window)
 
+    def takes_normed_rows(self, ctx, rows):
+        # the q/k/v product norms its rows itself where it is the fused kernel: a rotation it applies (or none)
+        fused = self.position is None or self.position.rotary() is not None
+        k = kernels()
+        return (fused and self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
+                and k.gemm_defers_norm(rows, self.w_qkv.shape[0], self.hidden))
+
     def forward(self, ctx, x, h, cache):
         k = kernels()
         T = x.shape[0]
@@ -123,7 +130,9 @@ class Attention(Mixer):
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
                     cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single)
-        k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o))
+        leave = ctx.room_for_next_norm(h, self.w_o)
+        k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o), **({} if leave is None else {"leave": leave}))
+        ctx.note_left(h, leave)
 
 
 register_mixer("attention", Attention)

@@ -62,6 +62,11 @@ class Part:
     def load(self, tensors: Mapping[str, torch.Tensor], device) -> None:
         pass
 
+    def takes_normed_rows(self, ctx, rows: int) -> bool:
+        """Whether `forward` may be given `kernels.NormedRows` (rows still to be normed, which the part's
+        first product norms itself) in place of the normed input `x`, for a step of `rows` tokens."""
+        return False
+
     def export(self) -> Dict[str, torch.Tensor]:
         """The tensors `load` took, under their names and in the layout of the file they came
         from (whatever `load` fused or reordered is undone), in the dtype the part keeps them in."""
@@ -74,6 +79,17 @@ class Norm(Part):
     def forward(self, ctx, h: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         """out[i] = norm(h[rows[i]]) (rows None: every row)."""
         raise NotImplementedError
+
+    def deferred_weight(self) -> Optional[torch.Tensor]:
+        """For a norm of the form x / rms(x) * weight: the float32 weight, which lets the product before it
+        prepare its rows and the product after it finish them (`kernels.NextNorm`, `kernels.NormedRows`);
+        None for any other norm."""
+        return None
+
+    def deferred(self, ctx, h: torch.Tensor):
+        """The norm of every row of `h`, not computed: a `kernels.NormedRows` for a part that
+        `takes_normed_rows`, or None when this norm cannot be left to the next product (then `forward` runs)."""
+        return None
 
 
 class PositionEncoding:
@@ -116,6 +132,16 @@ class Block:
 
     needs = ("mixer",)
 
+    # True only for an arrangement that vouches for this: when its `forward` returns, whatever
+    # `ctx.left_for(h)` gives describes `h` as it stands (the last thing that touched `h` was a part's
+    # `forward`, and what an earlier product left was dropped before that part ran).  The model drops
+    # it after any block that does not say so.
+    keeps_left_current = False
+
+    def first_norm(self) -> Optional[Norm]:
+        """The norm that reads the stream first when this block runs, if the block before may prepare it."""
+        return None
+
     def __init__(self, named: Mapping[str, Part]):
         missing = [n for n in self.needs if named.get(n) is None]
         if missing:
@@ -132,6 +158,22 @@ class Block:
     def cache_need(self):
         """What the layer asks of the cache manager: its mixer's need, or nothing."""
         return None if self.mixer is None else self.mixer.cache_need()
+
+    @staticmethod
+    def normed_input(ctx, h: torch.Tensor, norm: "Norm", part: Part, then: Optional["Norm"]):
+        """The input of `part`: norm(h), computed here, or left to the part's first product where the norm can be
+        deferred and the part takes such rows (a step of few tokens whose stream was last written by a product
+        that prepared this norm: then no norm kernel runs).  `then` is the norm that reads the stream after `part`."""
+        rows = norm.deferred(ctx, h) if part.takes_normed_rows(ctx, h.shape[0]) else None
+        # The part is about to change the stream: what was left stops describing it now.  (The rows handed over
+        # keep their own references; a part that leaves something for `then` notes it when it is done.)
+        ctx.note_left(h, None)
+        ctx.upcoming_norm = then
+        if rows is not None:
+            return rows
+        x = ctx.workspace("block.x", (h.shape[0], h.shape[1]), part.dtype)
+        norm.forward(ctx, h, x)
+        return x
 
     def forward(self, ctx, h: torch.Tensor, cache) -> None:
         raise NotImplementedError

@@ -10,13 +10,16 @@ from .base import Block, register_block
 
 class PreNormBlock(Block):
     needs = ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm")
+    keeps_left_current = True       # `normed_input` drops what was left before each part; the feed-forward runs last
+
+    def first_norm(self):
+        return self.mixer_norm
 
     def forward(self, ctx, h, cache):
-        x = ctx.workspace("block.x", (h.shape[0], h.shape[1]), self.mixer.dtype)
-        self.mixer_norm.forward(ctx, h, x)
-        self.mixer.forward(ctx, x, h, cache)
-        self.feed_forward_norm.forward(ctx, h, x)
-        self.feed_forward.forward(ctx, x, h)
+        after = ctx.norm_after_block
+        self.mixer.forward(ctx, self.normed_input(ctx, h, self.mixer_norm, self.mixer, self.feed_forward_norm), h, cache)
+        self.feed_forward.forward(ctx, self.normed_input(ctx, h, self.feed_forward_norm, self.feed_forward, after), h)
+        ctx.upcoming_norm = None
 
 
 register_block("prenorm", PreNormBlock)

@@ -38,11 +38,18 @@ class SwiGLU(FeedForward):
         return {self.name("gate_proj.weight"): both[:, 0, :].contiguous(), self.name("up_proj.weight"): both[:, 1, :].contiguous(),
                 self.name("down_proj.weight"): self.w_down.cpu()}
 
+    def takes_normed_rows(self, ctx, rows):
+        k = kernels()
+        return (self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
+                and k.gemm_defers_norm(rows, 2 * self.inter, self.hidden))
+
     def forward(self, ctx, x, h):
         k = kernels()
         act = ctx.workspace("mlp.act", (x.shape[0], self.inter), self.dtype)
         k.gemm(x, self.w_gate_up, act, EPI_SWIGLU, ctx.gemm_workspace(x, self.w_gate_up))
-        k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down))
+        leave = ctx.room_for_next_norm(h, self.w_down)
+        k.gemm(act, self.w_down, h, EPI_ACCUM_F32, ctx.gemm_workspace(act, self.w_down), **({} if leave is None else {"leave": leave}))
+        ctx.note_left(h, leave)
 
 
 register_feed_forward("swiglu", SwiGLU)

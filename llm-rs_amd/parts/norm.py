@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import kernels
+from ..kernels import NormedRows, kernels
 from .base import Norm, TensorSpec, place, register_norm
 
 
@@ -31,6 +31,15 @@ class RMSNorm(Norm):
 
     def forward(self, ctx, h, out, rows=None):
         kernels().rmsnorm(out, h, self.weight, self.eps, rows)
+
+    def deferred_weight(self):
+        return self.weight
+
+    def deferred(self, ctx, h):
+        left = ctx.left_for(h)
+        if left is None or left.weight is not self.weight or h.shape[1] != self.size or left.y.shape != h.shape:
+            return None         # nothing was left, or it was prepared for another norm
+        return NormedRows(left.y, left.sumsq, self.eps)
 
 
 register_norm("rmsnorm", RMSNorm)

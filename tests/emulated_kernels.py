@@ -39,8 +39,24 @@ class EmulatedKernels:
     def gemm_workspace_floats(M, N, K):
         return 0
 
-    def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None):
+    @staticmethod
+    def gemm_defers_norm(M, N, K):
+        return 1 <= M <= 16            # as the device: steps of up to 16 tokens leave their norms to the products
+
+    def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None, leave=None):
+        inv = None
+        if hasattr(a, "sumsq"):        # kernels.NormedRows: rows times the norm's weight, rounded; the scale comes after the sums
+            inv = 1.0 / torch.sqrt(a.sumsq.sum(-1, keepdim=True) / a.y.shape[1] + a.eps)
+            a = a.y
         acc = a.float() @ w.float().T
+        if inv is not None:
+            acc = acc * inv
+        if leave is not None:          # kernels.NextNorm, with the += epilogue
+            new = out + acc
+            pad = torch.zeros((new.shape[0], leave.sumsq.shape[1] * 16))
+            pad[:, :new.shape[1]] = new
+            leave.sumsq.copy_((pad * pad).view(new.shape[0], -1, 16).sum(-1))
+            leave.y.copy_((new * leave.weight).to(leave.y.dtype))
         if epilogue == EPI_STORE:
             out.copy_(acc.to(out.dtype))
         elif epilogue == EPI_STORE_F32:
@@ -82,6 +98,13 @@ class EmulatedKernels:
 
     def qkv_rope_cache(self, x, w, qkv, positions, slot_map, inv_freq, rotary_dim, k_cache, v_cache,
                        n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv, workspace=None):
+        if hasattr(x, "sumsq"):        # the device rotates the 32-bit sums and rounds once; so does this
+            full = torch.empty(qkv.shape, dtype=torch.float32)
+            self.gemm(x, w, full, EPI_STORE_F32)
+            self.rope_kv_write(full, positions, slot_map, inv_freq, rotary_dim, True, k_cache, v_cache,
+                               n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv)
+            qkv.copy_(full.to(qkv.dtype))
+            return
         self.gemm(x, w, qkv, EPI_STORE)
         self.rope_kv_write(qkv, positions, slot_map, inv_freq, rotary_dim, True, k_cache, v_cache,
                            n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv)

@@ -663,3 +663,120 @@ def test_scale_softcap_rows(scale, cap):
         ref = cap * torch.tanh(ref / cap)
     kernels().scale_softcap_rows(big, scale, cap)
     assert float((big.double().cpu() - ref).abs().max()) <= 1e-5 * max(1.0, float(ref.abs().max()))
+
+
+# ---- a norm without a kernel of its own -----------------------------------------------------------
+
+NORMED_SHAPES = [(8, 6144, 4096), (1, 6144, 4096), (1, 28672, 4096), (2, 28672, 4096), (8, 28672, 4096), (16, 28672, 4096),
+                 (5, 16400, 256), (3, 8192, 16384), (16, 520, 128), (7, 200, 2048), (9, 4096, 14336), (4, 96, 72)]
+
+
+def _left_for_norm(M, K, seed, weight):
+    """A 32-bit stream and what the product that wrote it last leaves for the norm that follows: the rows times the
+    norm's weight in bfloat16, and the sums of squares of each 16 features of a row."""
+    h = rnd((M, K), torch.float32, seed, 2.0)
+    parts = -(-K // 16)
+    padded = torch.zeros((M, parts * 16), dtype=torch.float32, device=DEV)
+    padded[:, :K] = h
+    y = torch.zeros((M, K + 8), dtype=torch.bfloat16, device=DEV)[:, :K]        # rows with a stride
+    y.copy_((h * weight).bfloat16())
+    return h, y, (padded * padded).view(M, parts, 16).sum(-1).contiguous()
+
+
+@pytest.mark.parametrize("epi", [EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU])
+@pytest.mark.parametrize("M,N,K", NORMED_SHAPES)
+def test_gemm_finishes_a_norm_left_to_it(M, N, K, epi):
+    """x W^T with x = h inv weight, computed as inv (h weight) W^T: against float64 on the same rounded rows (tight),
+    and against RMSNorm rounded to bfloat16 and then multiplied (the same up to where the one rounding falls)."""
+    from llm_rs_amd.kernels import NormedRows
+    k = kernels()
+    assert k.gemm_defers_norm(M, N, K)
+    eps = 1e-5
+    nw = rnd((K,), torch.float32, 41) * 0.1 + 1
+    h, y, sums = _left_for_norm(M, K, 40, nw)
+    w = rnd((N, K), torch.bfloat16, 42, 0.1)
+    inv = 1.0 / torch.sqrt((h.double().cpu() ** 2).sum(-1, keepdim=True) / K + eps)
+    acc = (y.double().cpu() @ w.double().cpu().T) * inv
+    other = plain_rmsnorm(h.double().cpu(), nw.double().cpu(), eps).bfloat16().double() @ w.double().cpu().T
+    floor = 1e-5 * math.sqrt(K)
+    if epi == EPI_STORE:
+        out, ref, odt = torch.zeros((M, N), dtype=torch.bfloat16, device=DEV), acc, torch.bfloat16
+    elif epi == EPI_STORE_F32:
+        out, ref, odt = torch.zeros((M, N), dtype=torch.float32, device=DEV), acc, torch.float32
+    elif epi == EPI_ACCUM_F32:
+        out = rnd((M, N), torch.float32, 5)
+        ref, other, odt = out.double().cpu() + acc, out.double().cpu() + other, torch.float32
+    else:
+        out = torch.zeros((M, N // 2), dtype=torch.bfloat16, device=DEV)
+        ref, other, odt = plain_silu(acc[:, 0::2]) * acc[:, 1::2], plain_silu(other[:, 0::2]) * other[:, 1::2], torch.bfloat16
+        floor *= 1 + 0.1 * math.sqrt(K)
+    k.gemm(NormedRows(y, sums, eps), w, out, epi)
+    err = (out.double().cpu() - ref).abs()
+    tol = out_tol(ref, odt, floor)
+    assert (err <= tol).all(), f"max err {float(err.max())} at {int(err.argmax())}, tol there {float(tol.flatten()[err.argmax()])}"
+    # Where the one rounding falls: both ways round every input (of size 1) by up to 2^-9 of itself, independently,
+    # (1.6e-3 of itself in standard deviation each), so an input differs by 2.3e-3 between them and a sum of K products
+    # with weights of size 0.1 by 2.3e-3 * 0.1 * sqrt(K); six of those bound the largest of many outputs.  SwiGLU
+    # multiplies a sum's deviation by the other sum, of size 0.1 sqrt(K).
+    spread = 6 * 2.3e-3 * 0.1 * math.sqrt(K) * (2 * (1 + 0.1 * math.sqrt(K)) if epi == EPI_SWIGLU else 1)
+    loose = out_tol(other, odt, floor + spread)
+    assert ((out.double().cpu() - other).abs() <= loose).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 14336), (16, 4096, 4096), (5, 200, 328), (3, 8192, 28672), (12, 100, 64)])
+def test_residual_product_leaves_what_the_next_norm_needs(M, N, K):
+    from llm_rs_amd.kernels import NextNorm
+    k = kernels()
+    assert k.gemm_defers_norm(M, N, K)
+    a = rnd((M, K), torch.bfloat16, 50)
+    w = rnd((N, K), torch.bfloat16, 51, 0.1)
+    h = rnd((M, N), torch.float32, 52, 2.0)
+    nw = rnd((N,), torch.float32, 53) * 0.1 + 1
+    want_h = h.double().cpu() + a.double().cpu() @ w.double().cpu().T
+    parts = -(-N // 16)
+    sums = torch.full((M, parts), -1.0, dtype=torch.float32, device=DEV)
+    y = torch.full((M, N + 4), 7.0, dtype=torch.bfloat16, device=DEV)
+    plain = h.clone()
+    k.gemm(a, w, plain, EPI_ACCUM_F32)
+    k.gemm(a, w, h, EPI_ACCUM_F32, None, leave=NextNorm(y[:, :N], sums, nw))
+    assert torch.equal(h, plain), "leaving something for the norm does not change the product"
+    assert torch.equal(y[:, :N], (h * nw).bfloat16()) and (y[:, N:] == 7.0).all()
+    padded = torch.zeros((M, parts * 16), dtype=torch.float64)
+    padded[:, :N] = h.double().cpu()
+    want = (padded * padded).view(M, parts, 16).sum(-1)
+    assert float((sums.double().cpu() - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    assert float((h.double().cpu() - want_h).abs().max()) <= 1e-5 * math.sqrt(K) + 1e-5 * float(want_h.abs().max())
+
+
+@pytest.mark.parametrize("M,n_heads,n_kv,hd,rot,K", [(8, 32, 8, 128, 128, 4096), (1, 32, 8, 128, 128, 4096), (16, 3, 1, 32, 32, 128),
+                                                      (5, 4, 2, 16, 8, 64), (3, 64, 8, 128, 128, 8192), (7, 2, 2, 64, 0, 192)])
+def test_qkv_rope_cache_finishes_a_norm_left_to_it(M, n_heads, n_kv, hd, rot, K):
+    """Norm, product, rotation and cache write in one kernel, against the same call on the norm kernel's output."""
+    from llm_rs_amd.kernels import NormedRows
+    k = kernels()
+    page_size, num_pages = 16, 12
+    N = (n_heads + 2 * n_kv) * hd
+    nw = rnd((K,), torch.float32, 61) * 0.1 + 1
+    h, y, sums = _left_for_norm(M, K, 60, nw)
+    w = rnd((N, K), torch.bfloat16, 62, 0.1)
+    positions = torch.randint(0, 400, (M,), generator=torch.Generator().manual_seed(32)).to(torch.int32).to(DEV)
+    slots = torch.randperm(num_pages * page_size, generator=torch.Generator().manual_seed(33))[:M].to(torch.int32).to(DEV)
+    inv_freq = plain_inv_freq(rot, 10000.0, None).to(DEV) if rot else None
+    results = []
+    for fused in (True, False):
+        qkv = torch.zeros((M, N + 8), dtype=torch.bfloat16, device=DEV)
+        kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros((num_pages, n_kv, hd, page_size), dtype=torch.bfloat16, device=DEV)
+        if fused:
+            x = NormedRows(y, sums, 1e-6)
+        else:
+            x = torch.empty((M, K), dtype=torch.bfloat16, device=DEV)
+            k.rmsnorm(x, h, nw, 1e-6)
+        k.qkv_rope_cache(x, w, qkv[:, :N], positions, slots, inv_freq, rot, kc, vc, n_heads, n_kv, hd, page_size, num_pages, True)
+        results.append((qkv[:, :n_heads * hd].double().cpu(), kc.double().cpu(), vc.double().cpu()))
+        assert (qkv[:, N:] == 0).all(), "padding touched"
+    scale = max(float(results[1][0].abs().max()), 1.0)
+    for name, a, b in zip("qkv", results[0], results[1]):
+        # the two differ in where the one rounding of the rows falls
+        assert float((a - b).abs().max()) <= 2e-2 * scale, name
+        assert float((a - b).abs().mean()) <= 1.5e-3 * scale, name
