@@ -67,7 +67,10 @@ __device__ __forceinline__ void block_sync_lds() { asm volatile("s_waitcnt lgkmc
 // where blocks of 64 features are needed to keep the tokens' rows from being
 // read too often, and would otherwise be too few to fill the device.
 // ---------------------------------------------------------------------------
-template <int MT, int NT, int NW, int U>
+// LAST < 16: the last of a block's feature tiles has only LAST features (a block of 24 features is a tile and a
+// half): the rows beyond are never asked for (their lanes load nothing and multiply zeros), so a weight whose
+// 16-feature blocks would be one and a half rounds of the device can be shared out evenly.
+template <int MT, int NT, int NW, int U, int LAST = 16>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ A, int lda,
                                                               const bf16* __restrict__ W, void* __restrict__ out,
                                                               int ldc, int M, int N, int K, int epi,
@@ -77,7 +80,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     float* red = (float*)skinny_smem;          // [NW][MT][NT][4][64]
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int row = lane & 15, g = lane >> 4;
-    int n0 = blockIdx.x * (NT * 16);
+    constexpr int BF = (NT - 1) * 16 + LAST;       // features of a block
+    static_assert(LAST == 16 || (LAST == 8 && NT >= 2), "a whole last tile, or half of one");
+    int n0 = blockIdx.x * BF;
+    const bool last_asks = LAST == 16 || row < LAST;   // whether this lane's row of the last tile exists
     const bf16* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) wp[nt] = W + (size_t)min(n0 + nt * 16 + row, N - 1) * K;
@@ -125,7 +131,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         for (int u = 0; u < U; ++u) {
             int k = turn(j + u * NW) * 64 + g * 8;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) { w[u][nt][0] = load8(wp[nt] + k); w[u][nt][1] = load8(wp[nt] + k + 32); }
+            for (int nt = 0; nt < NT; ++nt) {
+                if (LAST == 16 || nt < NT - 1 || last_asks) { w[u][nt][0] = load8(wp[nt] + k); w[u][nt][1] = load8(wp[nt] + k + 32); }
+                else { w[u][nt][0] = zero8(); w[u][nt][1] = zero8(); }
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) { x[u][mt][0] = load8(xp[mt] + k); x[u][mt][1] = load8(xp[mt] + k + 32); }
         }
@@ -149,8 +158,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         bf16x8 w0[NT], w1[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            w0[nt] = v0 ? load8(wp[nt] + k) : zero8();
-            w1[nt] = v1 ? load8(wp[nt] + k + 32) : zero8();
+            bool asks = LAST == 16 || nt < NT - 1 || last_asks;
+            w0[nt] = v0 && asks ? load8(wp[nt] + k) : zero8();
+            w1[nt] = v1 && asks ? load8(wp[nt] + k + 32) : zero8();
         }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -211,6 +221,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         int m = mt * 16 + row;
         int n = n0 + nt * 16 + 4 * g;
         if (m >= M) continue;
+        if (LAST < 16 && nt == NT - 1 && 4 * g >= LAST) continue;     // the half of the last tile that is the next block's
         if (partial != nullptr) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -312,7 +323,7 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
     }
 }
 
-template <int MT, int NT, int NW, int U>
+template <int MT, int NT, int NW, int U, int LAST = 16>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                           int M, int N, int K, int epi, const QkvEpilogue* qkv, int splits = 1,
                           float* partial = nullptr, int rot_feats = 0, const RowScale* scale = nullptr,
@@ -320,12 +331,12 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
     size_t bytes = (size_t)NW * MT * NT * 4 * 64 * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        (void)hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NT, NW, U>,
+        (void)hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NT, NW, U, LAST>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
         configured = true;
     }
-    dim3 grid(ceil_div(N, NT * 16), splits);
-    gemm_skinny_kernel<MT, NT, NW, U><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
+    dim3 grid(ceil_div(N, (NT - 1) * 16 + LAST), splits);
+    gemm_skinny_kernel<MT, NT, NW, U, LAST><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                           splits > 1 ? partial : nullptr,
                                                                           qkv ? *qkv : QkvEpilogue{}, rot_feats,
                                                                           scale ? *scale : RowScale{}, next ? *next : NextNorm{});
@@ -1004,7 +1015,17 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
 #define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, next)
         if (M <= 16) {
             if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else if (wide_nt == 7) SKINNY(1, 7, 4, 1); else SKINNY(1, 4, 4, 2); }
-            else if (eight) { if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4); else SKINNY(1, 1, 8, 4); }   // 8192 x 28672: 90 -> 83 us
+            else if (eight) {
+                // Blocks of 16 features, unless they come to a round and a half of the device's units (6144 features on
+                // 256: 384 blocks) and blocks of 24 to whole rounds: those, when nothing is to be left for a norm (which
+                // counts its sums by 16 features)
+                int b16 = ceil_div(N, 16), b24 = ceil_div(N, 24);
+                auto even = [&](int b) { return (double)b / ((double)ceil_div(b, cus) * cus); };
+                if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4);   // 8192 x 28672: 90 -> 83 us
+                else if (next == nullptr && N % 8 == 0 && even(b24) > even(b16) + 0.1)
+                    launch_skinny<1, 2, 8, 4, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, nullptr);
+                else SKINNY(1, 1, 8, 4);
+            }
             else SKINNY(1, 1, 4, 4);
         } else if (M <= 32) {
             int splits = skinny_splits(N, K);
