@@ -226,7 +226,7 @@ class HipKernels:
         n = out.shape[0]
         assert out.shape[1] == x.shape[1] == weight.shape[0]
         assert (rows is None and n == x.shape[0]) or (rows is not None and rows.dtype == torch.int32 and rows.shape[0] == n)
-        self._run("rmsnorm", n * x.shape[1] * (4 + out.element_size()) + x.shape[1] * 4, 5 * n * x.shape[1], None,
+        self._run(f"rmsnorm {n}x{x.shape[1]}", n * x.shape[1] * (4 + out.element_size()) + x.shape[1] * 4, 5 * n * x.shape[1], None,
                   self.lib.llmrs_rmsnorm, self._stream(), _code(out.dtype), _p(out), _p(x), _p(weight), _p(rows),
                   n, x.shape[1], eps)
 
@@ -250,7 +250,7 @@ class HipKernels:
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
         assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
         moved = (M * K + N * K) * a.element_size() + out.numel() * out.element_size() * (2 if epilogue == EPI_ACCUM_F32 else 1)
-        label = f"gemm {N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{'+next' if leave is not None else ''}"
+        label = f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{'+next' if leave is not None else ''}"
         self._run(label, moved, 2 * M * N * K, a.dtype,
                   self.lib.llmrs_gemm, self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
                   M, N, K, epilogue, _p(workspace),
@@ -291,7 +291,7 @@ class HipKernels:
             assert k_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
             assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
         M, K, N = x.shape[0], x.shape[1], w.shape[0]
-        self._run(f"gemm {N}x{K} {'norm+' if scale is not None else ''}qkv+rope+cache", (M * K + N * K + M * N) * x.element_size(), 2 * M * N * K, x.dtype,
+        self._run(f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}qkv+rope+cache", (M * K + N * K + M * N) * x.element_size(), 2 * M * N * K, x.dtype,
                   self.lib.llmrs_qkv_rope_cache,
                   self._stream(), _code(x.dtype), _p(x), x.stride(0), _p(w), _p(qkv), qkv.stride(0), x.shape[0], x.shape[1],
                   _p(positions), _p(slot_map), _p(inv_freq), rotary_dim, _p(k_cache), _p(v_cache), n_heads, n_kv_heads,
@@ -313,7 +313,7 @@ class HipKernels:
             seen = int((positions + 1).sum().item()) if window <= 0 else int((positions + 1).clamp(max=window).sum().item())
             moved = (2 * keys * n_kv_heads + 2 * T * n_heads) * head_dim * q.element_size()
             flops = 4 * seen * n_heads * head_dim
-        self._run("attention decode" if n_single == block_table.shape[0] else "attention", moved, flops, q.dtype,
+        self._run(f"attention {T} tokens" + (" (decode)" if n_single == block_table.shape[0] else ""), moved, flops, q.dtype,
                   self.lib.llmrs_attention,
                   self._stream(), _code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache),
                   _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
