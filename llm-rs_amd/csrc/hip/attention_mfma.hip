@@ -26,6 +26,8 @@
 // second product; their sum is not.
 #include "attention.h"
 
+#include <mutex>
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -596,6 +598,34 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
     }
 }
 
+// A step with a prompt portion beside decoding requests has two kinds of attention work that do not depend on
+// each other: tiles of many tokens, bound by the matrix cores, and single tokens over their whole caches, bound by
+// memory.  They run side by side: the single tokens' kernels go to a second stream of this library's own (default
+// priority), which waits for everything the caller's stream held when the call came and which the caller's stream
+// waits for before it goes on.  One such stream and pair of events per device, made at first use.  While the
+// caller's stream is being captured into a graph nothing is forked: the two kinds follow each other as before.
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+    bool tried = false;
+};
+static SideStream* side_stream() {
+    static SideStream per_device[64];
+    static std::mutex mutex;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(mutex);
+    SideStream& s = per_device[dev];
+    if (!s.tried) {
+        s.tried = true;
+        bool ok = hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) == hipSuccess &&
+                  hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) == hipSuccess &&
+                  hipEventCreateWithFlags(&s.join, hipEventDisableTiming) == hipSuccess;
+        if (!ok) { (void)hipGetLastError(); s.stream = nullptr; }
+    }
+    return s.stream != nullptr ? &s : nullptr;
+}
+
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
                   const int* positions, const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
@@ -618,6 +648,19 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     // Split the single-token entries when the caller gave room for their partial results.
     int split = max_chunks > 0 && scratch != nullptr && seq_lens != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
     int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
+    // both kinds of work: the single tokens' kernels on the second stream, beside the tiles
+    hipStream_t single_stream = stream;
+    SideStream* side = nullptr;
+    if (split && !only_single) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone) side = side_stream();
+        else (void)hipGetLastError();
+        if (side != nullptr) {
+            if (hipEventRecord(side->fork, stream) == hipSuccess && hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess)
+                single_stream = side->stream;
+            else { (void)hipGetLastError(); side = nullptr; }
+        }
+    }
     if (!only_single) {
         if constexpr (HD == 64 || HD == 128 || HD == 256) {
             int btiles = a.n_tokens / (4 * tpt) + n_entries;
@@ -631,8 +674,16 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     }
     if (split) {
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
-        attn_split_kernel<HD><<<grid, 64, 0, stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk);
-        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk);
+        attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk);
+        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk);
+    }
+    if (side != nullptr && single_stream != stream) {
+        // the caller's stream goes on only when the second stream's kernels are done (they write other rows of `out`)
+        if (hipEventRecord(side->join, side->stream) != hipSuccess || hipStreamWaitEvent(stream, side->join, 0) != hipSuccess) {
+            llmrs_fail("attention (mfma): cannot join the second stream: %s", hipGetErrorString(hipGetLastError()));
+            (void)hipStreamSynchronize(side->stream);
+            return -1;
+        }
     }
     return 1;
 }
