@@ -55,6 +55,8 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20),
                (64, 200, 2048), (40, 1000, 1096), (64, 4096, 4096), (24, 520, 2048), (50, 64, 8200),
                (8, 38, 100), (3, 130, 4099), (1, 6, 20),
+               # 256 x 192 tiles where they make whole rounds of the device and square ones do not; the last tile cut by N
+               (2048, 6144, 128), (2048, 6100, 192), (1800, 6144, 64),
                # a round and a half of 16-feature blocks: blocks of 24 features (a tile and a half), the last one cut by N
                (8, 6144, 4096), (1, 6144, 2048), (16, 5120, 2048), (3, 6000, 4096), (5, 6152, 2048),
                (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128),
