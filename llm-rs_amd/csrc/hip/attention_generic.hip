@@ -14,6 +14,8 @@
 #include "attention.h"
 #include "cache_layout.h"
 
+#include <type_traits>
+
 #define MAX_HEAD_DIM 512
 
 // Keys of a single-token entry that one wave of the split takes (aligned to absolute positions).
@@ -323,7 +325,7 @@ template <class T>
 static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cache, const T* v_cache,
                           const int* block_table, const int* token_entry, const int* positions, const int* q_starts,
                           const int* seq_lens, int n_entries, float* scratch, size_t scratch_bytes, int max_seq_len,
-                          int n_single, const AttnArgs& a) {
+                          int n_single, const AttnArgs& a, int allow_mfma) {
     bool vec = a.head_dim % 4 == 0 && (uintptr_t)k_cache % (4 * sizeof(T)) == 0;
     // Single-token entries are split by key range when the caller gave room for the partial results.
     int max_chunks = max_seq_len > 0 ? ceil_div(max_seq_len, GENERIC_CHUNK) : 0;
@@ -333,7 +335,17 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
     bool only_single = split && a.n_tokens == n_entries;     // every entry brings one token
     const int G = a.n_heads / a.n_kv_heads;
     const bool groupable = a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8);
-    if (!only_single) {
+    bool tiles_took = false;
+    if constexpr (std::is_same<T, float>::value) {
+        // 32-bit: entries with several tokens go to the matrix cores where the shape allows
+        if (!only_single && allow_mfma) {
+            int took = llmrs_attention_f32_mfma(stream, q, out, k_cache, v_cache, block_table, positions, q_starts, n_entries,
+                                                split ? 1 : 0, a);
+            if (took < 0) return -1;
+            tiles_took = took == 1;
+        }
+    }
+    if (!only_single && !tiles_took) {
         // a wave for all heads of a kv head when that still leaves two waves or more for each compute unit
         if (groupable && (long)a.n_tokens * a.n_kv_heads >= 2L * llmrs_compute_units()) {
             dim3 grid(a.n_tokens, a.n_kv_heads);
@@ -406,16 +418,18 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
                                              (float*)scratch, scratch_bytes, max_seq_len, n_single, a);
         if (took != 0) return took < 0 ? -1 : 0;
     }
+    int rc = 0;
     if (dtype == LLMRS_F32)
-        launch_generic<float>(stream, (const float*)q, (float*)out, (const float*)k_cache, (const float*)v_cache, block_table,
-                              token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
-                              max_seq_len, n_single, a);
+        rc = launch_generic<float>(stream, (const float*)q, (float*)out, (const float*)k_cache, (const float*)v_cache, block_table,
+                                   token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
+                                   max_seq_len, n_single, a, allow_mfma);
     else if (dtype == LLMRS_BF16)
-        launch_generic<bf16>(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
-                             token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
-                             max_seq_len, n_single, a);
+        rc = launch_generic<bf16>(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
+                                  token_entry, positions, q_starts, seq_lens, n_entries, (float*)scratch, scratch_bytes,
+                                  max_seq_len, n_single, a, allow_mfma);
     else
         return llmrs_fail("attention: unknown dtype %d", dtype);
+    if (rc != 0) return -1;
     LLMRS_LAUNCH_CHECK("attention");
     return 0;
 }
