@@ -961,6 +961,13 @@ extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
 // Up to 16 rows a bfloat16 product goes to the kernel for few rows with every tile of a block finished by a wave
 // of its own (not the widest weights, whose blocks take seven tiles): that kernel scales its rows' sums by a
 // norm left to it and leaves what the next norm needs.
+// Whether blocks of 24 features (a tile and a half) share a weight of N features out over the device's units more
+// evenly, by a tenth of a round or more, than blocks of `whole` features (16 or 32) do.
+static bool half_tile_blocks(int N, int whole, int cus) {
+    auto even = [&](int b) { return (double)b / ((double)ceil_div(b, cus) * cus); };
+    return N % 8 == 0 && even(ceil_div(N, 24)) > even(ceil_div(N, whole)) + 0.1;
+}
+
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K) { return M >= 1 && M <= 16 && N >= 1 && K % 8 == 0; }
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
@@ -1019,10 +1026,8 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                 // Blocks of 16 features, unless they come to a round and a half of the device's units (6144 features on
                 // 256: 384 blocks) and blocks of 24 to whole rounds: those, when nothing is to be left for a norm (which
                 // counts its sums by 16 features)
-                int b16 = ceil_div(N, 16), b24 = ceil_div(N, 24);
-                auto even = [&](int b) { return (double)b / ((double)ceil_div(b, cus) * cus); };
                 if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4);   // 8192 x 28672: 90 -> 83 us
-                else if (next == nullptr && N % 8 == 0 && even(b24) > even(b16) + 0.1)
+                else if (next == nullptr && half_tile_blocks(N, 16, cus))
                     launch_skinny<1, 2, 8, 4, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, nullptr);
                 else SKINNY(1, 1, 8, 4);
             }
@@ -1033,7 +1038,11 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
                 launch_skinny<2, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
             } else if (wide) { if (wide_nt == 7) SKINNY(2, 7, 4, 1); else SKINNY(2, 4, 4, 2); }
-            else if (N > 4096) { if (eight) SKINNY(2, 2, 8, 2); else SKINNY(2, 2, 4, 2); }
+            else if (N > 4096) {
+                if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<2, 2, 8, 2, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
+                else if (eight) SKINNY(2, 2, 8, 2);
+                else SKINNY(2, 2, 4, 2);
+            }
             else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {
             // 64 x 64 outputs per block; when that leaves no more than 64 blocks, K is split
@@ -1044,7 +1053,11 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
                 launch_skinny<4, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
             } else if (wide) { if (wide_nt == 7) SKINNY(4, 7, 4, 1); else SKINNY(4, 4, 4, 2); }
-            else if (N > 4096) { if (eight) SKINNY(4, 2, 8, 1); else SKINNY(4, 2, 4, 2); }
+            else if (N > 4096) {
+                if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<4, 2, 8, 1, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
+                else if (eight) SKINNY(4, 2, 8, 1);
+                else SKINNY(4, 2, 4, 2);
+            }
             else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
         }
 #undef SKINNY

@@ -59,6 +59,7 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (2048, 6144, 128), (2048, 6100, 192), (1800, 6144, 64),
                # a round and a half of 16-feature blocks: blocks of 24 features (a tile and a half), the last one cut by N
                (8, 6144, 4096), (1, 6144, 2048), (16, 5120, 2048), (3, 6000, 4096), (5, 6152, 2048),
+               (24, 6144, 2048), (64, 6144, 2048), (40, 6000, 2048), (30, 5128, 2048),
                (130, 200, 320), (300, 520, 768), (1000, 260, 1024), (65, 48, 64), (513, 1030, 128),
                # many features: blocks of several feature tiles that start their walk along k at staggered places
                (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192),
@@ -581,7 +582,8 @@ def test_sample_rows_frequencies():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M", [1, 8, 20, 50, 100])
 @pytest.mark.parametrize("n_heads,n_kv,hd,rot,K", [(4, 2, 32, 32, 256), (8, 2, 128, 128, 512), (3, 1, 64, 32, 96), (2, 2, 16, 0, 64),
-                                                  (36, 2, 128, 128, 8192)])    # long rows: at 50 tokens the product takes the tiles, the rotation its own kernel
+                                                  (36, 2, 128, 128, 8192),     # long rows: at 50 tokens the product takes the tiles, the rotation its own kernel
+                                                  (32, 8, 128, 128, 2048)])    # 6144 features: blocks of a tile and a half at 1 to 64 tokens
 def test_qkv_rope_cache(dtype, M, n_heads, n_kv, hd, rot, K):
     """The product, the rotation by neighbouring pairs and the cache write, as one call: for a few
     bfloat16 tokens it is one kernel that rotates the 32-bit sums; else product, then rotation."""
