@@ -17,6 +17,9 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
                               const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
                               size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a);
 
+// Keys per wave when the matrix-core kernels split `singles` single-token entries of up to max_seq_len keys.
+int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max_seq_len);
+
 // 32-bit tiles on the matrix cores for entries with several tokens (attention_f32_mfma.hip); skip_single: entries
 // with one token are left to the caller.  Return 1 when it took them, 0 when the shape is not its own, -1 on error.
 int llmrs_attention_f32_mfma(hipStream_t stream, const float* q, float* out, const float* k_cache, const float* v_cache,

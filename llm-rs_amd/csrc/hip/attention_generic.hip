@@ -321,6 +321,15 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
     }
 }
 
+// Room (in floats) for the partial results of the single-token entries (`singles` of n_entries, each of up to
+// max_seq_len keys) that a call splits by key range: what the caller brings as scratch, whichever kernels take the call.
+extern "C" long llmrs_attention_scratch_floats(int n_entries, int singles, int n_heads, int n_kv_heads, int head_dim,
+                                               int max_seq_len) {
+    if (max_seq_len <= 0 || n_entries <= 0 || n_heads <= 0 || n_kv_heads <= 0) return 0;
+    int chunk = min(GENERIC_CHUNK, llmrs_attention_split_chunk(singles > 0 ? singles : n_entries, n_kv_heads, max_seq_len));
+    return (long)n_entries * n_heads * ceil_div(max_seq_len, chunk) * (head_dim + 2);
+}
+
 template <class T>
 static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cache, const T* v_cache,
                           const int* block_table, const int* token_entry, const int* positions, const int* q_starts,

@@ -34,7 +34,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define ATTN_CHUNK 128
 
-extern "C" int llmrs_attention_chunk() { return ATTN_CHUNK; }
 
 // all of this wave's vector memory operations, loads into LDS among them, have completed
 __device__ __forceinline__ void wait_vmcnt_all() { __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8)); }
@@ -111,7 +110,8 @@ template <int HD>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16 (&O)[HD / 32], float& m, float& l,
                                              const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                              const int* __restrict__ table, int table_width, int num_pages,
-                                             int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale) {
+                                             int n_kv, int kvh, int t_begin, int t_end, int pos, int lo, float scale,
+                                             bool have_pages = false, int first_pages = 0) {
     int lane = threadIdx.x & 63;
     int r = lane & 31, h = lane >> 5;
     float scale_log2e = scale * 1.44269504088896341f;
@@ -123,7 +123,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
         int pg = table[min(first + lane, table_width - 1)];
         return min(max(pg, 0), num_pages - 1);
     };
-    int pv = load_pages(pv_base);
+    int pv = have_pages ? first_pages : load_pages(pv_base);     // (the caller's: those of pages t_begin / 16 + lane, clamped as here)
     for (int t0 = t_begin; t0 < t_end; t0 += 32) {
         int lp = t0 >> 4;
         if (lp + 1 - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
@@ -493,40 +493,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
 
 // ---- entries with one token: a wave for each (entry, kv head, chunk of keys) --
 // partial: [(entry * n_heads + head) * max_chunks + chunk][HD + 2] = m, l, O (not yet divided)
+// With `plain` (every entry brings one token and there is no window) a wave knows its token (the entry's number) and
+// where its keys begin (ch * chunk) without the request's length: it asks for its page numbers and its queries together
+// with the length, one trip to memory instead of two in a row.
 template <int HD>
 __global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
                                                         const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                                         const int* __restrict__ block_table,
                                                         const int* __restrict__ seq_lens,
                                                         const int* __restrict__ q_starts, AttnArgs a, int G,
-                                                        int max_chunks, int chunk) {
+                                                        int max_chunks, int chunk, int plain) {
     int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z;
-    int token = q_starts[e], count = q_starts[e + 1] - token;
-    int pos_t = seq_lens[e] - 1;                  // an entry with one token: its position is its length less one
-    if (count != 1) return;
-    int lo_t = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
-    int first_chunk = lo_t / chunk;
-    int n_chunks = pos_t / chunk - first_chunk + 1;
-    if (ch >= n_chunks) return;
-    int t_begin = (first_chunk + ch) * chunk;
-    int t_end = min(t_begin + chunk, pos_t + 1);
     int lane = threadIdx.x & 63, c = lane & 31, h = lane >> 5;
     bool cvalid = c < G;
     int head = kvh * G + min(c, G - 1);
-    int pos = cvalid ? pos_t : -1;
-
+    const int* table = block_table + (size_t)e * a.table_width;
     bf16x8 qf[HD / 16];
-    const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
+    int token, pos_t, lo_t, t_begin, first_pages = 0;
+    if (plain) {
+        token = e;
+        lo_t = 0;
+        t_begin = ch * chunk;
+        int pg = table[min((t_begin >> 4) + lane, a.table_width - 1)];
+        first_pages = min(max(pg, 0), a.num_pages - 1);
+        const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
 #pragma unroll
-    for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+        for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+        pos_t = seq_lens[e] - 1;                  // an entry with one token: its position is its length less one
+        if (t_begin > pos_t) return;
+    } else {
+        token = q_starts[e];
+        int count = q_starts[e + 1] - token;
+        pos_t = seq_lens[e] - 1;
+        if (count != 1) return;
+        lo_t = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
+        int first_chunk = lo_t / chunk;
+        int n_chunks = pos_t / chunk - first_chunk + 1;
+        if (ch >= n_chunks) return;
+        t_begin = (first_chunk + ch) * chunk;
+        const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + h * 8;
+#pragma unroll
+        for (int ks = 0; ks < HD / 16; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+    }
+    int t_end = min(t_begin + chunk, pos_t + 1);
+    int pos = cvalid ? pos_t : -1;
     f32x16 O[HD / 32];
 #pragma unroll
     for (int dt = 0; dt < HD / 32; ++dt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
     float m = -INFINITY, l = 0.0f;
-    attend_range<HD>(qf, O, m, l, kc, vc, block_table + (size_t)e * a.table_width, a.table_width, a.num_pages,
-                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale);
+    attend_range<HD>(qf, O, m, l, kc, vc, table, a.table_width, a.num_pages,
+                     a.n_kv_heads, kvh, t_begin, t_end, pos, lo_t, a.scale, plain != 0, first_pages);
     if (!cvalid) return;
     float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
     if (h == 0) { pp[0] = m; pp[1] = l; }
@@ -538,64 +556,77 @@ __global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__
 
 #define MERGE_MAX_CHUNKS 1024
 
-// One wave for each (entry, head): lanes share out the chunks for the common maximum and
-// the sum, then the features.  Chunks are added in ascending order.  Everything a lane needs
-// from memory is asked for at once (a chunk's m and l, and its features' sums for the first
+// One block for each (entry, head), a thread for each feature (a wave per 64 of them).  Every wave finds the common
+// maximum and the sum for itself, its lanes sharing out the chunks; chunks are added in ascending order.  Everything
+// a thread needs from memory is asked for at once (a chunk's m and l, and its feature's sums for the first
 // chunks): the kernel is a chain of trips to memory and little else.
-__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
-                                                        const int* __restrict__ seq_lens,
-                                                        const int* __restrict__ q_starts, AttnArgs a, int max_chunks,
-                                                        int chunk) {
+// With `plain` (every entry brings one token, no window) the token is the entry's number and the chunks are
+// counted from the first: the first chunks' sums, maxima and sums of weights are asked for before the
+// request's length is known (what lies beyond its chunks is read and never used), one trip instead of two.
+__global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
+                                                         const int* __restrict__ seq_lens,
+                                                         const int* __restrict__ q_starts, AttnArgs a, int max_chunks,
+                                                         int chunk, int plain) {
     __shared__ float weight[MERGE_MAX_CHUNKS];
-    constexpr int AHEAD = 16;                     // chunks whose sums are asked for before the weights are known
-    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim, lane = threadIdx.x;
-    int token = q_starts[e], count = q_starts[e + 1] - token;
-    int pos = seq_lens[e] - 1;
-    if (count != 1) return;
-    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-    int n_chunks = pos / chunk - lo / chunk + 1;
+    constexpr int AHEAD = 32;                     // chunks whose sums are asked for before the weights are known
+    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int d = threadIdx.x;                          // this thread's feature (threads past the head size only help with the weights)
     const float* pp = partial + (size_t)(e * a.n_heads + head) * max_chunks * (hd + 2);
     int stride = hd + 2;
-    // this lane's features d = lane, lane + 64 (head sizes up to 128 in registers; the rest in the loop below)
-    float ahead[2][AHEAD];
+    int token, pos, lo, n_chunks;
+    float ahead[AHEAD];
+    float m_mine = -INFINITY, l_mine = 0.0f;      // chunk `lane`'s maximum and sum (plain, up to 64 chunks)
+    const bool early = plain && max_chunks <= 64;
+    if (early) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+        for (int ch = 0; ch < AHEAD; ++ch) ahead[ch] = (ch < max_chunks && d < hd) ? pp[(size_t)ch * stride + 2 + d] : 0.0f;
+        if (lane < max_chunks) { m_mine = pp[(size_t)lane * stride]; l_mine = pp[(size_t)lane * stride + 1]; }
+        token = e;
+        pos = seq_lens[e] - 1;
+        lo = 0;
+        n_chunks = pos / chunk + 1;
+    } else {
+        token = q_starts[e];
+        int count = q_starts[e + 1] - token;
+        pos = seq_lens[e] - 1;
+        if (count != 1) return;
+        lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+        n_chunks = pos / chunk - lo / chunk + 1;
 #pragma unroll
-        for (int ch = 0; ch < AHEAD; ++ch) {
-            int d = lane + 64 * j;
-            ahead[j][ch] = (ch < n_chunks && d < hd) ? pp[(size_t)ch * stride + 2 + d] : 0.0f;
-        }
+        for (int ch = 0; ch < AHEAD; ++ch) ahead[ch] = (ch < n_chunks && d < hd) ? pp[(size_t)ch * stride + 2 + d] : 0.0f;
+    }
     float M = -INFINITY;
-    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * stride]);
-    M = wave_max(M);
     float L = 0.0f;
-    for (int ch = lane; ch < n_chunks; ch += 64) {
-        float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * stride] - M);     // the maxima are base-2 logarithms
-        weight[ch] = w;
-        L += pp[(size_t)ch * stride + 1] * w;
+    if (early) {
+        if (lane >= n_chunks) m_mine = -INFINITY;
+        M = wave_max(m_mine);
+        float w = lane < n_chunks ? __builtin_amdgcn_exp2f(m_mine - M) : 0.0f;     // the maxima are base-2 logarithms
+        if (lane < n_chunks) { if (wave == 0) weight[lane] = w; L = l_mine * w; }
+    } else {
+        for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * stride]);
+        M = wave_max(M);
+        for (int ch = lane; ch < n_chunks; ch += 64) {
+            float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * stride] - M);
+            if (wave == 0) weight[ch] = w;
+            L += pp[(size_t)ch * stride + 1] * w;
+        }
     }
     L = wave_sum(L);
     __syncthreads();
-    float inv = 1.0f / L;
-    for (int d = lane, j = 0; d < hd; d += 64, ++j) {
-        float o = 0.0f;
-        int ch = 0;
-        if (j < 2) {
+    if (d >= hd) return;
+    float o = 0.0f;
 #pragma unroll
-            for (int c = 0; c < AHEAD; ++c)
-                if (c < n_chunks) o = fmaf(ahead[j][c], weight[c], o);
-            ch = min(n_chunks, AHEAD);
-        }
-        for (; ch < n_chunks; ch += AHEAD) {      // the rest, a group's sums asked for together
-            float v[AHEAD];
+    for (int c = 0; c < AHEAD; ++c)
+        if (c < n_chunks) o = fmaf(ahead[c], weight[c], o);
+    for (int ch = AHEAD; ch < n_chunks; ch += AHEAD) {      // the rest, a group's sums asked for together
+        float v[AHEAD];
 #pragma unroll
-            for (int c = 0; c < AHEAD; ++c) v[c] = (ch + c < n_chunks) ? pp[(size_t)(ch + c) * stride + 2 + d] : 0.0f;
+        for (int c = 0; c < AHEAD; ++c) v[c] = (ch + c < n_chunks) ? pp[(size_t)(ch + c) * stride + 2 + d] : 0.0f;
 #pragma unroll
-            for (int c = 0; c < AHEAD; ++c)
-                if (ch + c < n_chunks) o = fmaf(v[c], weight[ch + c], o);
-        }
-        out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o * inv);
+        for (int c = 0; c < AHEAD; ++c)
+            if (ch + c < n_chunks) o = fmaf(v[c], weight[ch + c], o);
     }
+    out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / L);
 }
 
 // A step with a prompt portion beside decoding requests has two kinds of attention work that do not depend on
@@ -626,23 +657,29 @@ static SideStream* side_stream() {
     return s.stream != nullptr ? &s : nullptr;
 }
 
+// Keys per wave of the split, by what the host knows: the number of single-token entries and the bound on their
+// length.  ATTN_CHUNK, doubled while the waves would still fill the device's places (a wave begins with a chain of
+// trips to memory: lengths, page numbers, then keys; with many requests, longer ranges make that a smaller part of
+// its life; measured, 8B shapes at 2048 keys: 64 requests 6945 -> 7540 tokens/s, 256 requests 11960 -> 12740);
+// halved when even then there is no more than a wave per SIMD and the chunks stay few enough for the merge to
+// take in one go: with so few requests a wave's life is its chain of trips, one per 32 keys, and nothing else
+// competes for memory.
+int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max_seq_len) {
+    long cus = llmrs_compute_units();
+    auto waves = [&](int c) { return singles * n_kv_heads * ((3L * max_seq_len / 4 + c - 1) / c); };
+    int chunk = ATTN_CHUNK;
+    if (waves(ATTN_CHUNK / 2) <= cus * 4 && max_seq_len <= 64 * (ATTN_CHUNK / 2)) return ATTN_CHUNK / 2;
+    while (chunk < 8 * ATTN_CHUNK && waves(chunk * 2) >= cus * 8) chunk *= 2;
+    return chunk;
+}
+
 template <int HD>
 static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, const bf16* vc, const int* table,
                   const int* positions, const int* q_starts, const int* seq_lens, int n_entries, float* scratch,
                   size_t scratch_bytes, int max_seq_len, int n_single, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
     int tpt = 32 / G;
-    // Keys per wave of the split: ATTN_CHUNK, doubled while the waves would still fill the device's
-    // places (a wave begins with a chain of trips to memory: lengths, page numbers, then keys;
-    // with many requests, longer ranges make that a smaller part of its life).  By what the host
-    // knows: the number of such entries and the bound on their length.  (Measured, 8B shapes at 2048
-    // keys: 64 requests 6945 -> 7540 tokens/s, 256 requests 11960 -> 12740.)
-    int chunk = ATTN_CHUNK;
-    {
-        long places = (long)llmrs_compute_units() * 8;
-        auto waves = [&](int c) { return (long)(n_single > 0 ? n_single : n_entries) * a.n_kv_heads * ((3L * max_seq_len / 4 + c - 1) / c); };
-        while (chunk < 8 * ATTN_CHUNK && waves(chunk * 2) >= places) chunk *= 2;
-    }
+    int chunk = llmrs_attention_split_chunk(n_single > 0 ? n_single : n_entries, a.n_kv_heads, max_seq_len);
     int max_chunks = max_seq_len > 0 ? (max_seq_len + chunk - 1) / chunk : 0;
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.
@@ -674,8 +711,9 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     }
     if (split) {
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
-        attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk);
-        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64, 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk);
+        int plain = only_single && a.window == 0;
+        attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk, plain);
+        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64 * ((HD + 63) / 64), 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk, plain);
     }
     if (side != nullptr && single_stream != stream) {
         // the caller's stream goes on only when the second stream's kernels are done (they write other rows of `out`)

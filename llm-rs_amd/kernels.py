@@ -155,10 +155,10 @@ class HipKernels:
         # LLM_PERF in the environment (the reference's switch): every call is timed on the device and
         # steps are not recorded into graphs, so that each kernel can be seen by itself
         self.times: Optional[KernelTimes] = KernelTimes() if os.environ.get("LLM_PERF") else None
-        lib.llmrs_attention_chunk.restype = I
+        lib.llmrs_attention_scratch_floats.restype = ctypes.c_long
+        lib.llmrs_attention_scratch_floats.argtypes = [I, I, I, I, I, I]
         lib.llmrs_gemm_workspace_floats.restype = ctypes.c_long
         lib.llmrs_gemm_workspace_floats.argtypes = [I, I, I]
-        self.attention_chunk = lib.llmrs_attention_chunk()
 
     def gemm_workspace_floats(self, M: int, N: int, K: int) -> int:
         """Room that lets a product with too few blocks split K over blocks (the kernels' own rule)."""
@@ -169,9 +169,12 @@ class HipKernels:
         into the stream, leaves a `NextNorm` (that: for fewer than 16384 features)."""
         return self.allow_mfma and bool(self.lib.llmrs_gemm_defers_norm(int(M), int(N), int(K)))
 
-    def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int) -> int:
-        """Room the split of single-token entries needs for its partial results."""
-        return n_entries * n_heads * (-(-max_seq_len // self.attention_chunk)) * (head_dim + 2)
+    def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int,
+                                 n_kv_heads: Optional[int] = None, n_single: int = 0) -> int:
+        """Room the split of single-token entries needs for its partial results (the kernels' own rule: the key
+        ranges get shorter when there are few such entries)."""
+        return int(self.lib.llmrs_attention_scratch_floats(int(n_entries), int(n_single), int(n_heads),
+                                                            int(n_kv_heads or n_heads), int(head_dim), int(max_seq_len)))
 
     def _check(self, rc: int) -> None:
         if rc != 0:

@@ -125,7 +125,7 @@ class Attention(Mixer):
                                 self.heads, n_kv, self.head_dim, cache.page_size, cache.num_pages, write)
         o = ctx.workspace("attn.out", (T, self.q_size), self.dtype)
         # room for the partial results of single-token entries, which the kernel splits by key range
-        need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len) if ctx.n_single else 0
+        need = k.attention_scratch_floats(ctx.n_entries, self.heads, self.head_dim, ctx.max_seq_len, self.kv_heads, ctx.n_single) if ctx.n_single else 0
         scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,

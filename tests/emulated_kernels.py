@@ -15,7 +15,7 @@ EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 class EmulatedKernels:
     allow_mfma = False
 
-    def attention_scratch_floats(self, n_entries, n_heads, head_dim, max_seq_len):
+    def attention_scratch_floats(self, n_entries, n_heads, head_dim, max_seq_len, n_kv_heads=None, n_single=0):
         return 0
 
     def embed_rows(self, out, table, tokens, scale=1.0):

@@ -297,7 +297,7 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
     early key matches the query so strongly that the output must be its value."""
     n_heads, n_kv = 4, 2
     case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=3)
-    for far in (0, ps - 1, ps, n // 2 + 1, n - 2) + ((2053, n - 300) if n > 2100 else ()):
+    for far in (0, ps - 1, ps, 63, 64, n // 2 + 1, n - 2) + ((2053, n - 300) if n > 2100 else ()):    # (one request alone: ranges of 64 keys)
         q = torch.zeros((1, n_heads, hd))
         q[0, :, :] = case.k[0][far, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
         got = case.run([q.to(dtype)], [[n - 1]])
@@ -306,6 +306,42 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (ref[0].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
         tol = 1e-4 if dtype == torch.float32 else 2e-2
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
+
+
+@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("portion", [False, True])
+def test_attention_few_decoding_requests(window, portion):
+    """With few decoding requests a wave of the split takes 64 keys.  Each request's query matches one key
+    strongly, at the edges of such ranges and of the window: the output must be that key's value, with and
+    without a prompt portion in the same call (with one, a wave looks its token up instead of taking the
+    entry's number), and agree with the plain implementation."""
+    n_heads, n_kv, hd, ps = 8, 2, 128, 16
+    g = torch.Generator().manual_seed(7 + window)
+    lens = [130, 1000, 2047, 64, 65] + ([90] if portion else [])
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=13)
+    edges = [0, 63, 64, 65, 127, 128, 191, 192, 959, 960, 1983, 1984]
+    n_dec = 5
+    for shift in range(4):
+        qs, pos, fars = [], [], []
+        for r, n in enumerate(lens[:n_dec]):
+            lo = max(0, n - window) if window else 0
+            seen = [e for e in edges + [lo, lo + 1, n - 1] if lo <= e < n]
+            far = seen[(5 * r + 3 * shift) % len(seen)]
+            fars.append(far)
+            qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16))
+            pos.append([n - 1])
+        if portion:
+            qs.append(torch.randn((30, n_heads, hd), generator=g).to(torch.bfloat16))
+            pos.append(list(range(60, 90)))
+        got = case.run(qs, pos, window=window)
+        for r in range(n_dec):
+            want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
+            ref = case.reference(r, qs[r], pos[r], window=window)[0].float()
+            assert (ref - want).abs().max() < 0.05, "the case itself"
+            assert (got[r].float() - ref).abs().max() <= 2e-2, f"request of length {lens[r]}, key {fars[r]}"
+        if portion:
+            ref = case.reference(n_dec, qs[-1], pos[-1], window=window).float()
+            assert (got[n_dec:].float() - ref).abs().max() <= 3e-2
 
 
 @pytest.mark.parametrize("window", [0, 300])
