@@ -33,11 +33,16 @@ struct QkvEpilogue {
 // before its epilogue.  x W^T with x = h inv weight is the same number as inv (h weight) W^T; what
 // differs from the norm kernel's output is where the one rounding to bfloat16 falls (on h weight
 // instead of on h inv weight), not how many there are.
+// With more rows, a product whose sums are split over blocks (k ranges) has a kernel that adds the parts up, and
+// that kernel sees whole rows: with eps > 0 it finishes the following norm itself,
+//   y[m, n] = bfloat16(h[m, n] * inv[m] * weight[n])
+// which any product takes as plain rows (sumsq is not used then).
 struct NextNorm {
-    float* sumsq;          // [M, ceil(N / 16)]; null: nothing is left
-    bf16* y;               // [M, N], row stride ldy
+    float* sumsq;          // [M, ceil(N / 16)] (not used with eps > 0)
+    bf16* y;               // [M, N], row stride ldy; null: nothing is left
     int ldy;
     const float* weight;   // [N]
+    float eps;             // > 0: the norm is finished here (llmrs_gemm_norms_whole), else left to the next product
 };
 struct RowScale {
     const float* sumsq;    // [M, nparts]; null: no scale
@@ -57,9 +62,12 @@ __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int 
 // workspace: device memory for the partial sums of products that split K over blocks (may be null).
 // qkv: needed when epi is LLMRS_EPI_QKV; such a call is taken only by the kernels that fuse it.
 // scale, next: see RowScale and NextNorm; both only where llmrs_gemm_defers_norm(M, N, K) holds (next: with
-// LLMRS_EPI_ACCUM_F32 only).
+// LLMRS_EPI_ACCUM_F32 only), or next with eps where llmrs_gemm_norms_whole(M, N, K) holds.
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
                          const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr);
 // Whether the bfloat16 product of this shape goes to the kernel that can scale its rows' sums and leave a NextNorm.
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K);
+// Whether the bfloat16 product of this shape, adding into the stream and given the workspace that
+// llmrs_gemm_workspace_floats asks for, is split over blocks so that it can finish the following norm (NextNorm with eps).
+extern "C" int llmrs_gemm_norms_whole(int M, int N, int K);

@@ -323,6 +323,61 @@ __global__ void gemm_splitk_finish_kernel(const float* __restrict__ partial, int
     }
 }
 
+// The same for a product that adds into the 32-bit stream and is followed by a norm x / rms(x) * weight: a block
+// for each row adds the parts in the same order, writes the stream's new row, and, having the whole row, the
+// normed row as well (NextNorm with eps): no norm kernel runs.  Up to 16384 features (16 per thread), a multiple of 4.
+__global__ __launch_bounds__(1024) void gemm_splitk_finish_norm_kernel(const float* __restrict__ partial, int splits,
+                                                                        float* __restrict__ out, int ldc, int M, int N,
+                                                                        NextNorm nn) {
+    __shared__ float red[16];
+    int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+    const float* p0 = partial + (size_t)m * N;
+    float* o = out + (size_t)m * ldc;
+    f32x4 h[4];
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int n = (i * (int)blockDim.x + tid) * 4;
+        h[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (n < N) {
+            f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < splits; ++s) v += *(const f32x4*)(p0 + (size_t)s * M * N + n);
+            h[i] = *(const f32x4*)(o + n) + v;
+            *(f32x4*)(o + n) = h[i];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) ss = fmaf(h[i][r], h[i][r], ss);
+        }
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+    for (int w = 0; w < waves; ++w) total += red[w];
+    float inv = 1.0f / sqrtf(total / (float)N + nn.eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int n = (i * (int)blockDim.x + tid) * 4;
+        if (n < N) {
+            f32x4 w = *(const f32x4*)(nn.weight + n);
+            bf16x4 y;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) y[r] = (bf16)(h[i][r] * inv * w[r]);
+            *(bf16x4*)(nn.y + (size_t)m * nn.ldy + n) = y;
+        }
+    }
+}
+// Adds the parts of a split product up: with the norm that follows where one is to be finished (NextNorm with eps).
+static void launch_splitk_finish(hipStream_t stream, const float* partial, int splits, void* out, int ldc, int M, int N,
+                                 int epi, const NextNorm* next) {
+    if (next != nullptr && next->eps > 0.0f) {
+        int threads = min(1024, ceil_div(ceil_div(N, 4), 64) * 64);
+        gemm_splitk_finish_norm_kernel<<<M, threads, 0, stream>>>(partial, splits, (float*)out, ldc, M, N, *next);
+        return;
+    }
+    size_t pairs = (size_t)M * ((N + 1) / 2);
+    gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
+}
+
 template <int MT, int NT, int NW, int U, int LAST = 16>
 static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                           int M, int N, int K, int epi, const QkvEpilogue* qkv, int splits = 1,
@@ -339,11 +394,9 @@ static void launch_skinny(hipStream_t stream, const bf16* A, int lda, const bf16
     gemm_skinny_kernel<MT, NT, NW, U, LAST><<<grid, NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                           splits > 1 ? partial : nullptr,
                                                                           qkv ? *qkv : QkvEpilogue{}, rot_feats,
-                                                                          scale ? *scale : RowScale{}, next ? *next : NextNorm{});
-    if (splits > 1) {
-        size_t pairs = (size_t)M * ((N + 1) / 2);
-        gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
-    }
+                                                                          scale ? *scale : RowScale{},
+                                                                          next && splits == 1 ? *next : NextNorm{});
+    if (splits > 1) launch_splitk_finish(stream, partial, splits, out, ldc, M, N, epi, next);
 }
 
 // ---------------------------------------------------------------------------
@@ -706,7 +759,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
 
 template <int BM, int BN, int WGM, int WGN, int STAGES>
 static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                      int M, int N, int K, int epi, int splits = 1, float* partial = nullptr) {
+                      int M, int N, int K, int epi, int splits = 1, float* partial = nullptr, const NextNorm* next = nullptr) {
     static bool configured = false;
     size_t bytes = (size_t)STAGES * (BM + BN) * 128;
     if (!configured) {
@@ -719,10 +772,7 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
     gemm_dma_kernel<BM, BN, WGM, WGN, STAGES><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                                       splits > 1 ? partial : nullptr);
-    if (splits > 1) {
-        size_t pairs = (size_t)M * ((N + 1) / 2);
-        gemm_splitk_finish_kernel<<<ceil_div(pairs, 256), 256, 0, stream>>>(partial, splits, out, ldc, M, N, epi);
-    }
+    if (splits > 1) launch_splitk_finish(stream, partial, splits, out, ldc, M, N, epi, next);
     return 0;
 }
 
@@ -932,9 +982,9 @@ static int tiled_splits(int M, int N, int K) {
 }
 // The 128 x 128 tiles of a product, in whichever of the two forms its shape asks for.
 static int launch_tiles_128(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                            int M, int N, int K, int epi, int splits, float* partial) {
-    if (deep_tiles(M, N, K)) return launch_dma<128, 128, 2, 4, 4>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial);
-    return launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial);
+                            int M, int N, int K, int epi, int splits, float* partial, const NextNorm* next = nullptr) {
+    if (deep_tiles(M, N, K)) return launch_dma<128, 128, 2, 4, 4>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next);
+    return launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next);
 }
 // 17..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
 // get blocks of many feature tiles): the 128 x 128 tiles with k split over blocks read the tokens'
@@ -969,6 +1019,10 @@ static bool half_tile_blocks(int N, int whole, int cus) {
 }
 
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K) { return M >= 1 && M <= 16 && N >= 1 && K % 8 == 0; }
+// 17 to 256 rows whose sums are split over blocks: the kernel that adds the parts up can finish the following norm.
+extern "C" int llmrs_gemm_norms_whole(int M, int N, int K) {
+    return M > 16 && M <= 256 && N >= 4 && N % 4 == 0 && N <= 16384 && K % 8 == 0 && llmrs_gemm_workspace_floats(M, N, K) > 0;
+}
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
@@ -977,7 +1031,14 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         if (scale != nullptr || next != nullptr) { llmrs_fail("gemm: a deferred norm needs rows of a multiple of 8 values, 16-byte aligned"); return -1; }
         return 0;
     }
-    if (scale != nullptr || next != nullptr) {
+    const bool whole = next != nullptr && next->eps > 0.0f;      // the norm that follows is finished by the kernel that adds the parts up
+    if (whole) {
+        bool ok = scale == nullptr && epi == LLMRS_EPI_ACCUM_F32 && llmrs_gemm_norms_whole(M, N, K) && workspace != nullptr &&
+                  workspace_bytes >= (size_t)llmrs_gemm_workspace_floats(M, N, K) * sizeof(float) && next->y != nullptr &&
+                  next->weight != nullptr && next->ldy >= N && next->ldy % 4 == 0 && ((uintptr_t)next->y & 7) == 0 &&
+                  ((uintptr_t)next->weight & 15) == 0 && ldc % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)workspace & 15) == 0;
+        if (!ok) { llmrs_fail("gemm: a norm finished by a split product needs the += epilogue, 17 to 256 rows of a shape that is split, its workspace and aligned rows, got M=%d N=%d K=%d epilogue %d", M, N, K, epi); return -1; }
+    } else if (scale != nullptr || next != nullptr) {
         bool ok = llmrs_gemm_defers_norm(M, N, K) && (scale == nullptr || (scale->sumsq != nullptr && scale->nparts >= 1 && scale->eps > 0.0f)) &&
                   (next == nullptr || (epi == LLMRS_EPI_ACCUM_F32 && N < 16384 && next->sumsq != nullptr && next->y != nullptr &&
                                        next->weight != nullptr && next->ldy >= N && next->ldy % 4 == 0 && ((uintptr_t)next->y & 7) == 0));
@@ -998,7 +1059,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         tiles_for_few = workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float);
     }
     if (tiles_for_few) {
-        rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, tiled_splits(M, N, K), (float*)workspace);
+        rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, tiled_splits(M, N, K), (float*)workspace, next);
     } else if (M <= 64) {
         // Waves per block (NW) come from the weight's shape alone: k-blocks go to the
         // waves in turn and their sums are added in wave order, so for a given weight an
@@ -1013,6 +1074,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         // A wide weight's blocks take 7 or 4 feature tiles: whichever number of blocks fills the
         // device's compute units more evenly (28672 features are 256 blocks of 7 tiles).  Its blocks
         // start their walk along k at staggered places, by groups of that many features.
+        if (whole && skinny_splits(N, K) <= 1) { llmrs_fail("gemm: M=%d N=%d K=%d is not split after all: the norm cannot be finished here", M, N, K); return -1; }
         int cus = llmrs_compute_units();
         auto evenness = [&](int nt) { int b = ceil_div(N, 16 * nt); return (double)b / ((double)ceil_div(b, cus) * cus); };
         int wide_nt = (wide && evenness(7) >= evenness(4)) ? 7 : 4;
@@ -1036,7 +1098,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             int splits = skinny_splits(N, K);
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
-                launch_skinny<2, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
+                launch_skinny<2, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace, 0, nullptr, next);
             } else if (wide) { if (wide_nt == 7) SKINNY(2, 7, 4, 1); else SKINNY(2, 4, 4, 2); }
             else if (N > 4096) {
                 if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<2, 2, 8, 2, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
@@ -1051,7 +1113,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             int splits = skinny_splits(N, K);
             if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
                 workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
-                launch_skinny<4, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace);
+                launch_skinny<4, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace, 0, nullptr, next);
             } else if (wide) { if (wide_nt == 7) SKINNY(4, 7, 4, 1); else SKINNY(4, 4, 4, 2); }
             else if (N > 4096) {
                 if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<4, 2, 8, 1, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
@@ -1113,7 +1175,8 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         } else if (K % 64 == 0) {
             int splits = tiled_splits(M, N, K);
             if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
-                rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace);
+                rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace, next);
+            else if (whole) rc = llmrs_fail("gemm: M=%d N=%d K=%d is not split after all: the norm cannot be finished here", M, N, K);
             else
                 rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, 1, nullptr);
         }

@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A,
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
                           int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma,
                           const float* scale_sumsq, int scale_parts, float scale_eps, float* next_sumsq, void* next_y,
-                          int next_ldy, const float* next_weight) {
+                          int next_ldy, const float* next_weight, float next_eps) {
     LLMRS_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     LLMRS_REQUIRE(lda >= K, "gemm: row stride %d of A is shorter than K=%d", lda, K);
     LLMRS_REQUIRE(epi >= 0 && epi <= 3, "gemm: unknown epilogue %d", epi);
@@ -259,12 +259,12 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
     if (M == 0) return 0;
     if (dtype == LLMRS_BF16 && allow_mfma) {
         RowScale rs{scale_sumsq, scale_parts, scale_eps};
-        NextNorm nn{next_sumsq, (bf16*)next_y, next_ldy, next_weight};
+        NextNorm nn{next_sumsq, (bf16*)next_y, next_ldy, next_weight, next_eps};
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)A, lda, (const bf16*)W, out, ldc, M, N, K, epi, workspace,
-                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_sumsq ? &nn : nullptr);
+                                        workspace_bytes, nullptr, scale_sumsq ? &rs : nullptr, next_y ? &nn : nullptr);
         if (took != 0) return took < 0 ? -1 : 0;
     }
-    LLMRS_REQUIRE(scale_sumsq == nullptr && next_sumsq == nullptr, "gemm: a deferred norm needs the bfloat16 matrix-core kernels (M=%d N=%d K=%d)", M, N, K);
+    LLMRS_REQUIRE(scale_sumsq == nullptr && next_y == nullptr, "gemm: a deferred norm needs the bfloat16 matrix-core kernels (M=%d N=%d K=%d)", M, N, K);
     if (M <= GEMV_MAX_M) {
         size_t elt = dtype == LLMRS_F32 ? sizeof(float) : sizeof(bf16);
         bool vec = K % 4 == 0 && lda % 4 == 0 && (uintptr_t)A % (4 * elt) == 0 && (uintptr_t)W % (4 * elt) == 0;

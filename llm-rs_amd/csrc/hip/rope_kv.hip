@@ -218,7 +218,7 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
 extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda, const void* W, void* out, int ldc,
                           int M, int N, int K, int epi, void* workspace, size_t workspace_bytes, int allow_mfma,
                           const float* scale_sumsq, int scale_parts, float scale_eps, float* next_sumsq, void* next_y,
-                          int next_ldy, const float* next_weight);
+                          int next_ldy, const float* next_weight, float next_eps);
 
 // qkv = x W^T for W = [q heads; k heads; v heads], then what llmrs_rope_kv_write does,
 // with pairs (2i, 2i+1): in one kernel when the product is one the rotation fuses into
@@ -248,7 +248,7 @@ extern "C" int llmrs_qkv_rope_cache(hipStream_t stream, int dtype, const void* x
     }
     LLMRS_REQUIRE(scale_sumsq == nullptr, "qkv_rope_cache: a deferred norm needs the fused bfloat16 kernel (M=%d K=%d)", M, K);
     int rc = llmrs_gemm(stream, dtype, x, lda, w, qkv, row_stride, M, N, K, LLMRS_EPI_STORE, workspace, workspace_bytes,
-                        allow_mfma, nullptr, 0, 0.0f, nullptr, nullptr, 0, nullptr);
+                        allow_mfma, nullptr, 0, 0.0f, nullptr, nullptr, 0, nullptr, 0.0f);
     if (rc != 0) return rc;
     return llmrs_rope_kv_write(stream, dtype, qkv, row_stride, positions, slot_map, inv_freq, rotary_dim, 1, k_cache,
                                v_cache, M, n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv);

@@ -76,6 +76,7 @@ class StepContext:
         self.norm_after_block = None
         self._left = None               # kernels.NextNorm that describes the stream as it stands, or None
         self._left_of = 0               # the stream it describes
+        self._last_y = 0                # where the rows left last lie
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)
@@ -90,15 +91,29 @@ class StepContext:
         weight = norm.deferred_weight() if norm is not None else None
         defers = getattr(k, "gemm_defers_norm", None)
         T, N = h.shape[0], w.shape[0]
-        if (weight is None or defers is None or w.dtype != torch.bfloat16 or N != h.shape[1] or weight.shape[0] != N
-                or N >= 16384 or not defers(T, N, w.shape[1])):
+        if weight is None or defers is None or w.dtype != torch.bfloat16 or N != h.shape[1] or weight.shape[0] != N:
             return None
-        return NextNorm(self.workspace("model.prenormed", (T, N), torch.bfloat16),
-                        self.workspace("model.sumsq", (T, -(-N // 16)), torch.float32), weight)
+        if N < 16384 and defers(T, N, w.shape[1]):
+            return NextNorm(self._prenormed(T, N), self.workspace("model.sumsq", (T, -(-N // 16)), torch.float32), weight)
+        # more rows: a product that is split over blocks finishes the norm where its parts are added up
+        whole, eps = getattr(k, "gemm_norms_whole", None), norm.deferred_eps()
+        if whole is not None and eps is not None and eps > 0 and whole(T, N, w.shape[1]):
+            return NextNorm(self._prenormed(T, N), None, weight, eps)
+        return None
+
+    def _prenormed(self, T: int, N: int) -> torch.Tensor:
+        """Room for the rows a product leaves: not the rows that were left last, which the part at work may
+        still be reading as its input."""
+        y = self.workspace("model.prenormed", (T, N), torch.bfloat16)
+        if self._last_y == y.data_ptr():
+            y = self.workspace("model.prenormed.other", (T, N), torch.bfloat16)
+        return y
 
     def note_left(self, h: torch.Tensor, left) -> None:
         """`left` (a filled NextNorm, or None) is what describes `h` from now on."""
         self._left, self._left_of = left, (h.data_ptr() if left is not None else 0)
+        if left is not None:
+            self._last_y = left.y.data_ptr()
 
     def left_for(self, h: torch.Tensor):
         """What the last product that added into `h` left for the norm that follows, or None."""

@@ -48,10 +48,16 @@ class NormedRows:
 
 class NextNorm:
     """What a product that adds into the stream leaves for the norm that follows, see `NormedRows`:
-    `y` and `sumsq` to fill, `weight` the following norm's."""
+    `y` and `sumsq` to fill, `weight` the following norm's.  With `eps` (and no `sumsq`) the product finishes the
+    norm itself: `y` becomes the normed rows, for any product to take as they are (`gemm_norms_whole`: steps of
+    17 to 256 tokens whose product is split over blocks, where the kernel that adds the parts up sees whole rows)."""
 
-    def __init__(self, y: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor):
-        self.y, self.sumsq, self.weight = y, sumsq, weight
+    def __init__(self, y: torch.Tensor, sumsq: Optional[torch.Tensor], weight: torch.Tensor, eps: float = 0.0):
+        self.y, self.sumsq, self.weight, self.eps = y, sumsq, weight, float(eps)
+
+    @property
+    def whole(self) -> bool:
+        return self.eps > 0.0
 
 
 class KernelTimes:
@@ -132,8 +138,9 @@ class HipKernels:
             "llmrs_cast": [V, V, I, V, I, c_size_t],
             "llmrs_scale_softcap_rows": [V, V, I, I, I, F, F],
             "llmrs_rmsnorm": [V, I, V, V, V, V, I, I, F],
-            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V],
+            "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F],
             "llmrs_gemm_defers_norm": [I, I, I],
+            "llmrs_gemm_norms_whole": [I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
             "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I, V, I, F],
@@ -168,6 +175,11 @@ class HipKernels:
         """Whether the bfloat16 product of M rows with an [N, K] weight takes `NormedRows` as its rows and, adding
         into the stream, leaves a `NextNorm` (that: for fewer than 16384 features)."""
         return self.allow_mfma and bool(self.lib.llmrs_gemm_defers_norm(int(M), int(N), int(K)))
+
+    def gemm_norms_whole(self, M: int, N: int, K: int) -> bool:
+        """Whether the bfloat16 product of M rows with an [N, K] weight, adding into the stream with the workspace
+        `gemm_workspace_floats` asks for, can finish the norm that follows (a `NextNorm` with eps)."""
+        return self.allow_mfma and bool(self.lib.llmrs_gemm_norms_whole(int(M), int(N), int(K)))
 
     def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int,
                                  n_kv_heads: Optional[int] = None, n_single: int = 0) -> int:
@@ -244,24 +256,29 @@ class HipKernels:
         M, K = a.shape
         N = w.shape[0]
         assert w.shape[1] == K and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1 and a.dtype == w.dtype
+        whole = leave is not None and leave.whole
         if leave is not None:
-            assert epilogue == EPI_ACCUM_F32 and N < 16384 and leave.sumsq.dtype == torch.float32 and leave.sumsq.is_contiguous()
-            assert tuple(leave.sumsq.shape) == (M, -(-N // 16)) and tuple(leave.y.shape) == (M, N) and leave.y.stride(1) == 1
+            assert epilogue == EPI_ACCUM_F32 and tuple(leave.y.shape) == (M, N) and leave.y.stride(1) == 1
             assert leave.y.dtype == torch.bfloat16 and leave.weight.dtype == torch.float32 and leave.weight.shape[0] == N
-        if scale is not None or leave is not None:
+            if not whole:
+                assert N < 16384 and leave.sumsq.dtype == torch.float32 and leave.sumsq.is_contiguous()
+                assert tuple(leave.sumsq.shape) == (M, -(-N // 16))
+        if whole:
+            assert a.dtype == torch.bfloat16 and scale is None and self.gemm_norms_whole(M, N, K) and workspace is not None
+        elif scale is not None or leave is not None:
             assert a.dtype == torch.bfloat16 and self.gemm_defers_norm(M, N, K)
         want = torch.float32 if epilogue in (EPI_STORE_F32, EPI_ACCUM_F32) else a.dtype
         assert out.dtype == want and out.shape[0] == M and out.shape[1] == (N // 2 if epilogue == EPI_SWIGLU else N)
         moved = (M * K + N * K) * a.element_size() + out.numel() * out.element_size() * (2 if epilogue == EPI_ACCUM_F32 else 1)
-        label = f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{'+next' if leave is not None else ''}"
+        label = f"gemm {M}x{N}x{K} {'norm+' if scale is not None else ''}{_EPI_NAMES[epilogue]}{('+norm' if whole else '+next') if leave is not None else ''}"
         self._run(label, moved, 2 * M * N * K, a.dtype,
                   self.lib.llmrs_gemm, self._stream(), _code(a.dtype), _p(a), a.stride(0), _p(w), _p(out), out.stride(0),
                   M, N, K, epilogue, _p(workspace),
                   0 if workspace is None else workspace.numel() * workspace.element_size(), int(self.allow_mfma),
                   None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
-                  0.0 if scale is None else scale.eps, None if leave is None else _p(leave.sumsq),
+                  0.0 if scale is None else scale.eps, None if leave is None or whole else _p(leave.sumsq),
                   None if leave is None else _p(leave.y), 0 if leave is None else leave.y.stride(0),
-                  None if leave is None else _p(leave.weight))
+                  None if leave is None else _p(leave.weight), leave.eps if whole else 0.0)
 
     def rope_kv_write(self, qkv, positions, slot_map, inv_freq, rotary_dim, interleaved, k_cache, v_cache,
                       n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv) -> None:

@@ -86,9 +86,15 @@ class Norm(Part):
         None for any other norm."""
         return None
 
+    def deferred_eps(self) -> Optional[float]:
+        """For a norm of that form: its eps, which lets a product that sees whole rows finish the norm itself
+        (`kernels.NextNorm` with eps); None for any other norm."""
+        return None
+
     def deferred(self, ctx, h: torch.Tensor):
-        """The norm of every row of `h`, not computed: a `kernels.NormedRows` for a part that
-        `takes_normed_rows`, or None when this norm cannot be left to the next product (then `forward` runs)."""
+        """The norm of every row of `h`, not computed here: a `kernels.NormedRows` for a part that
+        `takes_normed_rows`, or the normed rows themselves (a tensor) where the last product that added into `h`
+        finished this norm, or None when neither holds (then `forward` runs)."""
         return None
 
 
@@ -164,7 +170,9 @@ class Block:
         """The input of `part`: norm(h), computed here, or left to the part's first product where the norm can be
         deferred and the part takes such rows (a step of few tokens whose stream was last written by a product
         that prepared this norm: then no norm kernel runs).  `then` is the norm that reads the stream after `part`."""
-        rows = norm.deferred(ctx, h) if part.takes_normed_rows(ctx, h.shape[0]) else None
+        rows = norm.deferred(ctx, h)
+        if not isinstance(rows, torch.Tensor) and not part.takes_normed_rows(ctx, h.shape[0]):
+            rows = None         # (rows already normed are any part's input; rows still to be scaled only the parts' that can)
         # The part is about to change the stream: what was left stops describing it now.  (The rows handed over
         # keep their own references; a part that leaves something for `then` notes it when it is done.)
         ctx.note_left(h, None)

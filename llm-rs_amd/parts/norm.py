@@ -35,10 +35,15 @@ class RMSNorm(Norm):
     def deferred_weight(self):
         return self.weight
 
+    def deferred_eps(self):
+        return self.eps
+
     def deferred(self, ctx, h):
         left = ctx.left_for(h)
         if left is None or left.weight is not self.weight or h.shape[1] != self.size or left.y.shape != h.shape:
             return None         # nothing was left, or it was prepared for another norm
+        if left.whole:          # finished by the product that added into the stream last
+            return left.y if left.eps == self.eps else None
         return NormedRows(left.y, left.sumsq, self.eps)
 
 

@@ -795,6 +795,54 @@ def test_residual_product_leaves_what_the_next_norm_needs(M, N, K):
     assert float((h.double().cpu() - want_h).abs().max()) <= 1e-5 * math.sqrt(K) + 1e-5 * float(want_h.abs().max())
 
 
+@pytest.mark.parametrize("M,N,K", [(64, 4096, 4096), (17, 4096, 14336), (24, 1024, 2048), (33, 2048, 8192), (200, 512, 4096),
+                                   (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192)])
+def test_split_residual_product_finishes_the_next_norm(M, N, K):
+    """17 to 256 rows, a product whose sums are split over blocks: the kernel that adds the parts writes the stream and
+    the normed rows: the stream bit for bit as without, the rows as the norm kernel makes them from that stream."""
+    from llm_rs_amd.kernels import NextNorm
+    k = kernels()
+    assert k.gemm_norms_whole(M, N, K), "the case itself: this shape is split"
+    a = rnd((M, K), torch.bfloat16, 70)
+    w = rnd((N, K), torch.bfloat16, 71, 0.1)
+    h = rnd((M, N), torch.float32, 72, 2.0)
+    h[M // 2] *= 30.0               # one row far larger than the others: its scale must be its own
+    nw = rnd((N,), torch.float32, 73) * 0.1 + 1
+    eps = 3e-4
+    ws = torch.empty(k.gemm_workspace_floats(M, N, K), dtype=torch.float32, device=DEV)
+    plain = h.clone()
+    k.gemm(a, w, plain, EPI_ACCUM_F32, ws)
+    y = torch.full((M, N + 4), 7.0, dtype=torch.bfloat16, device=DEV)
+    k.gemm(a, w, h, EPI_ACCUM_F32, ws, leave=NextNorm(y[:, :N], None, nw, eps))
+    assert torch.equal(h, plain), "finishing the norm does not change the product"
+    assert (y[:, N:] == 7.0).all(), "padding touched"
+    want_h = rnd((M, N), torch.float32, 72, 2.0).double().cpu()
+    want_h[M // 2] *= 30.0
+    want_h += a.double().cpu() @ w.double().cpu().T
+    assert float((h.double().cpu() - want_h).abs().max()) <= 1e-5 * math.sqrt(K) + 1e-5 * float(want_h.abs().max())
+    normed = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    k.rmsnorm(normed, h, nw, eps)
+    hd = h.double().cpu()
+    exact = hd / torch.sqrt((hd * hd).mean(-1, keepdim=True) + eps) * nw.double().cpu()
+    err = (y[:, :N].double().cpu() - exact).abs()
+    assert (err <= exact.abs() * 2 ** -8 + 1e-6).all(), "within a rounding to bfloat16 of the exact norm"
+    # the norm kernel adds the squares in another order: a unit in the last place here and there, no more
+    differ = (y[:, :N].float() - normed.float()).abs()
+    assert (differ <= normed.float().abs() * 2 ** -7 + 1e-6).all() and float((differ > 0).float().mean()) < 0.02
+
+
+def test_a_norm_cannot_be_finished_by_a_product_that_is_not_split():
+    from llm_rs_amd.kernels import KernelError, NextNorm
+    k = kernels()
+    M, N, K = 64, 24576, 4096
+    assert not k.gemm_norms_whole(M, N, K)
+    a, w = rnd((M, K), torch.bfloat16, 1), rnd((N, K), torch.bfloat16, 2, 0.1)
+    h = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+    y = torch.zeros((M, N), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises((KernelError, AssertionError)):
+        k.gemm(a, w, h, EPI_ACCUM_F32, torch.empty(1 << 20, dtype=torch.float32, device=DEV), leave=NextNorm(y, None, torch.ones(N, device=DEV), 1e-5))
+
+
 @pytest.mark.parametrize("M,n_heads,n_kv,hd,rot,K", [(8, 32, 8, 128, 128, 4096), (1, 32, 8, 128, 128, 4096), (16, 3, 1, 32, 32, 128),
                                                       (5, 4, 2, 16, 8, 64), (3, 64, 8, 128, 128, 8192), (7, 2, 2, 64, 0, 192)])
 def test_qkv_rope_cache_finishes_a_norm_left_to_it(M, n_heads, n_kv, hd, rot, K):
