@@ -1,7 +1,9 @@
-"""Builds and loads the two native libraries.
+"""Builds and loads the native libraries.
 
-`libllmrs_host.so`  g++     cache manager, batch builder, scheduler (csrc/host)
-`libllmrs_hip.so`   hipcc   the gfx950 kernels and their launchers (csrc/hip)
+`libllmrs_host.so`   g++     cache manager, batch builder, scheduler (csrc/host)
+`libllmrs_hip.so`    hipcc   the gfx950 kernels and their launchers (csrc/hip)
+`libllmrs_plain.so`  g++     plain C++ twins of the kernels (csrc/plain): the tests' second oracle, which
+                             nothing in the package loads
 
 They are built into `csrc/_build/` inside the package (or, when that folder
 cannot be written, into a per-user folder under the temporary directory) the
@@ -103,6 +105,22 @@ def build_host(force: bool = False) -> str:
     return lib
 
 
+def build_plain(force: bool = False) -> str:
+    """The kernels' plain C++ twins (test equipment: the package has no CPU path and never loads them)."""
+    d = _build_dir()
+    lib = os.path.join(d, "libllmrs_plain.so")
+    if not force and _is_current(lib, "plain"):
+        return lib
+    cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
+    if cxx is None:
+        raise BuildError("no C++ compiler (g++) to build the plain twins with")
+    _say("compiling the kernels' plain C++ twins ...")
+    tmp = f"{lib}.{os.getpid()}.tmp"
+    _run([cxx, *HOST_FLAGS, "-shared", "-o", tmp, *_sources("plain", (".cpp",))], "plain twins build")
+    _finish(lib, tmp, "plain")
+    return lib
+
+
 def _hipcc() -> Optional[str]:
     for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):
@@ -168,4 +186,5 @@ def load_hip() -> ctypes.CDLL:
 
 def build_all(force: bool = True) -> None:
     build_host(force)
+    build_plain(force)
     build_hip(force)
