@@ -42,6 +42,18 @@ __device__ __forceinline__ bf16x8 zero8() {
     return z;
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+// The value the neighbouring lane (lane ^ 1) passes: a DPP move within each group of four lanes, no LDS.
+__device__ __forceinline__ float swap_neighbours(float x) {
+    int u = __float_as_int(x);
+    return __int_as_float(__builtin_amdgcn_update_dpp(u, u, 0xB1, 0xf, 0xf, true));     // quad_perm [1, 0, 3, 2]
+}
+// x / (1 + exp(-x)) with the device's exponential and reciprocal instructions (each within an ulp; the result is
+// rounded to bfloat16 right after).  For the epilogues that finish thousands of values per wave.
+__device__ __forceinline__ float silu_fast_f32(float x) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
+}
+
 // The tile loops' barrier: this wave's LDS reads and writes are done, then every wave of the block
 // has arrived.  Unlike __syncthreads() it does not wait for loads from memory that are still in
 // flight (the later tiles of a pipeline); the "memory" clobber keeps the compiler from moving
@@ -596,18 +608,27 @@ __device__ __forceinline__ void tile_epilogue(f32x16 (&acc)[BM / WGM / 32][BN / 
         const int row_bytes = cols * 2;
         static_assert(TN * 2 * TM * WAVES <= SMEM_BYTES, "the waves' tiles must fit in the tile buffers");
         unsigned char* mine = smem + wave * (TN * 2 * TM);
+        // A lane holds one column of 16 rows, its neighbour (lane ^ 1) the next column.  Registers r and r + 1
+        // are two adjacent rows: the two lanes trade one value of each pair (one DPP move, no LDS), after which the
+        // even lane has both columns of row r and the odd lane both of row r + 1.  For the gate/up epilogue those
+        // are a gate and its up (each lane finishes one output of the pair, none idles); for a plain store two
+        // neighbouring results, written with one 4-byte store.
+        const bool odd = lane & 1;
         static_for<0, FM * FN>([&](auto idx) {
             constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
             int c = j * 32 + (lane & 31);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                int row = i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                float v = acc[i][j][r];
-                if (glu) {
-                    float other = __shfl_xor(v, 1, 64);           // even lane: gate here, up next door
-                    if (!(lane & 1)) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)(silu_f32(v) * other);
-                } else {
-                    *(bf16*)(mine + row * row_bytes + c * 2) = (bf16)v;
+            for (int r = 0; r < 16; r += 2) {
+                int row = i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3) + (odd ? 1 : 0);
+                float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
+                float got = swap_neighbours(odd ? v0 : v1);
+                float left = odd ? got : v0, right = odd ? v1 : got;       // columns c & ~1 and c | 1 of `row`
+                if (glu) *(bf16*)(mine + row * row_bytes + (c / 2) * 2) = (bf16)(silu_fast_f32(left) * right);
+                else {
+                    bf16x2 two;
+                    two[0] = (bf16)left;
+                    two[1] = (bf16)right;
+                    *(bf16x2*)(mine + row * row_bytes + (c & ~1) * 2) = two;
                 }
             }
         });
@@ -951,6 +972,266 @@ static int launch_pingpong(hipStream_t stream, const bf16* A, int lda, const bf1
     return 0;
 }
 
+// ---------------------------------------------------------------------------
+// tiled, four waves: for K % 64 == 0, tiles of 256 x 256.
+// One wave per SIMD with a tile of 128 x 128 outputs, all of them in the accumulation registers (256 of them):
+// a third fewer LDS reads per MFMA than the eight-wave tiles, and nothing shares the SIMD with the wave, so the
+// loop is written so that the wave itself always has work in flight.  A k-tile of 64 is four steps of 16; each
+// step asks LDS for the operands of the next step, moves a quarter of the next k-tile from registers into the
+// other LDS buffer, asks memory for the same quarter of the k-tile after that, and multiplies the operands the
+// step before it asked for.  Loads from memory pass through registers here, two k-tiles ahead of their use (the
+// loads straight into LDS of the loops above hold a wave that has no partner on its SIMD up while the memory
+// pipeline takes them).  The barrier between k-tiles stands before the last step's products, which run on
+// registers read before it: the matrix cores work across the barrier.  Same LDS layout and order of sums as the
+// loops above: bitwise the same results.  The epilogue is a template argument: with all of them in one kernel the
+// compiler keeps a tile's 256 sums and every epilogue's temporaries alive together and spills.
+// (Measured on MI355X, 2048 x 4096 times 24576 features with the gate/up epilogue, inside a prompt step of the 8B
+// shape: 356 us against 372-376 for the eight waves in two groups and 367 with loads straight into LDS.)
+// ---------------------------------------------------------------------------
+// What a wave of the four-wave tile does with its sums: one band of 32 rows at a time.  16-bit results go through
+// the wave's own part of LDS and leave as whole rows of the band, 16 bytes a lane; the 32-bit epilogues read and
+// write memory directly (a lane half holds 32 consecutive columns of a row: whole lines).
+template <int BM, int BN, int EPI>
+__device__ __forceinline__ void band_epilogue(f32x16 (&acc)[BM / 64][BN / 64], unsigned char* smem, void* __restrict__ out,
+                                              int ldc, int M, int N, int m0, int n0) {
+    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int wm = wave / 2, wn = wave % 2;
+    int c = lane & 31, hh = lane >> 5;
+    if constexpr (EPI == LLMRS_EPI_ACCUM_F32 || EPI == LLMRS_EPI_STORE_F32) {
+        float* o = (float*)out;
+        static_for<0, FM * FN>([&](auto idx) {
+            constexpr int i = decltype(idx)::value / FN, j = decltype(idx)::value % FN;
+            int n = n0 + wn * TN + j * 32 + c;
+            float old[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                old[r] = EPI == LLMRS_EPI_ACCUM_F32 ? o[(size_t)min(m, M - 1) * ldc + min(n, N - 1)] : 0.0f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int m = m0 + wm * TM + i * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+                if (m < M && n < N) o[(size_t)m * ldc + n] = old[r] + acc[i][j][r];
+            }
+            __builtin_amdgcn_sched_barrier(0);       // one part of the tile at a time: its old values are not asked for earlier
+        });
+    } else {
+        constexpr bool glu = EPI == LLMRS_EPI_SWIGLU;
+        constexpr int cols = glu ? TN / 2 : TN;      // columns of the wave's band as stored
+        constexpr int row_bytes = cols * 2;
+        unsigned char* mine = smem + wave * (32 * TN * 2);
+        constexpr int pieces_per_row = cols / 8;     // 16-byte pieces in a row of the band
+        int n_first = glu ? (n0 + wn * TN) / 2 : n0 + wn * TN, n_lim = glu ? N / 2 : N;
+        const bool odd = lane & 1;
+        static_for<0, FM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            static_for<0, FN>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                int cc = j * 32 + c;
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {                 // (pairs of lanes trade values as in tile_epilogue)
+                    int row = 8 * (r >> 2) + 4 * hh + (r & 3) + (odd ? 1 : 0);
+                    float v0 = acc[i][j][r], v1 = acc[i][j][r + 1];
+                    float got = swap_neighbours(odd ? v0 : v1);
+                    float left = odd ? got : v0, right = odd ? v1 : got;
+                    if (glu) *(bf16*)(mine + row * row_bytes + (cc / 2) * 2) = (bf16)(silu_fast_f32(left) * right);
+                    else {
+                        bf16x2 two;
+                        two[0] = (bf16)left;
+                        two[1] = (bf16)right;
+                        *(bf16x2*)(mine + row * row_bytes + (cc & ~1) * 2) = two;
+                    }
+                }
+            });
+            __builtin_amdgcn_s_waitcnt(0xc07f);                   // lgkmcnt(0): the wave's own LDS writes are done
+            for (int piece = lane; piece < 32 * pieces_per_row; piece += 64) {
+                int row = piece / pieces_per_row, lc = (piece % pieces_per_row) * 8;
+                int m = m0 + wm * TM + i * 32 + row;
+                if (m < M && n_first + lc < n_lim)                // (n_lim is a multiple of 8: a lane's 8 columns are in or out together)
+                    *(bf16x8*)((bf16*)out + (size_t)m * ldc + n_first + lc) = *(const bf16x8*)(mine + row * row_bytes + lc * 2);
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);                   // the band's rows are read before the next band overwrites them
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    }
+}
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int BM, int BN, int EPI>
+__global__ __launch_bounds__(256) void gemm_fourwave_kernel(const bf16* __restrict__ A, int lda, const bf16* __restrict__ W,
+                                                            void* __restrict__ out, int ldc, int M, int N, int K) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char fw_smem[];
+    constexpr int WAVES = 4;
+    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32;
+    constexpr int STAGE_BYTES = (BM + BN) * 128;
+    constexpr int A_GROUPS = BM / 8 / WAVES, W_GROUPS = BN / 8 / WAVES;   // 8-row groups per wave
+    constexpr int QA = A_GROUPS / 4, QW = W_GROUPS / 4, QL = QA + QW;     // a quarter of a wave's loads of a k-tile
+    static_assert(BM == 256 && BN % 64 == 0 && FM * FN <= 16, "a wave's sums fill at most the 256 accumulation registers");
+    static_assert(A_GROUPS % 4 == 0 && W_GROUPS % 4 == 0, "a quarter of a k-tile's loads in each of its four steps");
+    static_assert(32 * TN * 2 * WAVES <= 2 * STAGE_BYTES, "the waves' bands must fit in the tile buffers");
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int wm = wave / 2, wn = wave % 2;
+    int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    int lrow = lane >> 3, lslot = lane & 7;
+    // this lane's part of a tile: for each of its row groups, the byte offset of the chunk that belongs in the lane's
+    // slot of the LDS image (the caller sees to it that both operands are under 4 GB: buffer descriptors)
+    unsigned oa[A_GROUPS], ow[W_GROUPS];
+#pragma unroll
+    for (int i = 0; i < A_GROUPS; ++i) {
+        int row = (wave * A_GROUPS + i) * 8 + lrow;
+        oa[i] = (unsigned)(((size_t)min(m0 + row, M - 1) * lda + ((lslot ^ ((row >> 1) & 7)) * 8)) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+        int row = (wave * W_GROUPS + i) * 8 + lrow;
+        ow[i] = (unsigned)(((size_t)min(n0 + row, N - 1) * K + ((lslot ^ ((row >> 1) & 7)) * 8)) * 2);
+    }
+    const int nk = K / 64;
+#if defined(__HIP_DEVICE_COMPILE__)
+    __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)min((size_t)M * lda * 2, (size_t)0xffffffffu), 0x00020000);
+    __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)min((size_t)N * K * 2, (size_t)0xffffffffu), 0x00020000);
+#endif
+    u32x4 sa[A_GROUPS], sw_[W_GROUPS];          // the k-tile on its way, in registers
+    // quarter q of this wave's loads of k-tile kt, into registers (past the end: the last tile once more, never used)
+    auto ask = [&](int kt, auto qc) {
+        constexpr int q = decltype(qc)::value;
+        kt = min(kt, nk - 1);
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+        for (int i = q * QA; i < (q + 1) * QA; ++i) sa[i] = __builtin_amdgcn_raw_buffer_load_b128(ra, oa[i], kt * 128, 0);
+#pragma unroll
+        for (int i = q * QW; i < (q + 1) * QW; ++i) sw_[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, ow[i], kt * 128, 0);
+#endif
+    };
+    // quarter q of the registers into the LDS buffer of k-tile kt: a load's 64 lanes fill 1 KB in lane order
+    auto put = [&](int kt, auto qc) {
+        constexpr int q = decltype(qc)::value;
+        unsigned char* st = fw_smem + (kt & 1) * STAGE_BYTES;
+#pragma unroll
+        for (int i = q * QA; i < (q + 1) * QA; ++i) *(u32x4*)(st + (wave * A_GROUPS + i) * 1024 + lane * 16) = sa[i];
+#pragma unroll
+        for (int i = q * QW; i < (q + 1) * QW; ++i) *(u32x4*)(st + BM * 128 + (wave * W_GROUPS + i) * 1024 + lane * 16) = sw_[i];
+    };
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    int frow = lane & 31, h = lane >> 5;
+    int sw = (frow >> 1) & 7;
+    // LDS offsets of this lane's chunk for each of a tile's four k-steps (row tiles lie 4 KB apart)
+    unsigned offa[4], offb[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        unsigned chunk = (unsigned)(((ks * 2 + h) ^ sw) * 16);
+        offa[ks] = (wm * TM + frow) * 128 + chunk;
+        offb[ks] = BM * 128 + (wn * TN + frow) * 128 + chunk;
+    }
+    bf16x8 fa[2][FM], fb[2][FN];
+    auto read = [&](int kt, auto ksc, auto bufc) {
+        constexpr int ks = decltype(ksc)::value, buf = decltype(bufc)::value;
+        const unsigned char* st = fw_smem + (kt & 1) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) fa[buf][i] = *(const bf16x8*)(st + offa[ks] + i * 32 * 128);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) fb[buf][j] = *(const bf16x8*)(st + offb[ks] + j * 32 * 128);
+    };
+    auto mult = [&](auto bufc) {
+        constexpr int buf = decltype(bufc)::value;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+    };
+    // the order within a step: LDS reads, LDS writes and loads from memory each ahead of a group of the step's MFMAs
+    auto order = [] {
+        __builtin_amdgcn_sched_group_barrier(0x100, FM + FN, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, QL, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, QL, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - 8, 0);
+    };
+    // One step (a quarter of a k-tile).  While k-tile kt is multiplied, k-tile kt + 1 goes from registers into the
+    // other LDS buffer and k-tile kt + 2 is asked for into the registers that frees.  A quarter written now was
+    // asked for a k-tile ago; loads complete in order, so it is there when all but the three quarters asked for
+    // since have completed.
+    auto step = [&](int kt, auto ksc, auto qc, auto rbuf, auto mbuf, auto multiply) {
+        read(kt, ksc, rbuf);
+        wait_vmcnt<3 * QL>();
+        put(kt + 1, qc);
+        ask(kt + 2, qc);
+        if constexpr (decltype(multiply)::value) mult(mbuf);
+        order();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    // k-tile 0 into LDS, k-tile 1 into registers
+    ask(0, I0{}); ask(0, I1{}); ask(0, I2{}); ask(0, I3{});
+    wait_vmcnt<0>();
+    put(0, I0{}); put(0, I1{}); put(0, I2{}); put(0, I3{});
+    ask(1, I0{}); ask(1, I1{}); ask(1, I2{}); ask(1, I3{});
+    __syncthreads();               // (waits for the loads of k-tile 1 as well: once)
+    // A step multiplies the operands that the step before it read; the last step's products of a k-tile run in the
+    // first step of the next, on operands read before the barrier: the matrix cores work across it.
+    auto k_tile = [&](int kt, auto not_first) {
+        step(kt, I0{}, I0{}, I0{}, I1{}, not_first);
+        step(kt, I1{}, I1{}, I1{}, I0{}, std::true_type{});
+        step(kt, I2{}, I2{}, I0{}, I1{}, std::true_type{});
+        step(kt, I3{}, I3{}, I1{}, I0{}, std::true_type{});
+        block_sync_lds();          // this wave's LDS reads and writes are done, and everybody's
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    k_tile(0, std::false_type{});
+    for (int kt = 1; kt < nk; ++kt) k_tile(kt, std::true_type{});
+    mult(I1{});
+    wait_vmcnt<0>();
+    __syncthreads();
+    band_epilogue<BM, BN, EPI>(acc, fw_smem, out, ldc, M, N, m0, n0);
+}
+
+// Whether the four-wave tiles can finish this product: the epilogues it has, 16-bit results as whole 16-byte pieces.
+static bool fourwave_takes(int epi, const void* out, int ldc, int N) {
+    if (epi == LLMRS_EPI_ACCUM_F32 || epi == LLMRS_EPI_STORE_F32) return true;
+    if (epi == LLMRS_EPI_STORE) return ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 && N % 8 == 0;
+    if (epi == LLMRS_EPI_SWIGLU) return ldc % 8 == 0 && ((uintptr_t)out & 15) == 0 && N % 16 == 0;
+    return false;
+}
+template <int BM, int BN, int EPI>
+static int launch_fourwave_epi(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc, int M, int N, int K) {
+    static bool configured = false;
+    size_t bytes = (size_t)2 * (BM + BN) * 128;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_fourwave_kernel<BM, BN, EPI>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return llmrs_fail("gemm: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+        configured = true;
+    }
+    dim3 grid(ceil_div(N, BN), ceil_div(M, BM));
+    if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
+    gemm_fourwave_kernel<BM, BN, EPI><<<grid, 256, bytes, stream>>>(A, lda, W, out, ldc, M, N, K);
+    return 0;
+}
+// (operands under 4 GB each, K % 64 == 0, fourwave_takes(epi, ...): the caller's to check)
+template <int BM, int BN>
+static int launch_fourwave(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc, int M, int N, int K, int epi) {
+    switch (epi) {
+        case LLMRS_EPI_STORE: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE>(stream, A, lda, W, out, ldc, M, N, K);
+        case LLMRS_EPI_STORE_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_STORE_F32>(stream, A, lda, W, out, ldc, M, N, K);
+        case LLMRS_EPI_ACCUM_F32: return launch_fourwave_epi<BM, BN, LLMRS_EPI_ACCUM_F32>(stream, A, lda, W, out, ldc, M, N, K);
+        case LLMRS_EPI_SWIGLU: return launch_fourwave_epi<BM, BN, LLMRS_EPI_SWIGLU>(stream, A, lda, W, out, ldc, M, N, K);
+        default: return llmrs_fail("gemm: the four-wave tiles have no epilogue %d", epi);
+    }
+}
+
 // Into how many parts the k range is split over blocks (1: not at all), by the product's shape alone.
 // 17 to 64 rows (few-row kernel, 64 features per block): when the features give no more than 64
 // blocks, until there are 256 of them, each part at least 16 k-blocks long (measured at 64 rows:
@@ -1153,24 +1434,30 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         if (K % 64 == 0 && big_tiles >= 160 && M > 128) {
             // operands under 4 GB are read through buffer descriptors (32-bit offsets), 1-4 % faster
             const bool small = (size_t)M * lda * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32);
+            // square tiles: four waves with 128 x 128 outputs each where their epilogues and loads allow, else the
+            // eight waves in two groups
+            const bool four = small && fourwave_takes(epi, out, ldc, N);
             long whole = big_tiles / cus * cus, rest = big_tiles - whole;
             int n_split = (int)(whole / m_tiles) * 256;        // features of the whole rounds
             if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4) {
                 size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
                 void* out_rest = (char*)out + (size_t)(epi == LLMRS_EPI_SWIGLU ? n_split / 2 : n_split) * elt;
-                rc = small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
-                           : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
+                rc = four && fourwave_takes(epi, out, ldc, n_split)
+                         ? launch_fourwave<256, 256>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
+                     : small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
+                             : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
                 if (rc == 0)
                     rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
             } else if (long t192 = m_tiles * ceil_div(N, 192); rest > 0 && t192 % cus == 0) {
-                // 256 x 192 tiles (eight waves of 64 x 96) where they come to whole rounds of the device and the
-                // square ones do not: the q/k/v product of the 8B shape at 2048 rows is 192 square tiles on
-                // 256 units, or 256 of these
+                // 256 x 192 tiles where they come to whole rounds of the device and the square ones do not: the
+                // q/k/v product of the 8B shape at 2048 rows is 192 square tiles on 256 units, or 256 of these
+                // (eight waves of 64 x 96: in a prompt step 103 us, against 107 for four waves of 128 x 96)
                 rc = small ? launch_pingpong<256, 192, 4, 2, true>(stream, A, lda, W, out, ldc, M, N, K, epi)
                            : launch_pingpong<256, 192, 4, 2, false>(stream, A, lda, W, out, ldc, M, N, K, epi);
             } else {
-                rc = small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, N, K, epi)
-                           : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, N, K, epi);
+                rc = four ? launch_fourwave<256, 256>(stream, A, lda, W, out, ldc, M, N, K, epi)
+                     : small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, N, K, epi)
+                             : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, N, K, epi);
             }
         } else if (K % 64 == 0) {
             int splits = tiled_splits(M, N, K);

@@ -65,6 +65,9 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (1, 16400, 200), (8, 16500, 328), (30, 17000, 136), (64, 16390, 264), (8, 28672, 256), (40, 28672, 192),
                # more large tiles than compute units, the last round not full: the features are split between two tile sizes
                (513, 25600, 64),
+               # square large tiles of four waves (whole rounds; the last tile cut by M and N), and a width whose 16-bit
+               # rows are no whole 16-byte pieces, which the eight-wave tiles take
+               (2048, 8192, 512), (300, 41000, 192), (260, 41004, 128),
                # few tiles and a long k: the k range is split over blocks and the parts are added by a second kernel
                (100, 300, 4096), (257, 384, 1536), (200, 2048, 2048),
                # up to 256 rows and no more tiles than compute units: one block of eight waves per unit, four k-tiles in LDS
