@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context already in the cache, decode K steps
@@ -20,6 +20,8 @@ The other workloads print one line of the same form each:
             one 2,048-token prompt portion, as one step; value = tokens a second of that step.
   sizes     the 8B shape at further sizes: decode at context 8128 (up to the configuration's 8192 positions;
             batch 1/8/64) and at batch 128/256 (context 2048), each with its share of the HBM roofline.
+  sizes1b   the 1B shape decoding at batch 1/8/64 (context 2048) with its shares of the HBM roofline: batch 1 is
+            the case the reference states its own bandwidth figure for.
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -50,7 +52,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -145,12 +147,14 @@ def mixed_line(args, layers, step_s, weight_bytes, cache_bytes, host) -> dict:
     return line
 
 
-def sizes_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
+def sizes_line(args, layers, points, fractions, first_step_s=0.0, model="Llama-3.1-8B shape") -> dict:
     """`value` and `ms_per_step` are the first point's; the others stand under `points`."""
     first = next(iter(points))
-    line = base_line("decode tok/s of the 8B shape at further sizes (context 8128; batch 128 and 256), each with its share of the HBM roofline",
+    what = ("further sizes (context 8128; batch 128 and 256)" if model == "Llama-3.1-8B shape"
+            else "batch 1, 8 and 64 (context 2048; batch 1 is the reference's own headline case)")
+    line = base_line(f"decode tok/s of the {model.split()[0].split('-')[-1]} shape at {what}, each with its share of the HBM roofline",
                      points[first], args.steps, args.warmup, first_step_s, args.dtype,
-                     flat_config("Llama-3.1-8B shape", layers, 0, 8192, 16))
+                     flat_config(model, layers, 0, 8192 if model == "Llama-3.1-8B shape" else 2048, 16))
     line["points"] = points
     line["roofline_frac"] = fractions
     return line
@@ -268,9 +272,10 @@ def run_sizes(args) -> dict:
     steps, warmup = max(args.steps // 2, 8), max(args.warmup // 2, 2)
     long = 8192 - 64        # decoding ends just under the configuration's 8192 positions (block tables 512 pages wide)
     assert steps + warmup <= 56
-    cases = [(1, long), (8, long), (64, long), (128, 2048), (256, 2048)]
+    small = args.workload == "sizes1b"
+    cases = [(1, 2048), (8, 2048), (64, 2048)] if small else [(1, long), (8, long), (64, long), (128, 2048), (256, 2048)]
     pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
-    b = Bench(args, LLAMA_8B, pages, 256, 2048)
+    b = Bench(args, LLAMA_1B if small else LLAMA_8B, pages, 256, 2048)
     weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
     points, fractions, first_s = {}, {}, None
     for batch, ctx in cases:
@@ -280,7 +285,8 @@ def run_sizes(args) -> dict:
         points[key] = round(batch / s, 1)
         fractions[key] = round((weight_bytes + batch * (ctx + warmup + steps // 2) * per_token) / s / PEAK_HBM, 4)
         print(f"[bench] {key}: {s * 1e3:.3f} ms/step, {fractions[key] * 100:.1f}% of the HBM roofline", file=sys.stderr, flush=True)
-    return sizes_line(args, b.config.num_hidden_layers, points, fractions, first_s)
+    return sizes_line(args, b.config.num_hidden_layers, points, fractions, first_s,
+                      "Llama-3.2-1B shape" if small else "Llama-3.1-8B shape")
 
 
 def run_serve1b(args) -> dict:
@@ -354,7 +360,7 @@ def main() -> int:
     heavy = args.workload == "mixed70b"
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
-    line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes}[args.workload](args)
+    line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

@@ -71,3 +71,5 @@ def test_lines_of_every_workload():
     line = check_line(b.sizes_line(args, 32, {"decode_b1_ctx8192": 250.0, "decode_b256_ctx2048": 15000.0},
                                    {"decode_b1_ctx8192": 0.5, "decode_b256_ctx2048": 0.4}))
     assert set(line["points"]) == set(line["roofline_frac"])
+    line = check_line(b.sizes_line(args, 16, {"decode_b1_ctx2048": 900.0}, {"decode_b1_ctx2048": 0.4}, 0.0011, "Llama-3.2-1B shape"))
+    assert line["config"]["model"] == "Llama-3.2-1B shape" and line["config"]["hidden_size"] == 2048 and "1B shape" in line["metric"]
