@@ -27,7 +27,7 @@ struct QkvEpilogue {
 // RMSNorm without a kernel of its own, for steps of up to 16 tokens.  The product that adds into the
 // 32-bit stream (its last writer before a norm) also leaves, for the norm that follows,
 //   y[m, n]     = bfloat16(h[m, n] * weight[n])        the new row times the norm's weight, rounded once
-//   sumsq[m, p] = sum of h[m, n]^2 over the 16 features n of group p
+//   sumsq[m, p] = sum of h[m, n]^2 over the 16 (for some shapes 8) features n of group p
 // (NextNorm); the product that follows takes y as its rows and multiplies each of its 32-bit sums by
 //   inv[m] = 1 / sqrt(sum_p sumsq[m, p] / K + eps)       (RowScale; the groups are added in a fixed order)
 // before its epilogue.  x W^T with x = h inv weight is the same number as inv (h weight) W^T; what
@@ -38,7 +38,7 @@ struct QkvEpilogue {
 //   y[m, n] = bfloat16(h[m, n] * inv[m] * weight[n])
 // which any product takes as plain rows (sumsq is not used then).
 struct NextNorm {
-    float* sumsq;          // [M, ceil(N / 16)] (not used with eps > 0)
+    float* sumsq;          // [M, llmrs_gemm_next_parts(M, N, K)]: a part per 16 features, or per 8 (not used with eps > 0)
     bf16* y;               // [M, N], row stride ldy; null: nothing is left
     int ldy;
     const float* weight;   // [N]
@@ -68,6 +68,8 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                          const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr);
 // Whether the bfloat16 product of this shape goes to the kernel that can scale its rows' sums and leave a NextNorm.
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K);
+// The parts per row of the sums of squares that such a product leaves (NextNorm): what the caller sizes sumsq by.
+extern "C" int llmrs_gemm_next_parts(int M, int N, int K);
 // Whether the bfloat16 product of this shape, adding into the stream and given the workspace that
 // llmrs_gemm_workspace_floats asks for, is split over blocks so that it can finish the following norm (NextNorm with eps).
 extern "C" int llmrs_gemm_norms_whole(int M, int N, int K);

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int row = lane & 15, g = lane >> 4;
     constexpr int BF = (NT - 1) * 16 + LAST;       // features of a block
-    static_assert(LAST == 16 || (LAST == 8 && NT >= 2), "a whole last tile, or half of one");
+    static_assert(LAST == 16 || LAST == 8, "a whole last tile, or half of one");
     int n0 = blockIdx.x * BF;
     const bool last_asks = LAST == 16 || row < LAST;   // whether this lane's row of the last tile exists
     const bf16* wp[NT];
@@ -193,12 +193,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     if (rs.sumsq != nullptr && wave < MT * NT) {
         const float* sp = rs.sumsq + (size_t)min(row, M - 1) * rs.nparts;
         float ss = 0.0f;
-        if (rs.nparts % 256 == 0 && ((uintptr_t)rs.sumsq & 15) == 0) {
-            // sixteen loads on their way at a time (the sums were written on other XCDs and come from memory)
+        if (rs.nparts % 16 == 0 && ((uintptr_t)rs.sumsq & 15) == 0) {
+            // up to sixteen loads on their way at a time (the sums were written on other XCDs and come from memory);
+            // a group past the row's parts adds zeros
             for (int base = 4 * g; base < rs.nparts; base += 256) {
                 f32x4 p[16];
 #pragma unroll
-                for (int t = 0; t < 16; ++t) p[t] = *(const f32x4*)(sp + base + 16 * t);
+                for (int t = 0; t < 16; ++t)
+                    p[t] = base + 16 * t < rs.nparts ? *(const f32x4*)(sp + base + 16 * t) : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t = 0; t < 16; ++t) { ss += p[t][0]; ss += p[t][1]; ss += p[t][2]; ss += p[t][3]; }
             }
@@ -301,8 +303,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
                     for (int r = 0; r < 4; ++r)
                         if (n + r < N) nn.y[(size_t)m * nn.ldy + n + r] = y4[r];
                 ss += __shfl_xor(ss, 16, 64);
-                ss += __shfl_xor(ss, 32, 64);
-                if (g == 0) nn.sumsq[(size_t)m * ((N + 15) / 16) + (n0 / 16 + nt)] = ss;
+                if constexpr (LAST == 16) {
+                    ss += __shfl_xor(ss, 32, 64);
+                    if (g == 0) nn.sumsq[(size_t)m * ((N + 15) / 16) + (n0 / 16 + nt)] = ss;
+                } else {
+                    // blocks of 8 features (NT = 1: the launcher sees to it): a part is the block's 8, held by two lanes
+                    if (g == 0) nn.sumsq[(size_t)m * ((N + 7) / 8) + n0 / 8] = ss;
+                }
             }
         } else {
 #pragma unroll
@@ -1300,6 +1307,16 @@ static bool half_tile_blocks(int N, int whole, int cus) {
 }
 
 extern "C" int llmrs_gemm_defers_norm(int M, int N, int K) { return M >= 1 && M <= 16 && N >= 1 && K % 8 == 0; }
+// Up to 16 rows on a narrow weight with long rows (16-feature blocks would leave half of the compute units without
+// one): blocks of 8 features, half a tile each (the tile's other rows are never asked for).  Measured at 1 row:
+// 2048 x 8192 14.8 -> 12.3 us, 2048 x 2048 6.1 -> 5.6 us.
+static bool half_blocks_for_narrow(int N, int K) {
+    return N < 16384 && K >= 2048 && N % 8 == 0 && ceil_div(N, 16) * 2 <= llmrs_compute_units();
+}
+// How many partial sums of squares per row such a product leaves for the norm that follows (NextNorm without eps).
+extern "C" int llmrs_gemm_next_parts(int M, int N, int K) {
+    return M <= 16 && half_blocks_for_narrow(N, K) ? ceil_div(N, 8) : ceil_div(N, 16);
+}
 // 17 to 256 rows whose sums are split over blocks: the kernel that adds the parts up can finish the following norm.
 extern "C" int llmrs_gemm_norms_whole(int M, int N, int K) {
     return M > 16 && M <= 256 && N >= 4 && N % 4 == 0 && N <= 16384 && K % 8 == 0 && llmrs_gemm_workspace_floats(M, N, K) > 0;
@@ -1370,6 +1387,8 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                 // 256: 384 blocks) and blocks of 24 to whole rounds: those, when nothing is to be left for a norm (which
                 // counts its sums by 16 features)
                 if (K >= 16384 && N >= 8192) SKINNY(1, 2, 8, 4);   // 8192 x 28672: 90 -> 83 us
+                else if (half_blocks_for_narrow(N, K))
+                    launch_skinny<1, 1, 8, 4, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, next);
                 else if (next == nullptr && half_tile_blocks(N, 16, cus))
                     launch_skinny<1, 2, 8, 4, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, nullptr);
                 else SKINNY(1, 1, 8, 4);

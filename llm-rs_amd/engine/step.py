@@ -94,7 +94,8 @@ class StepContext:
         if weight is None or defers is None or w.dtype != torch.bfloat16 or N != h.shape[1] or weight.shape[0] != N:
             return None
         if N < 16384 and defers(T, N, w.shape[1]):
-            return NextNorm(self._prenormed(T, N), self.workspace("model.sumsq", (T, -(-N // 16)), torch.float32), weight)
+            parts = k.gemm_next_parts(T, N, w.shape[1]) if hasattr(k, "gemm_next_parts") else -(-N // 16)
+            return NextNorm(self._prenormed(T, N), self.workspace("model.sumsq", (T, parts), torch.float32), weight)
         # more rows: a product that is split over blocks finishes the norm where its parts are added up
         whole, eps = getattr(k, "gemm_norms_whole", None), norm.deferred_eps()
         if whole is not None and eps is not None and eps > 0 and whole(T, N, w.shape[1]):

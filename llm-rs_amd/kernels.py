@@ -141,6 +141,7 @@ class HipKernels:
             "llmrs_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, c_size_t, I, V, I, F, V, V, I, V, F],
             "llmrs_gemm_defers_norm": [I, I, I],
             "llmrs_gemm_norms_whole": [I, I, I],
+            "llmrs_gemm_next_parts": [I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
             "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I, V, I, F],
@@ -175,6 +176,11 @@ class HipKernels:
         """Whether the bfloat16 product of M rows with an [N, K] weight takes `NormedRows` as its rows and, adding
         into the stream, leaves a `NextNorm` (that: for fewer than 16384 features)."""
         return self.allow_mfma and bool(self.lib.llmrs_gemm_defers_norm(int(M), int(N), int(K)))
+
+    def gemm_next_parts(self, M: int, N: int, K: int) -> int:
+        """Partial sums of squares per row that a product leaving a `NextNorm` writes (one per 16 features, for some
+        shapes per 8): the second dimension of `NextNorm.sumsq`."""
+        return int(self.lib.llmrs_gemm_next_parts(int(M), int(N), int(K)))
 
     def gemm_norms_whole(self, M: int, N: int, K: int) -> bool:
         """Whether the bfloat16 product of M rows with an [N, K] weight, adding into the stream with the workspace
@@ -262,7 +268,7 @@ class HipKernels:
             assert leave.y.dtype == torch.bfloat16 and leave.weight.dtype == torch.float32 and leave.weight.shape[0] == N
             if not whole:
                 assert N < 16384 and leave.sumsq.dtype == torch.float32 and leave.sumsq.is_contiguous()
-                assert tuple(leave.sumsq.shape) == (M, -(-N // 16))
+                assert tuple(leave.sumsq.shape) == (M, self.gemm_next_parts(M, N, K))
         if whole:
             assert a.dtype == torch.bfloat16 and scale is None and self.gemm_norms_whole(M, N, K) and workspace is not None
         elif scale is not None or leave is not None:

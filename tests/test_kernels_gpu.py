@@ -773,17 +773,21 @@ def test_gemm_finishes_a_norm_left_to_it(M, N, K, epi):
     assert ((out.double().cpu() - other).abs() <= loose).all()
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 14336), (16, 4096, 4096), (5, 200, 328), (3, 8192, 28672), (12, 100, 64)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (8, 4096, 14336), (16, 4096, 4096), (5, 200, 328), (3, 8192, 28672), (12, 100, 64),
+                                   # narrow weights with long rows: blocks of 8 features, a partial sum for each
+                                   (1, 2048, 8192), (8, 2048, 2048), (16, 1024, 4096), (3, 2040, 2048)])
 def test_residual_product_leaves_what_the_next_norm_needs(M, N, K):
     from llm_rs_amd.kernels import NextNorm
     k = kernels()
     assert k.gemm_defers_norm(M, N, K)
+    parts = k.gemm_next_parts(M, N, K)
+    per = 16 if parts == -(-N // 16) else 8
+    assert parts == -(-N // per) and (per == 8) == (N <= 2048 and K >= 2048)
     a = rnd((M, K), torch.bfloat16, 50)
     w = rnd((N, K), torch.bfloat16, 51, 0.1)
     h = rnd((M, N), torch.float32, 52, 2.0)
     nw = rnd((N,), torch.float32, 53) * 0.1 + 1
     want_h = h.double().cpu() + a.double().cpu() @ w.double().cpu().T
-    parts = -(-N // 16)
     sums = torch.full((M, parts), -1.0, dtype=torch.float32, device=DEV)
     y = torch.full((M, N + 4), 7.0, dtype=torch.bfloat16, device=DEV)
     plain = h.clone()
@@ -791,9 +795,9 @@ def test_residual_product_leaves_what_the_next_norm_needs(M, N, K):
     k.gemm(a, w, h, EPI_ACCUM_F32, None, leave=NextNorm(y[:, :N], sums, nw))
     assert torch.equal(h, plain), "leaving something for the norm does not change the product"
     assert torch.equal(y[:, :N], (h * nw).bfloat16()) and (y[:, N:] == 7.0).all()
-    padded = torch.zeros((M, parts * 16), dtype=torch.float64)
+    padded = torch.zeros((M, parts * per), dtype=torch.float64)
     padded[:, :N] = h.double().cpu()
-    want = (padded * padded).view(M, parts, 16).sum(-1)
+    want = (padded * padded).view(M, parts, per).sum(-1)
     assert float((sums.double().cpu() - want).abs().max()) <= 1e-5 * float(want.abs().max())
     assert float((h.double().cpu() - want_h).abs().max()) <= 1e-5 * math.sqrt(K) + 1e-5 * float(want_h.abs().max())
 
