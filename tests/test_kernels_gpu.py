@@ -802,6 +802,34 @@ def test_residual_product_leaves_what_the_next_norm_needs(M, N, K):
     assert float((h.double().cpu() - want_h).abs().max()) <= 1e-5 * math.sqrt(K) + 1e-5 * float(want_h.abs().max())
 
 
+@pytest.mark.parametrize("M,hidden,inter", [(1, 2048, 8192), (8, 2048, 8192), (16, 1024, 2048), (5, 4096, 14336), (3, 4096, 4096)])
+def test_a_norm_left_by_one_product_and_finished_by_the_next(M, hidden, inter):
+    """down -> (norm) -> q/k/v-like product, as a layer's end and the next layer's start: the second product's result
+    against the norm kernel on the stream followed by the plain product.  Narrow streams leave a partial sum per 8
+    features, the others per 16; the consumer takes whatever number of parts it is given."""
+    from llm_rs_amd.kernels import NextNorm, NormedRows
+    k = kernels()
+    a = rnd((M, inter), torch.bfloat16, 80)
+    w_down = rnd((hidden, inter), torch.bfloat16, 81, 0.05)
+    w_next = rnd((3 * hidden // 2, hidden), torch.bfloat16, 82, 0.1)
+    nw = rnd((hidden,), torch.float32, 83) * 0.1 + 1
+    h = rnd((M, hidden), torch.float32, 84, 2.0)
+    parts = k.gemm_next_parts(M, hidden, inter)
+    left = NextNorm(torch.zeros((M, hidden), dtype=torch.bfloat16, device=DEV), torch.zeros((M, parts), device=DEV), nw)
+    k.gemm(a, w_down, h, EPI_ACCUM_F32, None, leave=left)
+    got = torch.zeros((M, w_next.shape[0]), dtype=torch.bfloat16, device=DEV)
+    k.gemm(NormedRows(left.y, left.sumsq, 1e-5), w_next, got)
+    x = torch.zeros((M, hidden), dtype=torch.bfloat16, device=DEV)
+    k.rmsnorm(x, h, nw, 1e-5)
+    want = torch.zeros_like(got)
+    k.gemm(x, w_next, want)
+    hd = h.double().cpu()
+    exact = (hd / torch.sqrt((hd * hd).mean(-1, keepdim=True) + 1e-5) * nw.double().cpu()) @ w_next.double().cpu().T
+    scale = float(exact.abs().max())
+    assert float((got.double().cpu() - exact).abs().max()) <= 1.5 * float((want.double().cpu() - exact).abs().max()) + 2e-3 * scale
+    assert float((got.double().cpu() - exact).abs().max()) <= 2e-2 * scale
+
+
 @pytest.mark.parametrize("M,N,K", [(64, 4096, 4096), (17, 4096, 14336), (24, 1024, 2048), (33, 2048, 8192), (200, 512, 4096),
                                    (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192)])
 def test_split_residual_product_finishes_the_next_norm(M, N, K):
