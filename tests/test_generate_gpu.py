@@ -195,16 +195,18 @@ def test_recorded_decode_steps_equal_eager_ones(folders, which, dtype):
     assert recorded.runner.graph_replays >= 30 and eager.runner.graph_replays == 0
 
 
-@pytest.mark.parametrize("hidden,heads,inter", [(4096, 32, 14336), (8192, 64, 28672)])
-def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter):
+@pytest.mark.parametrize("hidden,heads,inter,layers", [(4096, 32, 14336, 1), (8192, 64, 28672, 1), (2048, 32, 8192, 2)])
+def test_layers_of_real_width_at_every_batch_size(hidden, heads, inter, layers):
     """The tiny configurations never reach the kernels that wide layers get at 17 to 64 tokens (k ranges
     split over blocks, large tiles for few rows, a rotation kernel of its own after the qkv product).
-    One layer of an 8B and of a 70B model's widths: the same decoded token alone, among 8, 24 and 48 requests and beside a prompt
-    portion, in float32 and bfloat16, against the plain implementation run on the tensors the engine gives back."""
+    One layer of an 8B and of a 70B model's widths, and two of a 1B model's (narrow weights with long rows get blocks of their
+    own, and what the second layer's first norm needs is left by the first layer's last product): the same decoded token alone,
+    among 8, 24 and 48 requests and beside a prompt portion, in float32 and bfloat16, against the plain implementation run on
+    the tensors the engine gives back."""
     from llm_rs_amd import LlamaConfig
     cfg = LlamaConfig.from_dict(dict(
-        architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=hidden, num_attention_heads=heads,
-        num_key_value_heads=8, head_dim=128, intermediate_size=inter, vocab_size=2000, rope_theta=500000.0,
+        architectures=["LlamaForCausalLM"], num_hidden_layers=layers, hidden_size=hidden, num_attention_heads=heads,
+        num_key_value_heads=8, head_dim=hidden // heads, intermediate_size=inter, vocab_size=2000, rope_theta=500000.0,
         max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=True))
     n_req, plen = 48, 24
     prompts = [random_tokens(2000, plen + 1, seed=300 + i) for i in range(n_req)]
