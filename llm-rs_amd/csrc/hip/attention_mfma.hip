@@ -629,6 +629,89 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float* __restrict
     out[(size_t)token * a.out_stride + (size_t)head * hd + d] = (bf16)(o / L);
 }
 
+// The merge for more than a few chunks (131,000 keys of one request are 256 chunks of 512).  One thread per
+// feature walks the chunks one after the other, 32 loads at a time, each batch a trip to memory: 45 us for 256
+// chunks, where the split itself takes 97; 2.1 and 2.6 us a layer more than this kernel at 32 and 63 chunks (one
+// request, 2048 and 4000 keys), the same at 16 (8 to 32 requests).  Here the block's threads stand in groups, each group a
+// row of the partial sums wide (two features a thread), and the groups share out the chunks: with 16 loads asked
+// for at once a block has 128 chunks' rows (256 at head size 64) in flight.  The groups' sums meet in LDS and are
+// added in the order of the groups, so the result does not depend on timing.  Weights as in the kernel above.
+#define MERGE_GROUP_THREADS 512
+#define MERGE_ONE_WALK_CHUNKS 8       // up to here a thread per feature walks the chunks alone (many requests, short caches)
+__global__ __launch_bounds__(MERGE_GROUP_THREADS) void attn_merge_groups_kernel(
+        const float* __restrict__ partial, bf16* __restrict__ out, const int* __restrict__ seq_lens,
+        const int* __restrict__ q_starts, AttnArgs a, int max_chunks, int chunk, int plain) {
+    __shared__ float weight[MERGE_MAX_CHUNKS];
+    __shared__ float sums[2 * MERGE_GROUP_THREADS];
+    constexpr int AHEAD = 16;
+    int e = blockIdx.x, head = blockIdx.y, hd = a.head_dim, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int per_row = hd / 2;                         // threads to a chunk's row (head sizes are even)
+    int groups = blockDim.x / per_row;            // (the launch gives a group four chunks or more)
+    int g = tid / per_row, f = tid - g * per_row; // threads past the last whole group only help with the weights
+    const bool adds = g < groups;
+    int stride = hd + 2;
+    const float* pp = partial + (size_t)(e * a.n_heads + head) * max_chunks * stride;
+    int token, pos, lo;
+    if (plain) {
+        token = e;
+        pos = seq_lens[e] - 1;
+        lo = 0;
+    } else {
+        token = q_starts[e];
+        int count = q_starts[e + 1] - token;
+        if (count != 1) return;                   // (the whole block: nothing below is reached by a part of it)
+        pos = seq_lens[e] - 1;
+        lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    }
+    int n_chunks = pos / chunk - lo / chunk + 1;
+    const float* mine = pp + 2 + 2 * f;           // 8-byte aligned: rows of hd + 2 floats, hd even
+    float2 ahead[AHEAD];
+#pragma unroll
+    for (int c = 0; c < AHEAD; ++c) {
+        int ch = g + c * groups;
+        ahead[c] = (adds && ch < n_chunks) ? *reinterpret_cast<const float2*>(mine + (size_t)ch * stride) : make_float2(0.0f, 0.0f);
+    }
+    float M = -INFINITY, L = 0.0f;
+    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * stride]);
+    M = wave_max(M);
+    for (int ch = lane; ch < n_chunks; ch += 64) {
+        float w = __builtin_amdgcn_exp2f(pp[(size_t)ch * stride] - M);      // the maxima are base-2 logarithms
+        if (wave == 0) weight[ch] = w;
+        L += pp[(size_t)ch * stride + 1] * w;
+    }
+    L = wave_sum(L);
+    __syncthreads();
+    if (adds) {
+        float ox = 0.0f, oy = 0.0f;
+#pragma unroll
+        for (int c = 0; c < AHEAD; ++c) {
+            int ch = g + c * groups;
+            if (ch < n_chunks) { float w = weight[ch]; ox = fmaf(ahead[c].x, w, ox); oy = fmaf(ahead[c].y, w, oy); }
+        }
+        for (int base = g + AHEAD * groups; base < n_chunks; base += AHEAD * groups) {
+            float2 v[AHEAD];
+#pragma unroll
+            for (int c = 0; c < AHEAD; ++c) {
+                int ch = base + c * groups;
+                v[c] = ch < n_chunks ? *reinterpret_cast<const float2*>(mine + (size_t)ch * stride) : make_float2(0.0f, 0.0f);
+            }
+#pragma unroll
+            for (int c = 0; c < AHEAD; ++c) {
+                int ch = base + c * groups;
+                if (ch < n_chunks) { float w = weight[ch]; ox = fmaf(v[c].x, w, ox); oy = fmaf(v[c].y, w, oy); }
+            }
+        }
+        sums[g * hd + 2 * f] = ox;
+        sums[g * hd + 2 * f + 1] = oy;
+    }
+    __syncthreads();
+    if (tid < hd) {
+        float o = 0.0f;
+        for (int k = 0; k < groups; ++k) o += sums[k * hd + tid];
+        out[(size_t)token * a.out_stride + (size_t)head * hd + tid] = (bf16)(o / L);
+    }
+}
+
 // A step with a prompt portion beside decoding requests has two kinds of attention work that do not depend on
 // each other: tiles of many tokens, bound by the matrix cores, and single tokens over their whole caches, bound by
 // memory.  They run side by side: the single tokens' kernels go to a second stream of this library's own (default
@@ -661,14 +744,14 @@ static SideStream* side_stream() {
 // length.  ATTN_CHUNK, doubled while the waves would still fill the device's places (a wave begins with a chain of
 // trips to memory: lengths, page numbers, then keys; with many requests, longer ranges make that a smaller part of
 // its life; measured, 8B shapes at 2048 keys: 64 requests 6945 -> 7540 tokens/s, 256 requests 11960 -> 12740);
-// halved when even then there is no more than a wave per SIMD and the chunks stay few enough for the merge to
-// take in one go: with so few requests a wave's life is its chain of trips, one per 32 keys, and nothing else
-// competes for memory.
+// halved when even then there is no more than a wave per SIMD (and the chunks stay a quarter of what the merge
+// takes): with so few requests a wave's life is its chain of trips, one per 32 keys, and nothing else competes
+// for memory.
 int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max_seq_len) {
     long cus = llmrs_compute_units();
     auto waves = [&](int c) { return singles * n_kv_heads * ((3L * max_seq_len / 4 + c - 1) / c); };
     int chunk = ATTN_CHUNK;
-    if (waves(ATTN_CHUNK / 2) <= cus * 4 && max_seq_len <= 64 * (ATTN_CHUNK / 2)) return ATTN_CHUNK / 2;
+    if (waves(ATTN_CHUNK / 2) <= cus * 4 && max_seq_len <= (MERGE_MAX_CHUNKS / 4) * (ATTN_CHUNK / 2)) return ATTN_CHUNK / 2;
     while (chunk < 8 * ATTN_CHUNK && waves(chunk * 2) >= cus * 8) chunk *= 2;
     return chunk;
 }
@@ -713,7 +796,13 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
         int plain = only_single && a.window == 0;
         attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk, plain);
-        attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64 * ((HD + 63) / 64), 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk, plain);
+        if (max_chunks > MERGE_ONE_WALK_CHUNKS && HD <= MERGE_GROUP_THREADS) {
+            int threads = (HD / 2) * ((max_chunks + 3) / 4);          // groups of HD / 2 threads, a group for every four chunks
+            threads = std::min(MERGE_GROUP_THREADS, std::max(HD, (threads + 63) / 64 * 64));
+            attn_merge_groups_kernel<<<dim3(n_entries, a.n_heads), threads, 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk, plain);
+        }
+        else
+            attn_merge_kernel<<<dim3(n_entries, a.n_heads), 64 * ((HD + 63) / 64), 0, single_stream>>>(scratch, out, seq_lens, q_starts, a, max_chunks, chunk, plain);
     }
     if (side != nullptr && single_stream != stream) {
         // the caller's stream goes on only when the second stream's kernels are done (they write other rows of `out`)

@@ -260,6 +260,15 @@ class PagedCase:
         outs = []
         for i, p in enumerate(positions):
             n = p + 1
+            if n > 6000:        # the one row of the same formula: the table of all rows' scores would take gigabytes
+                G = self.n_heads // self.n_kv
+                sc = 1.0 / math.sqrt(self.hd) if scale is None else scale
+                s = torch.einsum("hd,nhd->hn", q[i].double(), self.k[r][:n].double().repeat_interleave(G, dim=1)) * sc
+                if window and n > window:
+                    s[:, :n - window] = -math.inf
+                w = torch.softmax(s, dim=-1)
+                outs.append(torch.einsum("hn,nhd->hd", w, self.v[r][:n].double().repeat_interleave(G, dim=1)))
+                continue
             qq = torch.zeros((n, self.n_heads, self.hd), dtype=torch.float64)
             qq[-1] = q[i].double()
             o = plain_attention(qq, self.k[r][:n].double(), self.v[r][:n].double(), scale, window)
@@ -294,13 +303,17 @@ def test_attention_mixed_batch(dtype, n_heads, n_kv, hd, ps):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hd,ps,n", [(64, 16, 700), (128, 16, 1500), (32, 4, 300),
-                                     (128, 16, 2300), (64, 16, 5000)])    # more than 16 ranges of 128 keys to merge: the merge kernel's later groups
+                                     (128, 16, 2300), (64, 16, 5000),    # more than 16 ranges of 128 keys to merge: the merge kernel's later groups
+                                     (128, 16, 8300), (64, 16, 17000), (96, 16, 9000)])   # more than 64 ranges: the merge whose threads share them out
 def test_attention_finds_a_far_key(dtype, hd, ps, n):
     """Random keys hide a key that is skipped or read from the wrong page: here one
     early key matches the query so strongly that the output must be its value."""
     n_heads, n_kv = 4, 2
     case = PagedCase(dtype, [n], n_heads, n_kv, hd, ps, seed=3)
-    for far in (0, ps - 1, ps, 63, 64, n // 2 + 1, n - 2) + ((2053, n - 300) if n > 2100 else ()):    # (one request alone: ranges of 64 keys)
+    fars = (0, ps - 1, ps, 63, 64, n // 2 + 1, n - 2) + ((2053, n - 300) if n > 2100 else ())    # (one request alone: ranges of 64 keys)
+    if n > 8192:        # one key in each of the last ranges of 128, and in ranges that different groups of the merge's threads take
+        fars = fars + tuple(n - 1 - 128 * i - 7 * i for i in range(1, 20)) + (129, 1024 + 5, 4096 - 1, 4096, 8191)
+    for far in fars:
         q = torch.zeros((1, n_heads, hd))
         q[0, :, :] = case.k[0][far, :, :].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0
         got = case.run([q.to(dtype)], [[n - 1]])
@@ -309,6 +322,33 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (ref[0].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
         tol = 1e-4 if dtype == torch.float32 else 2e-2
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
+
+
+@pytest.mark.parametrize("portion", [False, True])
+def test_attention_long_caches_with_a_window(portion):
+    """Two decoding requests over long caches with a window of 8500 keys (more than 64 ranges to merge, the first of
+    them cut by the window's edge), with and without a prompt portion beside them: a key just inside the window is
+    found, one just outside it is not seen."""
+    n_heads, n_kv, hd, ps, window = 8, 2, 128, 16, 8500
+    lens = [12000, 9100] + ([40] if portion else [])
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=29)
+    g = torch.Generator().manual_seed(5)
+    for inside in (True, False):
+        qs, pos, fars = [], [], []
+        for r, n in enumerate(lens[:2]):
+            far = n - window + (0 if inside else -1)
+            fars.append(far)
+            qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16))
+            pos.append([n - 1])
+        if portion:
+            qs.append(torch.randn((40, n_heads, hd), generator=g).to(torch.bfloat16))
+            pos.append(list(range(40)))
+        got = case.run(qs, pos, window=window)
+        for r in range(2):
+            want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
+            ref = case.reference(r, qs[r], pos[r], window=window)[0].float()
+            assert ((ref - want).abs().max() < 0.05) == inside, "the case itself"
+            assert (got[r].float() - ref).abs().max() <= 2e-2, f"request of length {lens[r]}, key {fars[r]}"
 
 
 @pytest.mark.parametrize("window", [0, 300])
