@@ -326,7 +326,7 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
 extern "C" long llmrs_attention_scratch_floats(int n_entries, int singles, int n_heads, int n_kv_heads, int head_dim,
                                                int max_seq_len) {
     if (max_seq_len <= 0 || n_entries <= 0 || n_heads <= 0 || n_kv_heads <= 0) return 0;
-    int chunk = min(GENERIC_CHUNK, llmrs_attention_split_chunk(singles > 0 ? singles : n_entries, n_kv_heads, max_seq_len));
+    int chunk = min(GENERIC_CHUNK, llmrs_attention_split_chunk(singles > 0 ? singles : n_entries, n_kv_heads, max_seq_len, 1));
     return (long)n_entries * n_heads * ceil_div(max_seq_len, chunk) * (head_dim + 2);
 }
 
@@ -405,13 +405,16 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // scratch: device memory for the partial results of single-token entries, which
 // are split over waves by key range (may be null: then they are not split);
 // max_seq_len: an upper bound of seq_lens that the host knows (0: unknown, no split);
-// n_single: how many entries bring one token, if the host knows (-1: it does not).
+// n_single: how many entries bring one token, if the host knows (-1: it does not);
+// single_keys: how many keys those entries see together (windows counted), if the host knows (0: it does not):
+// the matrix-core kernels choose the keys per wave by it.
 extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
                                const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                                const int* token_entry, const int* positions, const int* q_starts,
                                const int* seq_lens, int n_entries, int n_tokens, int n_heads, int n_kv_heads,
                                int head_dim, int page_size, int num_pages, int window, float scale,
-                               void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, int allow_mfma) {
+                               void* scratch, size_t scratch_bytes, int max_seq_len, int n_single, long single_keys,
+                               int allow_mfma) {
     LLMRS_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0, "attention: bad sizes");
     LLMRS_REQUIRE(n_heads % n_kv_heads == 0, "attention: %d heads are no multiple of %d kv heads", n_heads, n_kv_heads);
     LLMRS_REQUIRE(head_dim <= MAX_HEAD_DIM, "attention: head_dim %d exceeds %d", head_dim, MAX_HEAD_DIM);
@@ -424,7 +427,7 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     if (dtype == LLMRS_BF16 && allow_mfma) {
         int took = llmrs_attention_bf16_mfma(stream, (const bf16*)q, (bf16*)out, (const bf16*)k_cache, (const bf16*)v_cache,
                                              block_table, token_entry, positions, q_starts, seq_lens, n_entries,
-                                             (float*)scratch, scratch_bytes, max_seq_len, n_single, a);
+                                             (float*)scratch, scratch_bytes, max_seq_len, n_single, single_keys, a);
         if (took != 0) return took < 0 ? -1 : 0;
     }
     int rc = 0;

@@ -254,7 +254,7 @@ extern "C" int llmrs_plain_attention(void*, int dtype, const void* q, int q_stri
                                      const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                                      const int* token_entry, const int* positions, const int*, const int*, int n_entries,
                                      int n_tokens, int n_heads, int n_kv_heads, int head_dim, int page_size, int num_pages,
-                                     int window, float scale, void*, size_t, int, int, int) {
+                                     int window, float scale, void*, size_t, int, int, long, int) {
     if (!known(dtype) || n_kv_heads <= 0 || n_heads % n_kv_heads || head_dim <= 0 || page_size <= 0) return -1;
     int group = n_heads / n_kv_heads;
     std::vector<double> score, acc(head_dim);

@@ -24,6 +24,12 @@ class Model:
         self.final_norm = build_norm(spec.final_norm, dtype)
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
+        keyed = {}
+        for block in self.blocks:
+            for part in block.parts():
+                if part.recording_signature is not None:
+                    keyed.setdefault(part.recording_signature, part)
+        self._keyed_parts = list(keyed.values())
 
     # -- weights -------------------------------------------------------------
     def tensors(self) -> Dict[str, TensorSpec]:
@@ -89,6 +95,10 @@ class Model:
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph (every part says so)."""
         return all(part.graph_safe for block in self.blocks for part in block.parts()) and self.final_norm.graph_safe
+
+    def recording_key(self, ctx) -> tuple:
+        """What a recording of this step depends on beyond its sizes (its parts say)."""
+        return tuple(part.recording_key(ctx) for part in self._keyed_parts)
 
     # -- cache ---------------------------------------------------------------
     def cache_needs(self) -> List[Tuple[object, Optional[int]]]:

@@ -67,6 +67,8 @@ class StepContext:
         self.entries: List[Tuple[int, int, int]] = []   # host copy: (slot, start, count)
         self.max_seq_len = 0                            # largest start + count among the entries
         self.n_single = 0                               # entries that bring one token
+        self.single_lens: List[int] = []                # their lengths with that token
+        self._keys_seen = {}
         self.device = runner.device
         # A norm without a kernel of its own (steps of a few tokens): the part that adds into the stream last
         # before a norm leaves what that norm needs (`room_for_next_norm`, `note_left`), and the norm hands it on
@@ -80,6 +82,14 @@ class StepContext:
 
     def workspace(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         return self._runner.workspace(name, shape, dtype)
+
+    def single_keys(self, window: int = 0) -> int:
+        """How many keys the single-token entries see together, each through a window of `window` keys (0: all)."""
+        got = self._keys_seen.get(window)
+        if got is None:
+            got = sum(self.single_lens) if window <= 0 else sum(min(n, window) for n in self.single_lens)
+            self._keys_seen[window] = got
+        return got
 
     def room_for_next_norm(self, h: torch.Tensor, w: torch.Tensor):
         """For a part about to add a product with weight `w` into the stream `h`: a `kernels.NextNorm` for that
@@ -232,7 +242,9 @@ class StepRunner:
         c.n_tokens, c.n_entries, c.n_want = T, R, n_want
         c.entries = entries
         c.max_seq_len = max(start + count for _, start, count in entries)
-        c.n_single = sum(1 for _, _, count in entries if count == 1)
+        c.single_lens = [start + 1 for _, start, count in entries if count == 1]
+        c.n_single = len(c.single_lens)
+        c._keys_seen = {}
         c.tokens = dev[off.tokens:off.tokens + T]
         c.positions = dev[off.positions:off.positions + T]
         c.token_entry = dev[off.token_entry:off.token_entry + T]
@@ -308,7 +320,7 @@ class StepRunner:
         # A decode step.  Everything the kernels take from the host must be the same for
         # every step of this key: sizes, addresses, and the bound on the context length.
         ctx.max_seq_len = min(w * g.page_size for w, g in zip(graph_widths, self.cache.groups)) if graph_widths else ctx.max_seq_len
-        key = (ctx.n_tokens, ctx.n_want, tuple(graph_widths), self._dev_words.data_ptr())
+        key = (ctx.n_tokens, ctx.n_want, tuple(graph_widths), self._dev_words.data_ptr(), self.model.recording_key(ctx))
         hit = self._graphs.get(key)
         if hit is not None:
             self._graphs.move_to_end(key)

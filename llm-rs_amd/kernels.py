@@ -143,7 +143,7 @@ class HipKernels:
             "llmrs_gemm_norms_whole": [I, I, I],
             "llmrs_gemm_next_parts": [I, I, I],
             "llmrs_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
-            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, I],
+            "llmrs_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, c_size_t, I, I, ctypes.c_long, I],
             "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I, V, I, F],
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
@@ -165,6 +165,8 @@ class HipKernels:
         self.times: Optional[KernelTimes] = KernelTimes() if os.environ.get("LLM_PERF") else None
         lib.llmrs_attention_scratch_floats.restype = ctypes.c_long
         lib.llmrs_attention_scratch_floats.argtypes = [I, I, I, I, I, I]
+        lib.llmrs_attention_split_chunk.restype = I
+        lib.llmrs_attention_split_chunk.argtypes = [ctypes.c_long, I, I, ctypes.c_long]
         lib.llmrs_gemm_workspace_floats.restype = ctypes.c_long
         lib.llmrs_gemm_workspace_floats.argtypes = [I, I, I]
 
@@ -326,8 +328,16 @@ class HipKernels:
                   None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
                   0.0 if scale is None else scale.eps)
 
+    def attention_split_chunk(self, n_single: int, n_kv_heads: int, max_seq_len: int, single_keys: int = 0) -> int:
+        """Keys per wave that a call with these figures splits its single-token entries by: what a caller that
+        records steps into graphs has to key its recordings by, since a recording holds the chunk it was made with
+        while the number of keys moves with every step."""
+        return int(self.lib.llmrs_attention_split_chunk(int(n_single), int(n_kv_heads), int(max_seq_len), int(single_keys)))
+
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1) -> None:
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
+                  single_keys=0) -> None:
+        """single_keys: how many keys the single-token entries see together (windows counted), 0 if unknown."""
         assert q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
         assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
         assert k_cache.numel() == num_pages * n_kv_heads * page_size * head_dim == v_cache.numel()
@@ -345,7 +355,7 @@ class HipKernels:
                   _p(block_table), block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens),
                   block_table.shape[0], T, n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale,
                   _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size(), int(max_seq_len),
-                  int(n_single), int(self.allow_mfma))
+                  int(n_single), int(single_keys), int(self.allow_mfma))
 
     def argmax_rows(self, logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> None:
         """`scratch`: 256 bytes per row let several blocks share a long row."""

@@ -39,6 +39,7 @@ class Attention(Mixer):
         self.kv_heads = int(p["num_kv_heads"])
         self.head_dim = int(p["head_dim"])
         self.window = int(p.get("window") or 0)
+        self.recording_signature = ("attention", self.kv_heads, self.window)
         self.kv_proj = bool(p.get("kv_proj", True))
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
@@ -102,6 +103,13 @@ class Attention(Mixer):
         return (fused and self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
                 and k.gemm_defers_norm(rows, self.w_qkv.shape[0], self.hidden))
 
+    def recording_key(self, ctx):
+        # the keys per wave that the kernel library splits the decoding requests' caches by
+        k = kernels()
+        if not ctx.n_single or not hasattr(k, "attention_split_chunk"):
+            return 0
+        return k.attention_split_chunk(ctx.n_single, self.kv_heads, ctx.max_seq_len, ctx.single_keys(self.window))
+
     def forward(self, ctx, x, h, cache):
         k = kernels()
         T = x.shape[0]
@@ -129,7 +137,8 @@ class Attention(Mixer):
         scratch = ctx.workspace("attn.partial", (need,), torch.float32) if need else None
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
-                    cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single)
+                    cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single,
+                    ctx.single_keys(self.window) if ctx.n_single else 0)
         leave = ctx.room_for_next_norm(h, self.w_o)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o), **({} if leave is None else {"leave": leave}))
         ctx.note_left(h, leave)

@@ -46,6 +46,14 @@ class Part:
     # recorded into a HIP graph.  A part that looks at host values of the step, allocates, or
     # copies between host and device must leave this False; the model is then never recorded.
     graph_safe = False
+    # A part whose kernels take something from the host that moves from step to step though the step's sizes stay
+    # (a launch shape chosen by how many keys the step sees, say) names here what that choice depends on, any
+    # hashable value (parts with equal values are asked once), and says in `recording_key` what it comes to for a
+    # step: a recorded step is replayed only for steps with the same key.  None: nothing of the kind.
+    recording_signature = None
+
+    def recording_key(self, ctx):
+        return ()
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         self.spec = spec

@@ -110,7 +110,8 @@ class EmulatedKernels:
                            n_heads, n_kv_heads, head_dim, page_size, num_pages, write_kv)
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
-                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1):
+                  n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,
+                  single_keys=0):
         T = q.shape[0]
         kc = k_cache.view(num_pages, n_kv_heads, page_size, head_dim).float()
         vc = v_cache.view(num_pages, n_kv_heads, head_dim, page_size).float()

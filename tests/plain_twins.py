@@ -31,7 +31,7 @@ class PlainTwins:
             "llmrs_plain_gemm": [V, I, V, I, V, V, I, I, I, I, I, V, S, I, V, I, F, V, V, I, V, F],
             "llmrs_plain_rope_kv_write": [V, I, V, I, V, V, V, I, I, V, V, I, I, I, I, I, I, I],
             "llmrs_plain_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, S, I, V, I, F],
-            "llmrs_plain_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, S, I, I, I],
+            "llmrs_plain_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, S, I, I, ctypes.c_long, I],
             "llmrs_plain_argmax_rows": [V, V, I, I, I, V, V, S],
             "llmrs_plain_sample_rows": [V, V, I, I, I, V, V, V],
             "llmrs_plain_cast": [V, V, I, V, I, S],
@@ -91,11 +91,11 @@ class PlainTwins:
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0,
-                  n_single=-1) -> None:
+                  n_single=-1, single_keys=0) -> None:
         self._check(self.lib.llmrs_plain_attention(
             None, _CODE[q.dtype], _p(q), q.stride(0), _p(out), out.stride(0), _p(k_cache), _p(v_cache), _p(block_table),
             block_table.shape[1], _p(token_entry), _p(positions), _p(q_starts), _p(seq_lens), block_table.shape[0],
-            q.shape[0], n_heads, n_kv_heads, head_dim, page_size, num_pages, window, float(scale), None, 0, 0, 0, 0),
+            q.shape[0], n_heads, n_kv_heads, head_dim, page_size, num_pages, window, float(scale), None, 0, 0, 0, 0, 0),
             "attention")
 
     def argmax_rows(self, logits, out, scratch=None) -> None:

@@ -238,7 +238,7 @@ class PagedCase:
                 self.kc[page, :, :hi - lo, :] = self.k[r][lo:hi].permute(1, 0, 2)
                 self.vc[page, :, :, :hi - lo] = self.v[r][lo:hi].permute(1, 2, 0)
 
-    def run(self, q_list, q_pos_list, window=0, scale=None):
+    def run(self, q_list, q_pos_list, window=0, scale=None, scratch_floats=1 << 22, bound=None, n_single=-1, single_keys=0):
         """q_list[r]: [n_r, heads, hd] queries of request r at positions q_pos_list[r]."""
         scale = 1.0 / math.sqrt(self.hd) if scale is None else scale
         q = torch.cat(q_list).reshape(-1, self.n_heads * self.hd).to(DEV)
@@ -249,10 +249,10 @@ class PagedCase:
         q_starts = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
         seq_lens = torch.tensor([max(p) + 1 for p in q_pos_list], dtype=torch.int32, device=DEV)
         out = torch.zeros((T, self.n_heads * self.hd), dtype=self.dtype, device=DEV)
-        scratch = torch.empty(1 << 22, dtype=torch.float32, device=DEV)
+        scratch = torch.empty(scratch_floats, dtype=torch.float32, device=DEV)
         kernels().attention(q, out, self.kc.to(DEV), self.vc.to(DEV), self.tables.to(DEV), entry, pos, q_starts, seq_lens,
                             self.n_heads, self.n_kv, self.hd, self.ps, self.num_pages, window, scale, scratch,
-                            max(max(p) + 1 for p in q_pos_list))
+                            max(max(p) + 1 for p in q_pos_list) if bound is None else bound, n_single, single_keys)
         return out.cpu().view(T, self.n_heads, self.hd)
 
     def reference(self, r, q, positions, window=0, scale=None):
@@ -322,6 +322,36 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (ref[0].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
         tol = 1e-4 if dtype == torch.float32 else 2e-2
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
+
+
+def test_attention_chunk_rule_and_its_scratch():
+    """The keys per wave that the split takes: a power of two from 64 to 1024 whatever the host says about the
+    keys; never under what the scratch is sized by (the answer for one key); and the same results whichever chunk
+    the number of keys leads to, with a scratch of exactly the size the library asks for."""
+    k = kernels()
+    for n, kv, bound in ((1, 8, 2048), (8, 8, 2048), (12, 2, 4096), (64, 8, 2048), (200, 4, 8192), (1, 1, 131072), (3, 8, 40000)):
+        least = k.attention_split_chunk(n, kv, bound, 1)
+        for keys in (0, 1, n * bound // 16, n * bound // 3, n * bound, 10 * n * bound):
+            c = k.attention_split_chunk(n, kv, bound, keys)
+            assert c in (64, 128, 256, 512, 1024) and c >= least, (n, kv, bound, keys, c, least)
+            assert -(-bound // c) <= 256 or c == 1024
+    n_heads, n_kv, hd, ps = 8, 8, 64, 16
+    lens = [1500, 700, 1290, 40, 2047, 900, 1100, 333, 1999, 1203]
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=41)
+    g = torch.Generator().manual_seed(3)
+    qs = [torch.randn((1, n_heads, hd), generator=g).to(torch.bfloat16) for _ in lens]
+    pos = [[n - 1] for n in lens]
+    refs = [case.reference(r, qs[r], pos[r])[0].float() for r in range(len(lens))]
+    seen = set()
+    for keys in (0, 1, sum(lens), 40 * sum(lens), 400 * sum(lens)):
+        c = k.attention_split_chunk(len(lens), n_kv, 2048, keys)
+        seen.add(c)
+        need = k.attention_scratch_floats(len(lens), n_heads, hd, 2048, n_kv, len(lens))
+        assert need >= len(lens) * n_heads * -(-2048 // c) * (hd + 2)
+        got = case.run(qs, pos, scratch_floats=need, bound=2048, n_single=len(lens), single_keys=keys)
+        for r in range(len(lens)):
+            assert (got[r].float() - refs[r]).abs().max() <= 2e-2, f"{keys} keys, request {r}"
+    assert len(seen) >= 2, "the case itself: more than one chunk"
 
 
 @pytest.mark.parametrize("portion", [False, True])
