@@ -1381,7 +1381,11 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
         int rot = wide ? 16 * wide_nt : (K >= 8192 ? 64 : 0);
 #define SKINNY(MT, NT, NW, U) launch_skinny<MT, NT, NW, U>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot, scale, next)
         if (M <= 16) {
-            if (wide) { if (M <= 2) SKINNY(1, 1, 4, 8); else if (wide_nt == 7) SKINNY(1, 7, 4, 1); else SKINNY(1, 4, 4, 2); }
+            if (wide) {
+                // up to 4 rows blocks of 16 features (a decode step of eight 8B layers: 1.100 -> 1.086 ms at 3 rows,
+                // 1.121 -> 1.116 at 4, slower from 6 on: every block reads the tokens' rows again)
+                if (M <= 4) SKINNY(1, 1, 4, 8); else if (wide_nt == 7) SKINNY(1, 7, 4, 1); else SKINNY(1, 4, 4, 2);
+            }
             else if (eight) {
                 // Blocks of 16 features, unless they come to a round and a half of the device's units (6144 features on
                 // 256: 384 blocks) and blocks of 24 to whole rounds: those, when nothing is to be left for a norm (which
@@ -1407,20 +1411,24 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             }
             else { if (eight) SKINNY(2, 1, 8, 4); else SKINNY(2, 1, 4, 4); }
         } else {
-            // 64 x 64 outputs per block; when that leaves no more than 64 blocks, K is split
+            // 48 or 64 tokens and 64 features per block; when that leaves no more than 64 blocks, K is split
             // over blocks too, if the caller gave room for the partial sums (measured: it
             // pays for N = 4096, K = 14336, and no longer for N = 6144).
-            int splits = skinny_splits(N, K);
-            if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
-                workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
-                launch_skinny<4, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace, 0, nullptr, next);
-            } else if (wide) { if (wide_nt == 7) SKINNY(4, 7, 4, 1); else SKINNY(4, 4, 4, 2); }
-            else if (N > 4096) {
-                if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<4, 2, 8, 1, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
-                else if (eight) SKINNY(4, 2, 8, 1);
-                else SKINNY(4, 2, 4, 2);
-            }
-            else { if (eight) SKINNY(4, 1, 8, 2); else SKINNY(4, 1, 4, 2); }
+            auto rows_of = [&](auto tiles) {
+                constexpr int MT = decltype(tiles)::value;
+                int splits = skinny_splits(N, K);
+                if (splits > 1 && epi != LLMRS_EPI_QKV && workspace != nullptr &&
+                    workspace_bytes >= (size_t)splits * M * N * sizeof(float)) {
+                    launch_skinny<MT, 4, 8, 1>(stream, A, lda, W, out, ldc, M, N, K, epi, nullptr, splits, (float*)workspace, 0, nullptr, next);
+                } else if (wide) { if (wide_nt == 7) SKINNY(MT, 7, 4, 1); else SKINNY(MT, 4, 4, 2); }
+                else if (N > 4096) {
+                    if (eight && half_tile_blocks(N, 32, cus)) launch_skinny<MT, 2, 8, 1, 8>(stream, A, lda, W, out, ldc, M, N, K, epi, qkv, 1, nullptr, rot);
+                    else if (eight) SKINNY(MT, 2, 8, 1);
+                    else SKINNY(MT, 2, 4, 2);
+                }
+                else { if (eight) SKINNY(MT, 1, 8, 2); else SKINNY(MT, 1, 4, 2); }
+            };
+            if (M <= 48) rows_of(std::integral_constant<int, 3>{}); else rows_of(std::integral_constant<int, 4>{});
         }
 #undef SKINNY
     } else {

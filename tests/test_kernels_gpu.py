@@ -55,6 +55,8 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20),
                (64, 200, 2048), (40, 1000, 1096), (64, 4096, 4096), (24, 520, 2048), (50, 64, 8200),
                (8, 38, 100), (3, 130, 4099), (1, 6, 20),
+               # 33 to 48 rows: blocks of three row tiles, in each of the few-row kernel's shapes
+               (48, 4096, 4096), (36, 16400, 264), (47, 6144, 2048), (34, 2048, 2048), (41, 300, 136),
                # 256 x 192 tiles where they make whole rounds of the device and square ones do not; the last tile cut by N
                (2048, 6144, 128), (2048, 6100, 192), (1800, 6144, 64),
                # a round and a half of 16-feature blocks: blocks of 24 features (a tile and a half), the last one cut by N
@@ -901,7 +903,7 @@ def test_a_norm_left_by_one_product_and_finished_by_the_next(M, hidden, inter):
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 4096, 4096), (17, 4096, 14336), (24, 1024, 2048), (33, 2048, 8192), (200, 512, 4096),
-                                   (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192)])
+                                   (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192), (45, 4096, 4096)])
 def test_split_residual_product_finishes_the_next_norm(M, N, K):
     """17 to 256 rows, a product whose sums are split over blocks: the kernel that adds the parts writes the stream and
     the normed rows: the stream bit for bit as without, the rows as the norm kernel makes them from that stream."""
