@@ -20,7 +20,7 @@ int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, cons
 // Keys per wave when the matrix-core kernels split `singles` single-token entries of up to max_seq_len keys
 // that see single_keys keys together (0: unknown; 1 gives the smallest chunk any number of keys can give for these
 // entries and this bound, which is what the scratch is sized by).
-extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max_seq_len, long single_keys);
+extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int head_dim, int max_seq_len, long single_keys);
 
 // 32-bit tiles on the matrix cores for entries with several tokens (attention_f32_mfma.hip); skip_single: entries
 // with one token are left to the caller.  Return 1 when it took them, 0 when the shape is not its own, -1 on error.

@@ -326,7 +326,7 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
 extern "C" long llmrs_attention_scratch_floats(int n_entries, int singles, int n_heads, int n_kv_heads, int head_dim,
                                                int max_seq_len) {
     if (max_seq_len <= 0 || n_entries <= 0 || n_heads <= 0 || n_kv_heads <= 0) return 0;
-    int chunk = min(GENERIC_CHUNK, llmrs_attention_split_chunk(singles > 0 ? singles : n_entries, n_kv_heads, max_seq_len, 1));
+    int chunk = min(GENERIC_CHUNK, llmrs_attention_split_chunk(singles > 0 ? singles : n_entries, n_kv_heads, head_dim, max_seq_len, 1));
     return (long)n_entries * n_heads * ceil_div(max_seq_len, chunk) * (head_dim + 2);
 }
 

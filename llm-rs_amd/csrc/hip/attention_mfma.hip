@@ -742,24 +742,51 @@ static SideStream* side_stream() {
     return s.stream != nullptr ? &s : nullptr;
 }
 
+// How many waves of the split a compute unit holds at once: what the registers of the kernel for this head size
+// allow (two to a SIMD at head size 128, three at 64), asked of the runtime once per head size.  Head sizes
+// without a kernel here: 8.
+static int split_waves_to_a_unit(int head_dim) {
+    static int known[8] = {0, 0, 0, 0, 0, 0, 0, 0};      // by head_dim / 32 - 1
+    static std::mutex mutex;
+    if (head_dim % 32 || head_dim < 32 || head_dim > 256) return 8;
+    std::lock_guard<std::mutex> lock(mutex);
+    int& n = known[head_dim / 32 - 1];
+    if (n == 0) {
+        int blocks = 0;
+        hipError_t e = hipErrorInvalidValue;
+        switch (head_dim) {
+#define ASK(HD) case HD: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_split_kernel<HD>, 64, 0); break;
+            ASK(32) ASK(64) ASK(96) ASK(128) ASK(192) ASK(256)
+#undef ASK
+            default: break;
+        }
+        if (e != hipSuccess) (void)hipGetLastError();
+        n = (e == hipSuccess && blocks >= 1) ? std::min(blocks, 32) : 8;
+    }
+    return n;
+}
+
 // Keys per wave of the split, by what the host knows: the number of single-token entries, the bound on their
 // length, and (when it says so) how many keys they see together.  Measured on the 8B head shape (8 to 256 requests
-// of 520 to 4090 keys, every chunk from 64 to 1024 keys): a compute unit works through these waves eight at a
-// time.  Up to eight to a unit, all of the same length, end together, and the longest chunks that still give every
-// SIMD a wave are the fastest (a wave begins with a chain of trips to memory: lengths, page numbers, then keys);
-// a ninth wave on a unit costs a second turn.  So: the smallest chunk that gives fewer than eight waves to a unit;
-// and when even chunks of 1024 keys give more, 512 if the last turn of eight would be far from full (many short
-// waves share out evenly as they come).  Against the best chunk of each case (also at sizes and lengths between
-// those it was made from) this rule loses 0.7 % on average and 9 % at worst; the rule before it (128 keys, doubled
-// while the waves kept all units busy, by the bound alone) lost 7.5 % and 19 %.  The chunks of a request are never more than a quarter of what the merge takes.
+// of 520 to 8000 keys, every chunk from 64 to 1024 keys) and on the 1B one: a compute unit holds so many of these
+// waves at once (eight at head size 128, twelve at 64) and works through them in turns of that many.  Waves of one
+// turn, all of the same length, end together, and the longest chunks that still fill half a turn are the fastest
+// (a wave begins with a chain of trips to memory: lengths, page numbers, then keys); one wave more than a turn
+// costs a second turn.  So: the smallest chunk that gives a unit less than a turn; and when even chunks of 1024
+// keys give more, 512 if the last turn would be far from full (many short waves share out evenly as they come).
+// Against the best chunk of each case (also at sizes and lengths between those it was made from) this rule loses
+// 0.7 % on average and 9 % at worst at head size 128, 1 % and 14 % at 64; the rule before it (128 keys, doubled
+// while the waves kept all units busy, by the bound alone) lost 7.5 % and 19 %.  The chunks of a request are never
+// more than a quarter of what the merge takes.
 // The number of keys moves with every step while a recorded graph holds the chunk it was recorded with: callers that
 // record put this function's result into what they key their recordings by.  The scratch is sized by the smallest
 // chunk the entries and the bound allow, taken at an eighth of the bound for every entry; fewer keys than that get
 // that chunk too.
-extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max_seq_len, long single_keys) {
+extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int head_dim, int max_seq_len, long single_keys) {
     double cus = (double)llmrs_compute_units();
     if (singles < 1) singles = 1;
     if (max_seq_len < 1) max_seq_len = 1;
+    const double turn = split_waves_to_a_unit(head_dim);
     const int longest = 8 * ATTN_CHUNK;
     auto pick = [&](double keys) {
         // waves to a compute unit with chunks of c keys, every entry taken at the mean length; the last chunk of a
@@ -769,10 +796,10 @@ extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int max
             return singles * n_kv_heads * (whole + (rest > 0.125 ? 1.0 : rest)) / cus;
         };
         int c = ATTN_CHUNK / 2;
-        while (c < longest && to_a_unit(c) >= 8.0) c *= 2;
-        if (c == longest && to_a_unit(c) > 8.0) {
-            double last = fmod(to_a_unit(c), 8.0);
-            if (last > 0.05 && last < 5.5) c /= 2;
+        while (c < longest && to_a_unit(c) >= turn) c *= 2;
+        if (c == longest && to_a_unit(c) > turn) {
+            double last = fmod(to_a_unit(c), turn) / turn;
+            if (last > 0.006 && last < 0.69) c /= 2;
         }
         while (c < longest && (max_seq_len + c - 1) / c > MERGE_MAX_CHUNKS / 4) c *= 2;
         return c;
@@ -789,7 +816,7 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
                   size_t scratch_bytes, int max_seq_len, int n_single, long single_keys, const AttnArgs& a) {
     int G = a.n_heads / a.n_kv_heads;
     int tpt = 32 / G;
-    int chunk = llmrs_attention_split_chunk(n_single > 0 ? n_single : n_entries, a.n_kv_heads, max_seq_len, single_keys);
+    int chunk = llmrs_attention_split_chunk(n_single > 0 ? n_single : n_entries, a.n_kv_heads, HD, max_seq_len, single_keys);
     int max_chunks = max_seq_len > 0 ? (max_seq_len + chunk - 1) / chunk : 0;
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.

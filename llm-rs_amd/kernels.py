@@ -166,7 +166,7 @@ class HipKernels:
         lib.llmrs_attention_scratch_floats.restype = ctypes.c_long
         lib.llmrs_attention_scratch_floats.argtypes = [I, I, I, I, I, I]
         lib.llmrs_attention_split_chunk.restype = I
-        lib.llmrs_attention_split_chunk.argtypes = [ctypes.c_long, I, I, ctypes.c_long]
+        lib.llmrs_attention_split_chunk.argtypes = [ctypes.c_long, I, I, I, ctypes.c_long]
         lib.llmrs_gemm_workspace_floats.restype = ctypes.c_long
         lib.llmrs_gemm_workspace_floats.argtypes = [I, I, I]
 
@@ -328,11 +328,11 @@ class HipKernels:
                   None if scale is None else _p(scale.sumsq), 0 if scale is None else scale.sumsq.shape[1],
                   0.0 if scale is None else scale.eps)
 
-    def attention_split_chunk(self, n_single: int, n_kv_heads: int, max_seq_len: int, single_keys: int = 0) -> int:
+    def attention_split_chunk(self, n_single: int, n_kv_heads: int, head_dim: int, max_seq_len: int, single_keys: int = 0) -> int:
         """Keys per wave that a call with these figures splits its single-token entries by: what a caller that
         records steps into graphs has to key its recordings by, since a recording holds the chunk it was made with
         while the number of keys moves with every step."""
-        return int(self.lib.llmrs_attention_split_chunk(int(n_single), int(n_kv_heads), int(max_seq_len), int(single_keys)))
+        return int(self.lib.llmrs_attention_split_chunk(int(n_single), int(n_kv_heads), int(head_dim), int(max_seq_len), int(single_keys)))
 
     def attention(self, q, out, k_cache, v_cache, block_table, token_entry, positions, q_starts, seq_lens,
                   n_heads, n_kv_heads, head_dim, page_size, num_pages, window, scale, scratch=None, max_seq_len=0, n_single=-1,

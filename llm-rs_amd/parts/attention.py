@@ -39,7 +39,7 @@ class Attention(Mixer):
         self.kv_heads = int(p["num_kv_heads"])
         self.head_dim = int(p["head_dim"])
         self.window = int(p.get("window") or 0)
-        self.recording_signature = ("attention", self.kv_heads, self.window)
+        self.recording_signature = ("attention", self.kv_heads, self.head_dim, self.window)
         self.kv_proj = bool(p.get("kv_proj", True))
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
@@ -108,7 +108,7 @@ class Attention(Mixer):
         k = kernels()
         if not ctx.n_single or not hasattr(k, "attention_split_chunk"):
             return 0
-        return k.attention_split_chunk(ctx.n_single, self.kv_heads, ctx.max_seq_len, ctx.single_keys(self.window))
+        return k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, ctx.single_keys(self.window))
 
     def forward(self, ctx, x, h, cache):
         k = kernels()

@@ -331,13 +331,14 @@ def test_attention_chunk_rule_and_its_scratch():
     keys; never under what the scratch is sized by (the answer for one key); and the same results whichever chunk
     the number of keys leads to, with a scratch of exactly the size the library asks for."""
     k = kernels()
-    for n, kv, bound in ((1, 8, 2048), (8, 8, 2048), (12, 2, 4096), (64, 8, 2048), (200, 4, 8192), (1, 1, 131072), (3, 8, 40000)):
-        least = k.attention_split_chunk(n, kv, bound, 1)
+    for n, kv, hd, bound in ((1, 8, 128, 2048), (8, 8, 64, 2048), (12, 2, 96, 4096), (64, 8, 128, 2048), (200, 4, 256, 8192), (1, 1, 32, 131072),
+                             (3, 8, 80, 40000), (33, 8, 64, 2048)):
+        least = k.attention_split_chunk(n, kv, hd, bound, 1)
         for keys in (0, 1, n * bound // 16, n * bound // 3, n * bound, 10 * n * bound):
-            c = k.attention_split_chunk(n, kv, bound, keys)
+            c = k.attention_split_chunk(n, kv, hd, bound, keys)
             assert c in (64, 128, 256, 512, 1024) and c >= least, (n, kv, bound, keys, c, least)
             assert -(-bound // c) <= 256 or c == 1024
-    n_heads, n_kv, hd, ps = 8, 8, 64, 16
+    n_heads, n_kv, hd, ps = 8, 8, 128, 16
     lens = [1500, 700, 1290, 40, 2047, 900, 1100, 333, 1999, 1203]
     case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=41)
     g = torch.Generator().manual_seed(3)
@@ -346,7 +347,7 @@ def test_attention_chunk_rule_and_its_scratch():
     refs = [case.reference(r, qs[r], pos[r])[0].float() for r in range(len(lens))]
     seen = set()
     for keys in (0, 1, sum(lens), 40 * sum(lens), 400 * sum(lens)):
-        c = k.attention_split_chunk(len(lens), n_kv, 2048, keys)
+        c = k.attention_split_chunk(len(lens), n_kv, hd, 2048, keys)
         seen.add(c)
         need = k.attention_scratch_floats(len(lens), n_heads, hd, 2048, n_kv, len(lens))
         assert need >= len(lens) * n_heads * -(-2048 // c) * (hd + 2)
