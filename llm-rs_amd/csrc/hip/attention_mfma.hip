@@ -772,17 +772,22 @@ static int split_waves_to_a_unit(int head_dim) {
 // waves at once (eight at head size 128, twelve at 64) and works through them in turns of that many.  Waves of one
 // turn, all of the same length, end together, and the longest chunks that still fill half a turn are the fastest
 // (a wave begins with a chain of trips to memory: lengths, page numbers, then keys); one wave more than a turn
-// costs a second turn.  So: the smallest chunk that gives a unit less than a turn; and when even chunks of 1024
+// costs a second turn.  So: the smallest chunk that gives a unit no more than a turn; and when even chunks of 1024
 // keys give more, 512 if the last turn would be far from full (many short waves share out evenly as they come).
-// Against the best chunk of each case (also at sizes and lengths between those it was made from) this rule loses
-// 0.7 % on average and 9 % at worst at head size 128, 1 % and 14 % at 64; the rule before it (128 keys, doubled
-// while the waves kept all units busy, by the bound alone) lost 7.5 % and 19 %.  The chunks of a request are never
+// Against the best chunk of each case (also at sizes and lengths between those it was made from, at 4 and 8 heads
+// to a kv head, 2 and 8 kv heads) this rule loses 0.1-0.5 % on average and 9 % at worst; the rule before it (128
+// keys, doubled while the waves kept all units busy, by the bound alone) lost 7.5 % and 19 %.  The chunks of a request are never
 // more than a quarter of what the merge takes.
 // The number of keys moves with every step while a recorded graph holds the chunk it was recorded with: callers that
 // record put this function's result into what they key their recordings by.  The scratch is sized by the smallest
 // chunk the entries and the bound allow, taken at an eighth of the bound for every entry; fewer keys than that get
 // that chunk too.
+// LLMRS_SPLIT_CHUNK in the environment (64 to 1024, a power of two) takes the choice away from the rule, for measuring it.
 extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int head_dim, int max_seq_len, long single_keys) {
+    if (const char* e = getenv("LLMRS_SPLIT_CHUNK")) {
+        int c = atoi(e);
+        if (c >= ATTN_CHUNK / 2 && c <= 8 * ATTN_CHUNK && (c & (c - 1)) == 0) return c;
+    }
     double cus = (double)llmrs_compute_units();
     if (singles < 1) singles = 1;
     if (max_seq_len < 1) max_seq_len = 1;
@@ -793,11 +798,15 @@ extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int hea
         // request counts as a wave unless it is so short that it is gone before it matters
         auto to_a_unit = [&](int c) {
             double q = keys / singles / c, whole = floor(q), rest = q - whole;
-            return singles * n_kv_heads * (whole + (rest > 0.125 ? 1.0 : rest)) / cus;
+            return singles * n_kv_heads * (whole + (rest > 0.125 ? 1.0 : 0.0)) / cus;
         };
+        const double full = turn * 1.001;      // (a turn that is exactly full is the best case)
+        // (the shortest chunks are left a little before their turn is full: they gain nothing over the next length
+        // there, and a bound well above the lengths costs them twice the waves that find nothing to do)
         int c = ATTN_CHUNK / 2;
-        while (c < longest && to_a_unit(c) >= turn) c *= 2;
-        if (c == longest && to_a_unit(c) > turn) {
+        if (to_a_unit(c) >= 0.9 * turn) c *= 2;
+        while (c > ATTN_CHUNK / 2 && c < longest && to_a_unit(c) > full) c *= 2;
+        if (c == longest && to_a_unit(c) > full) {
             double last = fmod(to_a_unit(c), turn) / turn;
             if (last > 0.006 && last < 0.69) c /= 2;
         }

@@ -69,6 +69,8 @@ class StepContext:
         self.n_single = 0                               # entries that bring one token
         self.single_lens: List[int] = []                # their lengths with that token
         self._keys_seen = {}
+        self.serial = 0                                 # counts the steps bound to this context
+        self.part_state = {}                            # what parts keep from step to step, by `recording_signature`
         self.device = runner.device
         # A norm without a kernel of its own (steps of a few tokens): the part that adds into the stream last
         # before a norm leaves what that norm needs (`room_for_next_norm`, `note_left`), and the norm hands it on
@@ -245,6 +247,7 @@ class StepRunner:
         c.single_lens = [start + 1 for _, start, count in entries if count == 1]
         c.n_single = len(c.single_lens)
         c._keys_seen = {}
+        c.serial += 1
         c.tokens = dev[off.tokens:off.tokens + T]
         c.positions = dev[off.positions:off.positions + T]
         c.token_entry = dev[off.token_entry:off.token_entry + T]

@@ -103,12 +103,36 @@ class Attention(Mixer):
         return (fused and self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
                 and k.gemm_defers_norm(rows, self.w_qkv.shape[0], self.hidden))
 
+    # The kernel library shares the decoding requests' keys out over waves in chunks whose length it chooses by
+    # how many keys the step sees (`single_keys`).  A recorded step holds the chunk it was recorded with, so the
+    # chunk is part of what recordings are keyed by; and since recording a step again costs about as much as a step
+    # while a chunk that is no longer the best one costs a few per cent of the attention, a batch keeps the figure
+    # it was recorded with until the rule has asked for another chunk this many steps in a row.
+    chunk_patience = 256
+
     def recording_key(self, ctx):
-        # the keys per wave that the kernel library splits the decoding requests' caches by
         k = kernels()
         if not ctx.n_single or not hasattr(k, "attention_split_chunk"):
             return 0
-        return k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, ctx.single_keys(self.window))
+        keys = ctx.single_keys(self.window)
+        want = k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, keys)
+        held = ctx.part_state.setdefault(self.recording_signature, {})
+        at = (ctx.n_single, ctx.max_seq_len)
+        now = held.get(at)             # [chunk, a number of keys that gives it, steps in a row that wanted another, step]
+        if now is None or want == now[0] or now[2] >= self.chunk_patience:
+            now = held[at] = [want, keys, 0, ctx.serial]
+        else:
+            now[2] += 1
+            now[3] = ctx.serial
+        return now[0]
+
+    def _keys_for_the_split(self, ctx) -> int:
+        if not ctx.n_single:
+            return 0
+        now = ctx.part_state.get(self.recording_signature, {}).get((ctx.n_single, ctx.max_seq_len))
+        if now is not None and now[3] == ctx.serial:      # this step was keyed by a chunk: the figure that gives it
+            return now[1]
+        return ctx.single_keys(self.window)
 
     def forward(self, ctx, x, h, cache):
         k = kernels()
@@ -138,7 +162,7 @@ class Attention(Mixer):
         k.attention(qkv[:, :self.q_size], o, cache.k, cache.v, ctx.block_tables[g], ctx.token_entry, ctx.positions,
                     ctx.q_starts, ctx.seq_lens, self.heads, self.kv_heads, self.head_dim, cache.page_size,
                     cache.num_pages, self.window, self.scale, scratch, ctx.max_seq_len, ctx.n_single,
-                    ctx.single_keys(self.window) if ctx.n_single else 0)
+                    self._keys_for_the_split(ctx))
         leave = ctx.room_for_next_norm(h, self.w_o)
         k.gemm(o, self.w_o, h, EPI_ACCUM_F32, ctx.gemm_workspace(o, self.w_o), **({} if leave is None else {"leave": leave}))
         ctx.note_left(h, leave)
