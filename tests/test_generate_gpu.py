@@ -198,7 +198,7 @@ def test_recorded_decode_steps_equal_eager_ones(folders, which, dtype):
 def test_a_recording_is_kept_for_the_chunk_it_was_made_with():
     """The kernel library shares a decoding request's keys out over waves in chunks whose length it chooses by how
     many keys the step sees, and a recorded step holds the chunk it was recorded with.  Sixteen requests decode from
-    1335 keys on, past the length where that choice changes: the runner records a second graph for the same sizes
+    twenty keys before the length where that choice changes: the runner records a second graph for the same sizes
     there, and every step's logits stay those of an engine that records nothing."""
     from llm_rs_amd import LlamaConfig
     from llm_rs_amd.kernels import kernels
@@ -206,13 +206,16 @@ def test_a_recording_is_kept_for_the_chunk_it_was_made_with():
         architectures=["LlamaForCausalLM"], num_hidden_layers=1, hidden_size=512, num_attention_heads=8,
         num_key_value_heads=8, head_dim=64, intermediate_size=512, vocab_size=500, rope_theta=10000.0,
         max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=True))
-    n_req, plen, steps = 16, 1335, 40
+    n_req, steps = 16, 40
     k = kernels()
+    by_len = [k.attention_split_chunk(n_req, 8, 64, 2048, n_req * n) for n in range(1100, 1990)]
+    change = next(1100 + i + 1 for i, (a, b) in enumerate(zip(by_len, by_len[1:])) if a != b)
+    plen = change - 20           # (with the rule as it stands: 1335)
     chunks = {k.attention_split_chunk(n_req, 8, 64, 2048, n_req * (plen + 1 + i)) for i in range(steps)}
     assert len(chunks) == 2, "the case itself: the chunk must change on the way"
     prompts = [random_tokens(500, plen + steps + 1, seed=900 + i) for i in range(n_req)]
-    recorded = Engine.from_random(cfg, 11, dtype="bfloat16", page_size=16, num_pages=n_req * 100 + 8, max_requests=16)
-    eager = Engine.from_random(cfg, 11, dtype="bfloat16", page_size=16, num_pages=n_req * 100 + 8, max_requests=16)
+    recorded = Engine.from_random(cfg, 11, dtype="bfloat16", page_size=16, num_pages=n_req * 128 + 8, max_requests=16)
+    eager = Engine.from_random(cfg, 11, dtype="bfloat16", page_size=16, num_pages=n_req * 128 + 8, max_requests=16)
     eager.runner.use_graphs = False
     for block in recorded.model.blocks:          # (a batch would keep its first chunk for 256 steps otherwise)
         block.mixer.chunk_patience = 3
