@@ -17,7 +17,7 @@ struct RopeKvArgs {
     int rotary_dim, interleaved;
     int page_size, write_kv, num_pages;
     int row_stride;  // elements between tokens in qkv
-    int value_pages; // value_pages_kernel runs as well: it writes the values of pages that 16 tokens fill in order
+    int value_pages; // the values of a page that 16 tokens fill in order are written whole, by the first token's block
 };
 
 template <class T>
@@ -75,9 +75,9 @@ typedef __bf16 rope_bf16x8 __attribute__((ext_vector_type(8)));
 
 // Values lie transposed in a page ([head_dim][slot]), so a token's values are head_dim scattered
 // 2-byte stores.  Where 16 consecutive tokens of the batch fill one 16-slot page in order (a prompt
-// portion, page after page), that page's values are written by value_pages_kernel instead: through
-// LDS, 16 bytes a lane, whole lines.  Both kernels ask this of the same 16 tokens and get the same
-// answer.  The first 16 lanes of a block's first wave look; the answer is the same in all of them.
+// portion, page after page), that page's values are written by the block of the first of these tokens
+// instead: through LDS, 16 bytes a lane, whole lines.  All 16 blocks ask this of the same 16 tokens and get
+// the same answer.  The first 16 lanes of a block's first wave look; the answer is the same in all of them.
 __device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict__ slot_map, int t16, const RopeKvArgs& a) {
     int j = threadIdx.x & 15;
     bool mine = false;
@@ -88,34 +88,28 @@ __device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict
     return (__ballot(mine) & 0xffffull) == 0xffffull;
 }
 
-// One block per (16 tokens, kv head): [16 tokens][head_dim] in, [head_dim][16 slots] out.
-__global__ __launch_bounds__(256) void value_pages_kernel(const bf16* __restrict__ qkv, const int* __restrict__ slot_map,
-                                                          bf16* __restrict__ v_cache, RopeKvArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char vp_smem[];
-    __shared__ int whole;
-    int t16 = blockIdx.x * 16, kvh = blockIdx.y, hd = a.head_dim;
-    if (threadIdx.x < 64) {
-        bool w = first_lanes_see_whole_page(slot_map, t16, a);
-        if (threadIdx.x == 0) whole = w;
-    }
-    __syncthreads();
-    if (!whole) return;
-    bf16* tile = (bf16*)vp_smem;                        // [16][hd + 8]: rows 16 bytes apart in banks
-    int ld = hd + 8, chunks = hd / 8;
-    const bf16* src = qkv + (size_t)t16 * a.row_stride + (size_t)(a.n_heads + a.n_kv_heads + kvh) * hd;
-    for (int c = threadIdx.x; c < 16 * chunks; c += blockDim.x) {
-        int j = c / chunks, d0 = (c % chunks) * 8;
-        *(rope_bf16x8*)(tile + j * ld + d0) = *(const rope_bf16x8*)(src + (size_t)j * a.row_stride + d0);
-    }
-    __syncthreads();
+// The values of 16 tokens that fill a page, one kv head after the other: [16 tokens][head_dim] in,
+// [head_dim][16 slots] out, by all threads of a block, through `tile` ([16][head_dim + 8] in LDS).
+__device__ __forceinline__ void write_value_page(const bf16* __restrict__ qkv, const int* __restrict__ slot_map,
+                                                 bf16* __restrict__ v_cache, bf16* tile, int t16, const RopeKvArgs& a) {
+    int hd = a.head_dim, ld = hd + 8, chunks = hd / 8;       // rows 16 bytes apart in banks
     int page = slot_map[t16] / 16;
-    bf16* dst = v_cache + v_cache_index(page, kvh, 0, 0, a.n_kv_heads, 16, hd);     // this page and head: [hd][16], contiguous
-    for (int c = threadIdx.x; c < hd * 2; c += blockDim.x) {
-        int d = c >> 1, s0 = (c & 1) * 8;
-        rope_bf16x8 v;
+    for (int kvh = 0; kvh < a.n_kv_heads; ++kvh) {
+        const bf16* src = qkv + (size_t)t16 * a.row_stride + (size_t)(a.n_heads + a.n_kv_heads + kvh) * hd;
+        for (int c = threadIdx.x; c < 16 * chunks; c += blockDim.x) {
+            int j = c / chunks, d0 = (c % chunks) * 8;
+            *(rope_bf16x8*)(tile + j * ld + d0) = *(const rope_bf16x8*)(src + (size_t)j * a.row_stride + d0);
+        }
+        __syncthreads();
+        bf16* dst = v_cache + v_cache_index(page, kvh, 0, 0, a.n_kv_heads, 16, hd);     // this page and head: [hd][16], contiguous
+        for (int c = threadIdx.x; c < hd * 2; c += blockDim.x) {
+            int d = c >> 1, s0 = (c & 1) * 8;
+            rope_bf16x8 v;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = tile[(s0 + j) * ld + d];
-        *(rope_bf16x8*)(dst + d * 16 + s0) = v;
+            for (int j = 0; j < 8; ++j) v[j] = tile[(s0 + j) * ld + d];
+            *(rope_bf16x8*)(dst + d * 16 + s0) = v;
+        }
+        __syncthreads();
     }
 }
 
@@ -128,8 +122,8 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
                                                            const float* __restrict__ inv_freq,
                                                            bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
                                                            RopeKvArgs a) {
-    extern __shared__ float2 cs[];                 // [rotary_dim / 2]: cos, sin of the token's angles
-    __shared__ int values_elsewhere;               // this token's values are written by value_pages_kernel
+    extern __shared__ __attribute__((aligned(16))) float2 cs[];   // [rotary_dim / 2]: cos, sin of the token's angles; then a page's values
+    __shared__ int values_elsewhere;               // this token's values are written with its page, by the page's first token's block
     int t = blockIdx.x;
     if (threadIdx.x < 64) {
         bool w = a.write_kv && a.value_pages && first_lanes_see_whole_page(slot_map, t & ~15, a);
@@ -175,6 +169,8 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
                 v_cache[v_cache_index(page, kvh, off, d0 + j, a.n_kv_heads, a.page_size, a.head_dim)] = v[j];
         }
     }
+    if (values_elsewhere && (t & 15) == 0)         // (the same in all threads of the block)
+        write_value_page(qkv, slot_map, v_cache, (bf16*)(cs + (a.rotary_dim / 2 + 1) / 2 * 2), t, a);
 }
 
 // qkv: [n_tokens, row_stride], a row is q heads, then k heads, then v heads.
@@ -200,12 +196,10 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
              ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && rotary_dim / 2 * sizeof(float2) <= 32768)
     {
         a.value_pages = write_kv && page_size == 16 && n_kv_heads > 0 && ((uintptr_t)v_cache & 15) == 0 &&
-                        (size_t)16 * (head_dim + 8) * 2 <= 65536;
-        rope_kv_rows_kernel<<<n_tokens, 256, rotary_dim / 2 * sizeof(float2), stream>>>((bf16*)qkv, positions, slot_map, inv_freq,
-                                                                                        (bf16*)k_cache, (bf16*)v_cache, a);
-        if (a.value_pages)
-            value_pages_kernel<<<dim3(n_tokens / 16, n_kv_heads), 256, (size_t)16 * (head_dim + 8) * 2, stream>>>(
-                (const bf16*)qkv, slot_map, (bf16*)v_cache, a);
+                        (size_t)16 * (head_dim + 8) * 2 <= 32768;
+        size_t smem = (size_t)(rotary_dim / 2 + 1) / 2 * 2 * sizeof(float2) + (a.value_pages ? (size_t)16 * (head_dim + 8) * 2 : 0);
+        rope_kv_rows_kernel<<<n_tokens, 256, smem, stream>>>((bf16*)qkv, positions, slot_map, inv_freq,
+                                                             (bf16*)k_cache, (bf16*)v_cache, a);
     }
     else if (dtype == LLMRS_BF16)
         rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
