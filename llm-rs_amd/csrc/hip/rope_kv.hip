@@ -17,7 +17,7 @@ struct RopeKvArgs {
     int rotary_dim, interleaved;
     int page_size, write_kv, num_pages;
     int row_stride;  // elements between tokens in qkv
-    int value_pages; // the values of a page that 16 tokens fill in order are written whole, by the first token's block
+    int value_pages; // the values of a page that 16 tokens fill in order are written whole, a kv head by each token's block
 };
 
 template <class T>
@@ -75,8 +75,8 @@ typedef __bf16 rope_bf16x8 __attribute__((ext_vector_type(8)));
 
 // Values lie transposed in a page ([head_dim][slot]), so a token's values are head_dim scattered
 // 2-byte stores.  Where 16 consecutive tokens of the batch fill one 16-slot page in order (a prompt
-// portion, page after page), that page's values are written by the block of the first of these tokens
-// instead: through LDS, 16 bytes a lane, whole lines.  All 16 blocks ask this of the same 16 tokens and get
+// portion, page after page), that page's values are written whole instead, the 16 tokens' blocks sharing out
+// the kv heads: through LDS, 16 bytes a lane, whole lines.  All 16 blocks ask this of the same 16 tokens and get
 // the same answer.  The first 16 lanes of a block's first wave look; the answer is the same in all of them.
 __device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict__ slot_map, int t16, const RopeKvArgs& a) {
     int j = threadIdx.x & 15;
@@ -88,13 +88,14 @@ __device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict
     return (__ballot(mine) & 0xffffull) == 0xffffull;
 }
 
-// The values of 16 tokens that fill a page, one kv head after the other: [16 tokens][head_dim] in,
+// The values of 16 tokens that fill a page, for the kv heads first, first + 16, ...: [16 tokens][head_dim] in,
 // [head_dim][16 slots] out, by all threads of a block, through `tile` ([16][head_dim + 8] in LDS).
 __device__ __forceinline__ void write_value_page(const bf16* __restrict__ qkv, const int* __restrict__ slot_map,
-                                                 bf16* __restrict__ v_cache, bf16* tile, int t16, const RopeKvArgs& a) {
+                                                 bf16* __restrict__ v_cache, bf16* tile, int t16, int first,
+                                                 const RopeKvArgs& a) {
     int hd = a.head_dim, ld = hd + 8, chunks = hd / 8;       // rows 16 bytes apart in banks
     int page = slot_map[t16] / 16;
-    for (int kvh = 0; kvh < a.n_kv_heads; ++kvh) {
+    for (int kvh = first; kvh < a.n_kv_heads; kvh += 16) {
         const bf16* src = qkv + (size_t)t16 * a.row_stride + (size_t)(a.n_heads + a.n_kv_heads + kvh) * hd;
         for (int c = threadIdx.x; c < 16 * chunks; c += blockDim.x) {
             int j = c / chunks, d0 = (c % chunks) * 8;
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
                                                            bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
                                                            RopeKvArgs a) {
     extern __shared__ __attribute__((aligned(16))) float2 cs[];   // [rotary_dim / 2]: cos, sin of the token's angles; then a page's values
-    __shared__ int values_elsewhere;               // this token's values are written with its page, by the page's first token's block
+    __shared__ int values_elsewhere;               // this token's values are written with its page, the page's blocks sharing out the kv heads
     int t = blockIdx.x;
     if (threadIdx.x < 64) {
         bool w = a.write_kv && a.value_pages && first_lanes_see_whole_page(slot_map, t & ~15, a);
@@ -169,8 +170,8 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
                 v_cache[v_cache_index(page, kvh, off, d0 + j, a.n_kv_heads, a.page_size, a.head_dim)] = v[j];
         }
     }
-    if (values_elsewhere && (t & 15) == 0)         // (the same in all threads of the block)
-        write_value_page(qkv, slot_map, v_cache, (bf16*)(cs + (a.rotary_dim / 2 + 1) / 2 * 2), t, a);
+    if (values_elsewhere)                          // (the same in all threads of the block) the page's 16 blocks share out the kv heads
+        write_value_page(qkv, slot_map, v_cache, (bf16*)(cs + (a.rotary_dim / 2 + 1) / 2 * 2), t & ~15, t & 15, a);
 }
 
 // qkv: [n_tokens, row_stride], a row is q heads, then k heads, then v heads.
