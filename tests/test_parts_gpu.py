@@ -470,6 +470,48 @@ def test_decode_steps_of_a_stateful_mixer_are_recorded_and_replayed():
     assert eng.runner.graph_replays >= 60, eng.runner.graph_replays
 
 
+class KeyedDecayMixer(RecordableDecayMixer):
+    """The same again, but what a decode step launches follows a host value that moves from step to step though
+    the step's sizes stay (here: whether the requests' lengths add up to an even number of fours): the part names
+    what that depends on and what it comes to for a step, and the step function keeps a recording for each value."""
+    recording_signature = "test_keyed_decay"
+
+    def recording_key(self, ctx):
+        return (sum(ctx.single_lens) // 4) % 2
+
+    def forward(self, ctx, x, h, cache):
+        super().forward(ctx, x, h, cache)
+        if ctx.n_single == ctx.n_entries and self.recording_key(ctx):
+            h += 0.25
+
+
+def test_a_part_whose_launches_follow_a_host_value_gets_a_recording_for_each_value():
+    register_mixer("test_decay_keyed", KeyedDecayMixer)
+    register_architecture("TestToyForCausalLM", ToyConfig)
+    H, V = 40, 90
+    from llm_rs_amd.engine import Model
+    cfg = ToyConfig({"architectures": ["TestToyForCausalLM"], "hidden_size": H, "vocab_size": V, "decay_kind": "test_decay_keyed"})
+    names = Model(cfg.model_spec(), torch.float32, "cpu").tensors()
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.2)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    recorded = Engine(cfg, ws, dtype="float32", page_size=16, num_pages=32, max_requests=4)
+    eager = Engine(cfg, ws, dtype="float32", page_size=16, num_pages=32, max_requests=4)
+    eager.runner.use_graphs = False
+    assert recorded.runner.use_graphs
+    seqs = [torch.randint(0, V, (40,), generator=torch.Generator().manual_seed(5 + i)).tolist() for i in range(2)]
+    slots = {eng: [eng.open_request() for _ in seqs] for eng in (recorded, eager)}
+    for eng in (recorded, eager):
+        eng.step([StepEntry(slots[eng][i], 0, seqs[i][:6], []) for i in range(2)])
+    with_it = 0
+    for p in range(6, 40):
+        a, b = (eng.step([StepEntry(slots[eng][i], p, [seqs[i][p]], [0]) for i in range(2)]).clone() for eng in (recorded, eager))
+        torch.cuda.synchronize()
+        assert torch.equal(a, b), f"position {p}"
+        with_it += ((2 * (p + 1)) // 4) % 2
+    assert 10 <= with_it <= 24, "the case itself: both values come"
+    assert len(recorded.runner._graphs) == 2 and recorded.runner.graph_replays >= 28
+
+
 # ---- other arrangements of a layer, a scaled embedding and bent logits ---------------------------
 
 class ParallelBlock(Block):
