@@ -10,6 +10,50 @@ struct AttnArgs {
     float scale;
 };
 
+#if defined(__HIPCC__)
+// A step's entries bring their tokens as tiles of `per` tokens that never cross an entry; entries with one token
+// bring none when the caller splits those by key range instead.  Which entry holds tile `tile`, and which of that
+// entry's tiles it is: a wave finds out together, 64 entries at a time (a serving step has hundreds of entries,
+// and a walk from entry to entry by every block cost a prompt portion's kernel more than its own work: 102 ->
+// 182 us beside 230 decoding requests).  All lanes of a wave call these with the same arguments and get the same
+// answers; false when the tile lies beyond the last one.
+__device__ __forceinline__ int tiles_of_entry(const int* __restrict__ q_starts, int n_entries, int i, int per, int skip_single) {
+    if (i >= n_entries) return 0;
+    int cnt = q_starts[i + 1] - q_starts[i];
+    return (cnt == 1 && skip_single) ? 0 : (cnt + per - 1) / per;
+}
+__device__ __forceinline__ int count_tiles(const int* __restrict__ q_starts, int n_entries, int per, int skip_single) {
+    int lane = threadIdx.x & 63, mine = 0;
+    for (int i = lane; i < n_entries; i += 64) mine += tiles_of_entry(q_starts, n_entries, i, per, skip_single);
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mine += __shfl_xor(mine, d);
+    return mine;
+}
+__device__ __forceinline__ bool locate_tile(const int* __restrict__ q_starts, int n_entries, int per, int skip_single,
+                                            int tile, int& entry, int& within) {
+    int lane = threadIdx.x & 63, left = tile;
+    for (int base = 0; base < n_entries; base += 64) {
+        int nt = tiles_of_entry(q_starts, n_entries, base + lane, per, skip_single);
+        int incl = nt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int v = __shfl_up(incl, d);
+            if (lane >= d) incl += v;
+        }
+        int total = __shfl(incl, 63);
+        if (left < total) {
+            unsigned long long holds = __ballot(left >= incl - nt && left < incl);    // one lane: its entry has tiles, and this one
+            int src = __ffsll((long long)holds) - 1;
+            entry = base + src;
+            within = left - __shfl(incl - nt, src);
+            return true;
+        }
+        left -= total;
+    }
+    return false;
+}
+#endif
+
 // The matrix-core kernels (attention_mfma.hip).  Return 1 when they took the
 // call, 0 when its shape is not theirs, -1 on error.
 int llmrs_attention_bf16_mfma(hipStream_t stream, const bf16* q, bf16* out, const bf16* k_cache, const bf16* v_cache,

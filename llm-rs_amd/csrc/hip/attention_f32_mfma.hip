@@ -43,14 +43,8 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
     int task = blockIdx.x * 4 + wave;
     int kvh = (task >> 2) % a.n_kv_heads;
     int tile = (task / (4 * a.n_kv_heads)) * 4 + (task & 3);
-    int e = 0, rem = tile;
-    for (; e < n_entries; ++e) {
-        int cnt = q_starts[e + 1] - q_starts[e];
-        int nt = (cnt == 1 && skip_single) ? 0 : (cnt + tpt - 1) / tpt;
-        if (rem < nt) break;
-        rem -= nt;
-    }
-    if (e == n_entries) return;
+    int e = 0, rem = 0;
+    if (!locate_tile(q_starts, n_entries, tpt, skip_single, tile, e, rem)) return;
     int tok0 = q_starts[e] + rem * tpt;
     int ntok = min(tpt, q_starts[e + 1] - tok0);
     int tq = c / G, hg = c - tq * G;

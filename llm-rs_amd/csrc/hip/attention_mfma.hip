@@ -187,14 +187,8 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
     int task = blockIdx.x * 4 + wave;
     int kvh = (task >> 2) % a.n_kv_heads;
     int tile = (task / (4 * a.n_kv_heads)) * 4 + (task & 3);
-    int e = 0, rem = tile;
-    for (; e < n_entries; ++e) {
-        int cnt = q_starts[e + 1] - q_starts[e];
-        int nt = (cnt == 1 && skip_single) ? 0 : (cnt + tpt - 1) / tpt;
-        if (rem < nt) break;
-        rem -= nt;
-    }
-    if (e == n_entries) return;
+    int e = 0, rem = 0;
+    if (!locate_tile(q_starts, n_entries, tpt, skip_single, tile, e, rem)) return;
     int tok0 = q_starts[e] + rem * tpt;
     int ntok = min(tpt, q_starts[e + 1] - tok0);
     int tq = c / G, hg = c - tq * G;
@@ -269,24 +263,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     // blocks of the first two rounds (a round: as many blocks as the device holds at once in one
     // layer, `round_blocks`) are resident together, the second round beside the first on the same
     // units, so the second round runs in the opposite order and puts the shortest beside the longest.
-    int n_btiles = 0;
-    for (int i = 0; i < n_entries; ++i) {
-        int cnt = q_starts[i + 1] - q_starts[i];
-        n_btiles += (cnt == 1 && skip_single) ? 0 : (cnt + 4 * tpt - 1) / (4 * tpt);
-    }
+    int n_btiles = count_tiles(q_starts, n_entries, 4 * tpt, skip_single);      // (every wave for itself: the same figures)
     int g = blockIdx.x / a.n_kv_heads;
     if (g >= n_btiles) return;                       // the grid is sized for the most tiles the tokens could make
     int gr = round_blocks / a.n_kv_heads;
     if (g >= gr && g < 2 * gr) g = gr + (min(2 * gr, n_btiles) - 1 - g);
     int btile = n_btiles - 1 - g;                    // 4 * tpt tokens of one entry
-    int e = 0, rem = btile;
-    for (; e < n_entries; ++e) {
-        int cnt = q_starts[e + 1] - q_starts[e];
-        int nt = (cnt == 1 && skip_single) ? 0 : (cnt + 4 * tpt - 1) / (4 * tpt);
-        if (rem < nt) break;
-        rem -= nt;
-    }
-    if (e == n_entries) return;
+    int e = 0, rem = 0;
+    if (!locate_tile(q_starts, n_entries, 4 * tpt, skip_single, btile, e, rem)) return;
     int e_end = q_starts[e + 1];
     int btok0 = q_starts[e] + rem * 4 * tpt;
     int btok_last = min(btok0 + 4 * tpt, e_end) - 1;
