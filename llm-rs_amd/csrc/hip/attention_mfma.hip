@@ -126,19 +126,53 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
         return min(max(pg, 0), num_pages - 1);
     };
     int pv = have_pages ? first_pages : load_pages(pv_base);     // (the caller's: those of pages t_begin / 16 + lane, clamped as here)
-    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+    // Small heads leave registers for a second set of key operands: the next tile's keys are asked for before this
+    // tile's products, one trip to memory per tile instead of two in a row (keys, then values).  At head size 128
+    // that set would push the wave past 256 registers.
+    constexpr bool KEYS_AHEAD = HD <= 64;
+    int p0 = 0, p1 = 0;
+    auto pages_of = [&](int t0, int& a0, int& a1) {
         int lp = t0 >> 4;
         if (lp + 1 - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
-        int p0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
-        int p1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : p0;   // a tile's second page may lie past the last key
-        const bf16* kp = kc + (((size_t)(kk < 16 ? p0 : p1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8;
+        a0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
+        a1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : a0;   // a tile's second page may lie past the last key
+    };
+    auto keys_at = [&](int a0, int a1) { return kc + (((size_t)(kk < 16 ? a0 : a1) * n_kv + kvh) * 16 + (kk & 15)) * HD + h * 8; };
+    bf16x8 kf[HD / 16];
+    if constexpr (KEYS_AHEAD) {
+        pages_of(t_begin, p0, p1);
+        const bf16* kp = keys_at(p0, p1);
+#pragma unroll
+        for (int ks = 0; ks < HD / 16; ++ks) kf[ks] = *(const bf16x8*)(kp + ks * 16);
+    }
+    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
         f32x16 S;
 #pragma unroll
         for (int i = 0; i < 16; ++i) S[i] = 0.0f;
+        int n0 = 0, n1 = 0;
+        if constexpr (KEYS_AHEAD) {
+            bf16x8 kn[HD / 16];
+            const bool more = t0 + 32 < t_end;                   // (the same in all lanes)
+            if (more) {
+                pages_of(t0 + 32, n0, n1);
+                const bf16* kp = keys_at(n0, n1);
 #pragma unroll
-        for (int ks = 0; ks < HD / 16; ++ks) {
-            bf16x8 kf = *(const bf16x8*)(kp + ks * 16);
-            S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], S, 0, 0, 0);
+                for (int ks = 0; ks < HD / 16; ++ks) kn[ks] = *(const bf16x8*)(kp + ks * 16);
+            }
+#pragma unroll
+            for (int ks = 0; ks < HD / 16; ++ks) S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], S, 0, 0, 0);
+            if (more) {
+#pragma unroll
+                for (int ks = 0; ks < HD / 16; ++ks) kf[ks] = kn[ks];
+            }
+        } else {
+            pages_of(t0, p0, p1);
+            const bf16* kp = keys_at(p0, p1);
+#pragma unroll
+            for (int ks = 0; ks < HD / 16; ++ks) {
+                bf16x8 k1 = *(const bf16x8*)(kp + ks * 16);
+                S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(k1, qf[ks], S, 0, 0, 0);
+            }
         }
         // values of both pages: issued here so that their latency hides behind the softmax
         bf16x8 vf[HD / 32][2];
@@ -168,6 +202,7 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[HD / 16], f32x16
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][0], pf[0], O[dt], 0, 0, 0);
             O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[dt][1], pf[1], O[dt], 0, 0, 0);
         }
+        if constexpr (KEYS_AHEAD) { p0 = n0; p1 = n1; }
     }
 }
 
@@ -483,7 +518,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
 // where its keys begin (ch * chunk) without the request's length: it asks for its page numbers and its queries together
 // with the length, one trip to memory instead of two in a row.
 template <int HD>
-__global__ __launch_bounds__(64) void attn_split_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 3 : 1))) void attn_split_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
                                                         const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                                         const int* __restrict__ block_table,
                                                         const int* __restrict__ seq_lens,
