@@ -1292,7 +1292,15 @@ extern "C" long llmrs_gemm_workspace_floats(int M, int N, int K) {
         int s = skinny_splits(N, K);            // the rows beyond whole large tiles go to the kernel for few rows
         return s > 1 ? (long)s * (M % 256) * N : 0;
     }
-    if (M > 64 && (long)ceil_div(M, 256) * ceil_div(N, 256) < 160) { int s = tiled_splits(M, N, K); return s > 1 ? (long)s * M * N : 0; }
+    if (M > 64 && (long)ceil_div(M, 256) * ceil_div(N, 256) < 160) {
+        int s = tiled_splits(M, N, K);
+        long own = s > 1 ? (long)s * M * N : 0;
+        // a few rows beyond whole 128-row tiles may go to the kernel for few rows, and the whole tiles be split then
+        int over128 = M % 128;
+        if (M >= 1024 && over128 > 0 && over128 <= 64 && K % 64 == 0)
+            own = std::max(own, std::max(llmrs_gemm_workspace_floats(M - over128, N, K), llmrs_gemm_workspace_floats(over128, N, K)));
+        return own;
+    }
     return 0;
 }
 
@@ -1487,6 +1495,27 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                              : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, N, K, epi);
             }
         } else if (K % 64 == 0) {
+            // The same for the 128 x 128 tiles, whose blocks run two to a compute unit: a few rows beyond whole
+            // tiles that cost them another round of the device, or the split of k that filled it, go to the kernel
+            // for few rows (the o and down products of the 8B shape: 2049 rows 526 -> about 350 us, 1025 rows 287 -> 240).
+            // Counted in k-tiles that a place works through, round after round.
+            int over128 = M % 128;
+            if (M >= 1024 && over128 > 0 && over128 <= 64 && !whole && next == nullptr && scale == nullptr) {
+                auto walk = [&](int rows) {
+                    int s = tiled_splits(rows, N, K);
+                    if (s > 1 && (workspace == nullptr || workspace_bytes < (size_t)s * rows * N * sizeof(float))) s = 1;
+                    long blocks = (long)ceil_div(rows, 128) * ceil_div(N, 128) * s;
+                    return ceil_div(blocks, (long)cus * 2) * (K / 64 / s);
+                };
+                if (walk(M) - walk(M - over128) >= 32) {
+                    size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
+                    int whole_rows = M - over128;
+                    rc = llmrs_gemm_bf16_mfma(stream, A, lda, W, out, ldc, whole_rows, N, K, epi, workspace, workspace_bytes, qkv);
+                    if (rc != 1) return rc;
+                    return llmrs_gemm_bf16_mfma(stream, A + (size_t)whole_rows * lda, lda, W, (char*)out + (size_t)whole_rows * ldc * elt,
+                                                ldc, over128, N, K, epi, workspace, workspace_bytes, qkv);
+                }
+            }
             int splits = tiled_splits(M, N, K);
             if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
                 rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace, next);

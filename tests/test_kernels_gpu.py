@@ -55,6 +55,8 @@ GEMM_SHAPES = [(1, 40, 72), (5, 100, 200), (16, 48, 64), (17, 96, 320), (64, 256
                (130, 96, 320), (300, 520, 776), (257, 384, 96), (8, 1000, 4096), (33, 64, 20),
                (64, 200, 2048), (40, 1000, 1096), (64, 4096, 4096), (24, 520, 2048), (50, 64, 8200),
                (8, 38, 100), (3, 130, 4099), (1, 6, 20),
+               # a few rows beyond whole 128-row tiles that would cost another round of the device (or the split of k): the few-row kernel takes them
+               (2049, 4096, 2048), (1025, 4096, 4096), (2088, 4096, 2048),
                # 33 to 48 rows: blocks of three row tiles, in each of the few-row kernel's shapes
                (48, 4096, 4096), (36, 16400, 264), (47, 6144, 2048), (34, 2048, 2048), (41, 300, 136),
                # 256 x 192 tiles where they make whole rounds of the device and square ones do not; the last tile cut by N
