@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context already in the cache, decode K steps
@@ -22,6 +22,8 @@ The other workloads print one line of the same form each:
             batch 1/8/64) and at batch 128/256 (context 2048), each with its share of the HBM roofline.
   sizes1b   the 1B shape decoding at batch 1/8/64 (context 2048) with its shares of the HBM roofline: batch 1 is
             the case the reference states its own bandwidth figure for.
+  prompts   the 8B shape's prompt step at lengths from 256 to 8192 tokens, among them lengths one token past whole
+            tiles: tokens a second and the share of the matrix cores' peak for each; value = the 2,048-token one.
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -52,7 +54,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -157,6 +159,17 @@ def sizes_line(args, layers, points, fractions, first_step_s=0.0, model="Llama-3
                      flat_config(model, layers, 0, 8192 if model == "Llama-3.1-8B shape" else 2048, 16))
     line["points"] = points
     line["roofline_frac"] = fractions
+    return line
+
+
+def prompts_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
+    """`value` and `ms_per_step` are the 2,048-token prompt's (the first point); a step is one prompt step."""
+    first = next(iter(points))
+    line = base_line("prefill tok/s of the 8B shape over prompt lengths (one request, its whole prompt in one step), each with its "
+                     "share of the matrix cores' peak", points[first], args.steps, args.warmup, first_step_s, args.dtype,
+                     flat_config("Llama-3.1-8B shape", layers, 1, 8192, 16))
+    line["points"] = points
+    line["peak_frac"] = fractions
     return line
 
 
@@ -289,6 +302,30 @@ def run_sizes(args) -> dict:
                       "Llama-3.2-1B shape" if small else "Llama-3.1-8B shape")
 
 
+def run_prompts(args) -> dict:
+    from llm_rs_amd import StepEntry
+    lengths = (2048, 256, 512, 1024, 1025, 2049, 4096, 8192)
+    b = Bench(args, LLAMA_8B, max(lengths) // 16 + 16, 8, max(lengths))
+    engine = b.engine
+    reps = max(2, min(args.steps // 8, 8))
+    points, fractions, first_s = {}, {}, None
+    for T in lengths:
+        toks = b.prompt(T)
+
+        def prompt_once():
+            slot = engine.open_request()
+            engine.step([StepEntry(slot, 0, toks, [T - 1])])
+            engine.close_request(slot)
+
+        prompt_once()
+        s = b.timed(prompt_once, reps)
+        first_s = s if first_s is None else first_s
+        points[f"prefill_{T}"] = round(T / s, 1)
+        fractions[f"prefill_{T}"] = round(prefill_flops(LLAMA_8B, b.config.num_hidden_layers, T) / s / PEAK_FLOPS[args.dtype], 4)
+        print(f"[bench] prompt of {T} tokens: {s * 1e3:.2f} ms, {fractions[f'prefill_{T}'] * 100:.1f}% of the peak", file=sys.stderr, flush=True)
+    return prompts_line(args, b.config.num_hidden_layers, points, fractions, first_s)
+
+
 def run_serve1b(args) -> dict:
     n, new = args.requests, args.new_tokens
     b = Bench(args, LLAMA_1B, (n * (4096 + new)) // 16 + 64, n, args.max_batch_tokens)
@@ -360,7 +397,8 @@ def main() -> int:
     heavy = args.workload == "mixed70b"
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
-    line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes}[args.workload](args)
+    line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
+            "prompts": run_prompts}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()
