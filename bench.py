@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context already in the cache, decode K steps
@@ -24,6 +24,8 @@ The other workloads print one line of the same form each:
             the case the reference states its own bandwidth figure for.
   prompts   the 8B shape's prompt step at lengths from 256 to 8192 tokens, among them lengths one token past whole
             tiles: tokens a second and the share of the matrix cores' peak for each; value = the 2,048-token one.
+  long      the 8B shape with the 131,072 positions of Llama 3.1: one request decoding over 131,000 keys and four over
+            32,700 each, with their shares of the HBM roofline (filling the caches takes about ten seconds).
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -54,7 +56,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -157,6 +159,17 @@ def sizes_line(args, layers, points, fractions, first_step_s=0.0, model="Llama-3
     line = base_line(f"decode tok/s of the {model.split()[0].split('-')[-1]} shape at {what}, each with its share of the HBM roofline",
                      points[first], args.steps, args.warmup, first_step_s, args.dtype,
                      flat_config(model, layers, 0, 8192 if model == "Llama-3.1-8B shape" else 2048, 16))
+    line["points"] = points
+    line["roofline_frac"] = fractions
+    return line
+
+
+def long_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
+    """`value` and `ms_per_step` are the first point's (one request over the longest cache)."""
+    first = next(iter(points))
+    line = base_line("decode tok/s of the 8B shape over long caches (131,072 positions), each with its share of the HBM roofline",
+                     points[first], args.steps, args.warmup, first_step_s, args.dtype,
+                     flat_config("Llama-3.1-8B shape", layers, 0, 131072, 16, max_context=131072))
     line["points"] = points
     line["roofline_frac"] = fractions
     return line
@@ -302,6 +315,27 @@ def run_sizes(args) -> dict:
                       "Llama-3.2-1B shape" if small else "Llama-3.1-8B shape")
 
 
+def run_long(args) -> dict:
+    steps, warmup = 16, 4
+    shape = dict(LLAMA_8B, max_position_embeddings=131072)
+    cases = [(1, 131072 - 64), (4, 32768 - 64)]
+    pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
+    b = Bench(args, shape, pages, 8, 2048)
+    weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
+    points, fractions, first_s = {}, {}, None
+    for batch, ctx in cases:
+        t0 = time.time()
+        s, _ = b.decode_run(batch, ctx, steps, warmup)
+        first_s = s if first_s is None else first_s
+        key = f"decode_b{batch}_ctx{ctx}"
+        points[key] = round(batch / s, 1)
+        fractions[key] = round((weight_bytes + batch * (ctx + warmup + steps // 2) * per_token) / s / PEAK_HBM, 4)
+        print(f"[bench] {key}: {s * 1e3:.3f} ms/step, {fractions[key] * 100:.1f}% of the HBM roofline (with filling the caches: "
+              f"{time.time() - t0:.0f} s)", file=sys.stderr, flush=True)
+    args.steps, args.warmup = steps, warmup
+    return long_line(args, b.config.num_hidden_layers, points, fractions, first_s)
+
+
 def run_prompts(args) -> dict:
     from llm_rs_amd import StepEntry
     lengths = (2048, 256, 512, 1024, 1025, 2049, 4096, 8192)
@@ -398,7 +432,7 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts}[args.workload](args)
+            "prompts": run_prompts, "long": run_long}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

@@ -73,5 +73,8 @@ def test_lines_of_every_workload():
     assert set(line["points"]) == set(line["roofline_frac"])
     line = check_line(b.sizes_line(args, 16, {"decode_b1_ctx2048": 900.0}, {"decode_b1_ctx2048": 0.4}, 0.0011, "Llama-3.2-1B shape"))
     assert line["config"]["model"] == "Llama-3.2-1B shape" and line["config"]["hidden_size"] == 2048 and "1B shape" in line["metric"]
+    line = check_line(b.long_line(args, 32, {"decode_b1_ctx131008": 130.0, "decode_b4_ctx32704": 400.0},
+                                  {"decode_b1_ctx131008": 0.6, "decode_b4_ctx32704": 0.6}, 0.0077))
+    assert line["config"]["max_context"] == 131072 and set(line["points"]) == set(line["roofline_frac"])
     line = check_line(b.prompts_line(args, 32, {"prefill_2048": 67000.0, "prefill_2049": 60000.0}, {"prefill_2048": 0.39, "prefill_2049": 0.35}, 0.0305))
     assert set(line["points"]) == set(line["peak_frac"]) and line["value"] == 67000.0 and abs(line["ms_per_step"] - 30.5) < 1e-6
