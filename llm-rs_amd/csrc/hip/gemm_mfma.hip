@@ -1474,7 +1474,12 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
             const bool four = small && fourwave_takes(epi, out, ldc, N);
             long whole = big_tiles / cus * cus, rest = big_tiles - whole;
             int n_split = (int)(whole / m_tiles) * 256;        // features of the whole rounds
-            if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4) {
+            // (the features beyond whole rounds run on 128 x 128 tiles, two to a unit, a round of which takes about 0.62 of
+            // a round of large tiles: when they come to more than one such round, a last round of large tiles that is
+            // not full may be the shorter way: the o and down products at 6144 rows, 1.5 rounds of large tiles)
+            long small_blocks = (long)ceil_div(N - n_split, 128) * ceil_div(M, 128);
+            bool split_pays = (double)(whole / cus) + 0.62 * ceil_div(small_blocks, 2L * cus) < (double)ceil_div(big_tiles, (long)cus);
+            if (n_split > 0 && n_split < N && rest > 0 && 2 * rest <= cus + cus / 4 && split_pays) {
                 size_t elt = (epi == LLMRS_EPI_STORE_F32 || epi == LLMRS_EPI_ACCUM_F32) ? sizeof(float) : sizeof(bf16);
                 void* out_rest = (char*)out + (size_t)(epi == LLMRS_EPI_SWIGLU ? n_split / 2 : n_split) * elt;
                 rc = four && fourwave_takes(epi, out, ldc, n_split)
