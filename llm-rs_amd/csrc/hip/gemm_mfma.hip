@@ -1522,7 +1522,16 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                 }
             }
             int splits = tiled_splits(M, N, K);
-            if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
+            // Many rows on a weight too narrow for the square tiles: four waves on 256 x 128 (128 x 64 a wave, a block
+            // to a unit) where such tiles come to whole rounds of the device, or nearly: a k-step brings 48 KB into a
+            // unit for the work that two 128 x 128 blocks bring 64 KB for (the o and down products of the 8B shape at
+            // 2048 rows: a prompt step 31.55 -> 31.03 ms).
+            long wide_blocks = (long)ceil_div(M, 256) * ceil_div(N, 128);
+            const bool small4 = (size_t)M * lda * 2 < ((size_t)1 << 32) && (size_t)N * K * 2 < ((size_t)1 << 32);
+            if (splits == 1 && !whole && next == nullptr && M >= 1024 && small4 && fourwave_takes(epi, out, ldc, N) &&
+                10 * wide_blocks >= 9 * (long)ceil_div(wide_blocks, (long)cus) * cus)
+                rc = launch_fourwave<256, 128>(stream, A, lda, W, out, ldc, M, N, K, epi);
+            else if (splits > 1 && workspace != nullptr && workspace_bytes >= (size_t)splits * M * N * sizeof(float))
                 rc = launch_tiles_128(stream, A, lda, W, out, ldc, M, N, K, epi, splits, (float*)workspace, next);
             else if (whole) rc = llmrs_fail("gemm: M=%d N=%d K=%d is not split after all: the norm cannot be finished here", M, N, K);
             else
