@@ -1486,8 +1486,14 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                          ? launch_fourwave<256, 256>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
                      : small ? launch_pingpong<256, 256, 2, 4, true>(stream, A, lda, W, out, ldc, M, n_split, K, epi)
                              : launch_pingpong<256, 256, 2, 4, false>(stream, A, lda, W, out, ldc, M, n_split, K, epi);
-                if (rc == 0)
-                    rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
+                if (rc == 0) {
+                    long wide_rest = m_tiles * ceil_div(N - n_split, 128);      // (256 x 128 tiles where they come to whole rounds, as below)
+                    if (four && M >= 1024 && fourwave_takes(epi, out_rest, ldc, N - n_split) &&
+                        10 * wide_rest >= 9 * (long)ceil_div(wide_rest, (long)cus) * cus)
+                        rc = launch_fourwave<256, 128>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
+                    else
+                        rc = launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W + (size_t)n_split * K, out_rest, ldc, M, N - n_split, K, epi);
+                }
             } else if (long t192 = m_tiles * ceil_div(N, 192); rest > 0 && t192 % cus == 0) {
                 // 256 x 192 tiles where they come to whole rounds of the device and the square ones do not: the
                 // q/k/v product of the 8B shape at 2048 rows is 192 square tiles on 256 units, or 256 of these
