@@ -452,6 +452,38 @@ def test_attention_many_decoding_requests(n_req, window):
         assert (got[r].float() - want).abs().max() < 0.07, f"request {r} of length {lens[r]}, key {fars[r]}"
 
 
+@pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.bfloat16, 8, 2, 128, 16), (torch.bfloat16, 8, 2, 96, 16),
+                                                     (torch.float32, 4, 2, 64, 16), (torch.bfloat16, 8, 8, 64, 16)])
+def test_attention_prompt_portions_among_many_entries(dtype, n_heads, n_kv, hd, ps):
+    """A serving step: prompt portions at the start, in the middle and at the end of 150 entries that bring one
+    token each.  A tile's entry is looked up 64 entries at a time (the kernels with shared tiles, those without, and the
+    32-bit tiles each do it): every portion's rows against the plain implementation, and some of the single tokens."""
+    g = torch.Generator().manual_seed(hd)
+    n_single = 150
+    single_lens = [int(x) for x in torch.randint(3, 200, (n_single,), generator=g)]
+    portions = {0: (40, 70), 77: (0, 33), 151: (100, 45), 152: (5, 1)}      # entry -> (start, tokens); the last brings one token of a prompt
+    lens, counts = [], []
+    singles = iter(single_lens)
+    for e in range(n_single + len(portions)):
+        if e in portions:
+            start, cnt = portions[e]
+            lens.append(start + cnt); counts.append(cnt)
+        else:
+            lens.append(next(singles)); counts.append(1)
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=hd + 1)
+    qs = [torch.randn((c, n_heads, hd), generator=g).to(dtype) for c in counts]
+    pos = [list(range(n - c, n)) for n, c in zip(lens, counts)]
+    got = case.run(qs, pos, n_single=sum(1 for c in counts if c == 1))
+    at = [0]
+    for c in counts:
+        at.append(at[-1] + c)
+    floor = 2e-6 if dtype == torch.float32 else 4e-3
+    for e in list(portions) + [1, 63, 64, 76, 78, 127, 128, 150]:
+        ref = case.reference(e, qs[e], pos[e])
+        err = (got[at[e]:at[e + 1]].double() - ref).abs()
+        assert (err <= out_tol(ref, dtype, floor)).all(), f"entry {e} ({counts[e]} tokens): max err {float(err.max())}"
+
+
 @pytest.mark.parametrize("window", [0, 200])
 @pytest.mark.parametrize("dtype,n_heads,n_kv,hd,ps", [(torch.float32, 4, 2, 64, 16), (torch.float32, 3, 1, 20, 4),
                                                      (torch.bfloat16, 6, 3, 48, 8), (torch.bfloat16, 5, 5, 80, 16),
