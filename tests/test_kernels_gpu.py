@@ -206,7 +206,8 @@ def test_rope_kv_write(dtype, n_heads, n_kv, hd, rot, layout, page_size):
 
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,rot,page_size", [(5, 5, 48, 48, 16), (2, 1, 128, 128, 16), (8, 2, 64, 32, 16),
-                                                           (32, 8, 128, 128, 16), (3, 1, 80, 0, 8)])
+                                                           (32, 8, 128, 128, 16), (3, 1, 80, 0, 8),
+                                                           (20, 20, 32, 32, 16)])    # more kv heads than a page has tokens' blocks to share them out to
 def test_rope_kv_write_many_tokens(n_heads, n_kv, hd, rot, page_size):
     _rope_case(torch.bfloat16, n_heads, n_kv, hd, rot, "interleaved", page_size, repeat=4)
     _rope_case(torch.float32, n_heads, n_kv, hd, rot, "interleaved", page_size, repeat=4)
