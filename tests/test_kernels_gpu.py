@@ -423,6 +423,31 @@ def test_attention_few_decoding_requests(window, portion):
             assert (got[n_dec:].float() - ref).abs().max() <= 3e-2
 
 
+@pytest.mark.parametrize("n_req,hd", [(3, 128), (20, 128), (70, 64), (70, 128), (160, 128)])
+def test_attention_decoding_requests_a_few_keys_past_a_chunk(n_req, hd):
+    """Lengths a few keys (and a few more than a few) past multiples of every chunk length: a request's last chunk
+    then holds a handful of keys.  The strong key among those last keys, at the first of them and just before: the
+    output must be that key's value, for every number of requests (which decides the chunk length)."""
+    n_heads, n_kv, ps = 8, 2, 16
+    tails = [1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129]
+    lens = [(64 << (r % 5)) * (1 + r % 2) + tails[r % len(tails)] for r in range(n_req)]
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=17)
+    for which in range(3):
+        qs, fars = [], []
+        for r, n in enumerate(lens):
+            t = tails[r % len(tails)]
+            far = (n - 1, n - t, n - t - 1)[which]
+            fars.append(far)
+            qs.append((case.k[r][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16))
+        got = case.run(qs, [[n - 1] for n in lens], n_single=n_req, single_keys=sum(lens))
+        for r in range(n_req):
+            want = case.v[r][fars[r]].float().repeat_interleave(n_heads // n_kv, dim=0)
+            assert (got[r].float() - want).abs().max() < 0.07, f"request {r} of length {lens[r]}, key {fars[r]}"
+            if r < 6:
+                ref = case.reference(r, qs[r], [lens[r] - 1])[0].float()
+                assert (got[r].float() - ref).abs().max() <= 2e-2, f"request {r}"
+
+
 @pytest.mark.parametrize("window", [0, 300])
 @pytest.mark.parametrize("n_req", [70, 150])
 def test_attention_many_decoding_requests(n_req, window):
