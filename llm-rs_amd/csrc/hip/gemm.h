@@ -63,6 +63,10 @@ __device__ __forceinline__ void epilogue_store(int epi, void* out, int ldc, int 
 // qkv: needed when epi is LLMRS_EPI_QKV; such a call is taken only by the kernels that fuse it.
 // scale, next: see RowScale and NextNorm; both only where llmrs_gemm_defers_norm(M, N, K) holds (next: with
 // LLMRS_EPI_ACCUM_F32 only), or next with eps where llmrs_gemm_norms_whole(M, N, K) holds.
+// The product left as the parts of its sum over k, [parts][M][N] 32-bit in `workspace` (gemm_mfma.hip): the number of
+// parts, 0 when this product would not be split (nothing launched), -1 on error.
+int llmrs_gemm_bf16_split_parts(hipStream_t stream, const bf16* A, int lda, const bf16* W, int M, int N, int K,
+                                void* workspace, size_t workspace_bytes);
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
                          int M, int N, int K, int epi, void* workspace, size_t workspace_bytes,
                          const QkvEpilogue* qkv = nullptr, const RowScale* scale = nullptr, const NextNorm* next = nullptr);

@@ -787,7 +787,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_dma_kernel(const bf16* __
 
 template <int BM, int BN, int WGM, int WGN, int STAGES>
 static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                      int M, int N, int K, int epi, int splits = 1, float* partial = nullptr, const NextNorm* next = nullptr) {
+                      int M, int N, int K, int epi, int splits = 1, float* partial = nullptr, const NextNorm* next = nullptr,
+                      bool finish = true) {
     static bool configured = false;
     size_t bytes = (size_t)STAGES * (BM + BN) * 128;
     if (!configured) {
@@ -800,7 +801,7 @@ static int launch_dma(hipStream_t stream, const bf16* A, int lda, const bf16* W,
     if (grid.y > 65535) return llmrs_fail("gemm: M=%d is too large for one launch", M);
     gemm_dma_kernel<BM, BN, WGM, WGN, STAGES><<<grid, 64 * WGM * WGN, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi,
                                                                                       splits > 1 ? partial : nullptr);
-    if (splits > 1) launch_splitk_finish(stream, partial, splits, out, ldc, M, N, epi, next);
+    if (splits > 1 && finish) launch_splitk_finish(stream, partial, splits, out, ldc, M, N, epi, next);
     return 0;
 }
 
@@ -1270,9 +1271,10 @@ static int tiled_splits(int M, int N, int K) {
 }
 // The 128 x 128 tiles of a product, in whichever of the two forms its shape asks for.
 static int launch_tiles_128(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,
-                            int M, int N, int K, int epi, int splits, float* partial, const NextNorm* next = nullptr) {
-    if (deep_tiles(M, N, K)) return launch_dma<128, 128, 2, 4, 4>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next);
-    return launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next);
+                            int M, int N, int K, int epi, int splits, float* partial, const NextNorm* next = nullptr,
+                            bool finish = true) {
+    if (deep_tiles(M, N, K)) return launch_dma<128, 128, 2, 4, 4>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next, finish);
+    return launch_dma<128, 128, 2, 2, 2>(stream, A, lda, W, out, ldc, M, N, K, epi, splits, partial, next, finish);
 }
 // 17..64 rows on a weight of middling width (more than 4096 features, fewer than the wide ones that
 // get blocks of many feature tiles): the 128 x 128 tiles with k split over blocks read the tokens'
@@ -1328,6 +1330,22 @@ extern "C" int llmrs_gemm_next_parts(int M, int N, int K) {
 // 17 to 256 rows whose sums are split over blocks: the kernel that adds the parts up can finish the following norm.
 extern "C" int llmrs_gemm_norms_whole(int M, int N, int K) {
     return M > 16 && M <= 256 && N >= 4 && N % 4 == 0 && N <= 16384 && K % 8 == 0 && llmrs_gemm_workspace_floats(M, N, K) > 0;
+}
+
+// The product as parts of its sum over k, [parts][M][N] 32-bit in `workspace`, for a caller that adds them up itself
+// (the rotation and cache write after the q/k/v product does, and saves the kernel that would): only where this
+// file would split such a product over blocks anyway.  Returns the number of parts, 0 when the product is not
+// one of those (nothing was launched), -1 on error.
+int llmrs_gemm_bf16_split_parts(hipStream_t stream, const bf16* A, int lda, const bf16* W, int M, int N, int K,
+                                void* workspace, size_t workspace_bytes) {
+    if (K % 64 || lda % 8 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || workspace == nullptr || M > 512) return 0;
+    const bool tiles = M > 64 ? !((long)ceil_div(M, 256) * ceil_div(N, 256) >= 160 && M > 128) : few_rows_take_tiles(M, N, K);
+    int splits = tiles ? tiled_splits(M, N, K) : 1;
+    if (splits <= 1 || workspace_bytes < (size_t)splits * M * N * sizeof(float)) return 0;
+    if (launch_tiles_128(stream, A, lda, W, nullptr, N, M, N, K, LLMRS_EPI_STORE, splits, (float*)workspace, nullptr, false) != 0) return -1;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { llmrs_fail("gemm (mfma): launch failed: %s", hipGetErrorString(e)); return -1; }
+    return splits;
 }
 
 int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16* W, void* out, int ldc,

@@ -18,6 +18,10 @@ struct RopeKvArgs {
     int page_size, write_kv, num_pages;
     int row_stride;  // elements between tokens in qkv
     int value_pages; // the values of a page that 16 tokens fill in order are written whole, a kv head by each token's block
+    // The projection's output still as the parts of its sum over k ([n_parts][n_tokens][n_cols], 32-bit), when the
+    // product before was split over blocks and left the adding up to this kernel (null: the rows are in qkv).
+    const float* parts;
+    int n_parts, n_cols;
 };
 
 template <class T>
@@ -88,6 +92,24 @@ __device__ __forceinline__ bool first_lanes_see_whole_page(const int* __restrict
     return (__ballot(mine) & 0xffffull) == 0xffffull;
 }
 
+// Eight values of token t's row from column col on: from qkv, or added up from the parts of a split product, in
+// the parts' order and rounded to 16 bits as the kernel that adds parts up rounds them (the same bits either way).
+__device__ __forceinline__ rope_bf16x8 row_values(const bf16* __restrict__ qkv, int t, int col, const RopeKvArgs& a) {
+    if (a.parts == nullptr) return *(const rope_bf16x8*)(qkv + (size_t)t * a.row_stride + col);
+    const float* p = a.parts + (size_t)t * a.n_cols + col;
+    size_t part = (size_t)a.n_tokens * a.n_cols;
+    float4 lo = *(const float4*)p, hi = *(const float4*)(p + 4);
+    for (int s = 1; s < a.n_parts; ++s) {
+        float4 l2 = *(const float4*)(p + s * part), h2 = *(const float4*)(p + s * part + 4);
+        lo.x += l2.x; lo.y += l2.y; lo.z += l2.z; lo.w += l2.w;
+        hi.x += h2.x; hi.y += h2.y; hi.z += h2.z; hi.w += h2.w;
+    }
+    rope_bf16x8 v;
+    v[0] = (bf16)lo.x; v[1] = (bf16)lo.y; v[2] = (bf16)lo.z; v[3] = (bf16)lo.w;
+    v[4] = (bf16)hi.x; v[5] = (bf16)hi.y; v[6] = (bf16)hi.z; v[7] = (bf16)hi.w;
+    return v;
+}
+
 // The values of 16 tokens that fill a page, for the kv heads first, first + 16, ...: [16 tokens][head_dim] in,
 // [head_dim][16 slots] out, by all threads of a block, through `tile` ([16][head_dim + 8] in LDS).
 __device__ __forceinline__ void write_value_page(const bf16* __restrict__ qkv, const int* __restrict__ slot_map,
@@ -96,10 +118,10 @@ __device__ __forceinline__ void write_value_page(const bf16* __restrict__ qkv, c
     int hd = a.head_dim, ld = hd + 8, chunks = hd / 8;       // rows 16 bytes apart in banks
     int page = slot_map[t16] / 16;
     for (int kvh = first; kvh < a.n_kv_heads; kvh += 16) {
-        const bf16* src = qkv + (size_t)t16 * a.row_stride + (size_t)(a.n_heads + a.n_kv_heads + kvh) * hd;
+        int col = (a.n_heads + a.n_kv_heads + kvh) * hd;
         for (int c = threadIdx.x; c < 16 * chunks; c += blockDim.x) {
             int j = c / chunks, d0 = (c % chunks) * 8;
-            *(rope_bf16x8*)(tile + j * ld + d0) = *(const rope_bf16x8*)(src + (size_t)j * a.row_stride + d0);
+            *(rope_bf16x8*)(tile + j * ld + d0) = row_values(qkv, t16 + j, col + d0, a);
         }
         __syncthreads();
         bf16* dst = v_cache + v_cache_index(page, kvh, 0, 0, a.n_kv_heads, 16, hd);     // this page and head: [hd][16], contiguous
@@ -148,7 +170,7 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
         bool is_q = ch < q_chunks, is_k = !is_q && head < a.n_heads + a.n_kv_heads;
         if (!is_q && !cache_ok) continue;
         if (!is_q && !is_k && values_elsewhere) continue;
-        rope_bf16x8 v = *(const rope_bf16x8*)(row + (size_t)head * a.head_dim + d0);
+        rope_bf16x8 v = row_values(qkv, t, head * a.head_dim + d0, a);
         if ((is_q || is_k) && d0 < a.rotary_dim) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -174,6 +196,19 @@ __global__ __launch_bounds__(256) void rope_kv_rows_kernel(bf16* __restrict__ qk
         write_value_page(qkv, slot_map, v_cache, (bf16*)(cs + (a.rotary_dim / 2 + 1) / 2 * 2), t & ~15, t & 15, a);
 }
 
+// Whether the kernel above (16-bit rows, pairs that are neighbours) takes these rows.
+static bool rows_kernel_takes(const void* qkv, int row_stride, const void* k_cache, int n_tokens, int head_dim, int rotary_dim) {
+    return n_tokens >= 16 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0 &&
+           ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && rotary_dim / 2 * sizeof(float2) <= 32768;
+}
+static void launch_rope_rows(hipStream_t stream, bf16* qkv, const int* positions, const int* slot_map, const float* inv_freq,
+                             bf16* k_cache, bf16* v_cache, RopeKvArgs a) {
+    a.value_pages = a.write_kv && a.page_size == 16 && a.n_kv_heads > 0 && ((uintptr_t)v_cache & 15) == 0 &&
+                    (size_t)16 * (a.head_dim + 8) * 2 <= 32768;
+    size_t smem = (size_t)(a.rotary_dim / 2 + 1) / 2 * 2 * sizeof(float2) + (a.value_pages ? (size_t)16 * (a.head_dim + 8) * 2 : 0);
+    rope_kv_rows_kernel<<<a.n_tokens, 256, smem, stream>>>(qkv, positions, slot_map, inv_freq, k_cache, v_cache, a);
+}
+
 // qkv: [n_tokens, row_stride], a row is q heads, then k heads, then v heads.
 // q is rotated in place; k is rotated and written to k_cache; v is copied to
 // v_cache.  Slots outside [0, num_pages * page_size) are skipped.
@@ -188,20 +223,14 @@ extern "C" int llmrs_rope_kv_write(hipStream_t stream, int dtype, void* qkv, int
     LLMRS_REQUIRE(row_stride >= (n_heads + 2 * n_kv_heads) * head_dim, "rope_kv_write: row stride %d too short", row_stride);
     LLMRS_REQUIRE(page_size > 0, "rope_kv_write: page_size %d", page_size);
     if (n_tokens == 0) return 0;
-    RopeKvArgs a{n_tokens, n_heads, n_kv_heads, head_dim, rotary_dim, interleaved, page_size, write_kv, num_pages, row_stride, 0};
+    RopeKvArgs a{n_tokens, n_heads, n_kv_heads, head_dim, rotary_dim, interleaved, page_size, write_kv, num_pages, row_stride, 0,
+                 nullptr, 0, 0};
     int pairs = (n_heads + 2 * n_kv_heads) * (head_dim / 2);
     dim3 grid(n_tokens, ceil_div(pairs, 256));
     if (dtype == LLMRS_F32)
         rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, positions, slot_map, inv_freq, (float*)k_cache, (float*)v_cache, a);
-    else if (dtype == LLMRS_BF16 && interleaved && n_tokens >= 16 && head_dim % 8 == 0 && rotary_dim % 8 == 0 && row_stride % 8 == 0 &&
-             ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)k_cache & 15) == 0 && rotary_dim / 2 * sizeof(float2) <= 32768)
-    {
-        a.value_pages = write_kv && page_size == 16 && n_kv_heads > 0 && ((uintptr_t)v_cache & 15) == 0 &&
-                        (size_t)16 * (head_dim + 8) * 2 <= 32768;
-        size_t smem = (size_t)(rotary_dim / 2 + 1) / 2 * 2 * sizeof(float2) + (a.value_pages ? (size_t)16 * (head_dim + 8) * 2 : 0);
-        rope_kv_rows_kernel<<<n_tokens, 256, smem, stream>>>((bf16*)qkv, positions, slot_map, inv_freq,
-                                                             (bf16*)k_cache, (bf16*)v_cache, a);
-    }
+    else if (dtype == LLMRS_BF16 && interleaved && rows_kernel_takes(qkv, row_stride, k_cache, n_tokens, head_dim, rotary_dim))
+        launch_rope_rows(stream, (bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
     else if (dtype == LLMRS_BF16)
         rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
     else
@@ -240,6 +269,20 @@ extern "C" int llmrs_qkv_rope_cache(hipStream_t stream, int dtype, const void* x
         int took = llmrs_gemm_bf16_mfma(stream, (const bf16*)x, lda, (const bf16*)w, qkv, row_stride, M, N, K,
                                         LLMRS_EPI_QKV, nullptr, 0, &qe, scale_sumsq ? &rs : nullptr);
         if (took != 0) return took < 0 ? -1 : 0;
+        // A product that is split over blocks along k (65 to 512 rows, and some shapes from 17 rows on) leaves its parts:
+        // the rotation kernel adds them up as it reads its rows, and the kernel that would do that is saved.
+        if (scale_sumsq == nullptr && rows_kernel_takes(qkv, row_stride, k_cache, M, head_dim, rotary_dim) &&
+            ((uintptr_t)workspace & 15) == 0 && N % 8 == 0) {
+            int parts = llmrs_gemm_bf16_split_parts(stream, (const bf16*)x, lda, (const bf16*)w, M, N, K, workspace, workspace_bytes);
+            if (parts < 0) return -1;
+            if (parts > 1) {
+                RopeKvArgs a{M, n_heads, n_kv_heads, head_dim, rotary_dim, 1, page_size, write_kv, num_pages, row_stride, 0,
+                             (const float*)workspace, parts, N};
+                launch_rope_rows(stream, (bf16*)qkv, positions, slot_map, inv_freq, (bf16*)k_cache, (bf16*)v_cache, a);
+                LLMRS_LAUNCH_CHECK("qkv_rope_cache");
+                return 0;
+            }
+        }
     }
     LLMRS_REQUIRE(scale_sumsq == nullptr, "qkv_rope_cache: a deferred norm needs the fused bfloat16 kernel (M=%d K=%d)", M, K);
     int rc = llmrs_gemm(stream, dtype, x, lda, w, qkv, row_stride, M, N, K, LLMRS_EPI_STORE, workspace, workspace_bytes,

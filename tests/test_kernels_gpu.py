@@ -796,6 +796,59 @@ def test_qkv_rope_cache(dtype, M, n_heads, n_kv, hd, rot, K):
     assert (qkv[:, N:] == 0).all(), "padding touched"
 
 
+@pytest.mark.parametrize("M,n_heads,n_kv,hd,rot,K", [(100, 32, 8, 128, 128, 4096), (300, 16, 4, 64, 64, 2048), (64, 36, 2, 128, 128, 8192),
+                                                    (200, 8, 8, 128, 64, 2048), (512, 32, 8, 64, 64, 2048), (65, 32, 8, 128, 128, 4096)])
+def test_qkv_rope_cache_adds_up_a_split_product(M, n_heads, n_kv, hd, rot, K):
+    """With 65 to 512 rows (and long rows from 33 on) the product is split over blocks along k and leaves the parts
+    of its sums; the rotation kernel adds them up as it reads its rows.  The first 48 tokens fill three pages in
+    order (their values are written page-wise, through LDS), the rest lie scattered."""
+    page_size, num_pages = 16, 40
+    N = (n_heads + 2 * n_kv) * hd
+    k = kernels()
+    n_ws = k.gemm_workspace_floats(M, N, K)
+    assert n_ws >= 2 * M * N, "the case itself: a product that is split"
+    x = rnd((M, K), torch.bfloat16, 30)
+    w = rnd((N, K), torch.bfloat16, 31, 0.1)
+    positions = torch.randint(0, 400, (M,), generator=torch.Generator().manual_seed(32)).to(torch.int32).to(DEV)
+    pages = torch.randperm(num_pages, generator=torch.Generator().manual_seed(33)).tolist()
+    in_order = [pages[i] * 16 + j for i in range(3) for j in range(16)]
+    rest = [pg * 16 + j for pg in pages[3:] for j in range(16)]
+    rest = [rest[i] for i in torch.randperm(len(rest), generator=torch.Generator().manual_seed(34)).tolist()]
+    slots = torch.tensor((in_order + rest)[:M], dtype=torch.int32, device=DEV)
+    inv_freq = plain_inv_freq(rot, 10000.0, None).to(DEV)
+    qkv = torch.zeros((M, N + 8), dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros((num_pages, n_kv, page_size, hd), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros((num_pages, n_kv, hd, page_size), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(n_ws, dtype=torch.float32, device=DEV)
+    k.qkv_rope_cache(x, w, qkv[:, :N], positions, slots, inv_freq, rot, kc, vc, n_heads, n_kv, hd, page_size, num_pages, True, ws)
+    acc = x.double().cpu() @ w.double().cpu().T
+    q = plain_rope(acc[:, :n_heads * hd].view(M, n_heads, hd), positions.cpu(), inv_freq.cpu(), "interleaved")
+    kk = plain_rope(acc[:, n_heads * hd:(n_heads + n_kv) * hd].view(M, n_kv, hd), positions.cpu(), inv_freq.cpu(), "interleaved")
+    v = acc[:, (n_heads + n_kv) * hd:].view(M, n_kv, hd)
+    page, off = (slots // page_size).long().cpu(), (slots % page_size).long().cpu()
+    got_q = qkv[:, :n_heads * hd].double().cpu().view(M, n_heads, hd)
+    got_k = kc.double().cpu()[page, :, off, :]
+    got_v = vc.double().cpu()[page, :, :, off]
+    for name, got, ref in (("q", got_q, q), ("k", got_k, kk), ("v", got_v, v)):
+        err = (got - ref).abs()
+        size = ref.abs()
+        if name != "v":
+            pair = ref[..., :rot].unflatten(-1, (rot // 2, 2)).norm(dim=-1, keepdim=True).expand(-1, -1, -1, 2).flatten(-2)
+            size = torch.cat([pair, size[..., rot:]], dim=-1)
+        assert (err <= size / 40 + 2e-2).all(), f"{name}: max err {float(err.max())}"
+    assert (qkv[:, N:] == 0).all(), "padding touched"
+    written = torch.zeros(num_pages * page_size, dtype=torch.bool)
+    written[slots.long().cpu()] = True
+    assert (kc.cpu().permute(0, 2, 1, 3).reshape(num_pages * page_size, -1)[~written] == 0).all(), "a slot that no token maps to was written"
+    assert (vc.cpu().permute(0, 3, 1, 2).reshape(num_pages * page_size, -1)[~written] == 0).all(), "a slot that no token maps to was written"
+    # the same call with room for nothing: product, then rotation, each a kernel of its own; the same results to rounding
+    qkv2, kc2, vc2 = torch.zeros_like(qkv), torch.zeros_like(kc), torch.zeros_like(vc)
+    k.qkv_rope_cache(x, w, qkv2[:, :N], positions, slots, inv_freq, rot, kc2, vc2, n_heads, n_kv, hd, page_size, num_pages, True)
+    scale = float(acc.abs().max())
+    assert (qkv2[:, :n_heads * hd].float() - qkv[:, :n_heads * hd].float()).abs().max() <= scale / 64
+    assert (kc2.float() - kc.float()).abs().max() <= scale / 64 and (vc2.float() - vc.float()).abs().max() <= scale / 64
+
+
 # ---- utilities ----------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", DTYPES)
