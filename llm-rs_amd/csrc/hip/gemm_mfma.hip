@@ -1327,9 +1327,13 @@ static bool half_blocks_for_narrow(int N, int K) {
 extern "C" int llmrs_gemm_next_parts(int M, int N, int K) {
     return M <= 16 && half_blocks_for_narrow(N, K) ? ceil_div(N, 8) : ceil_div(N, 16);
 }
-// 17 to 256 rows whose sums are split over blocks: the kernel that adds the parts up can finish the following norm.
+// 17 rows or more whose sums are split over blocks: the kernel that adds the parts up can finish the following norm.
+// (Beyond 256 rows that is where the 128 x 128 tiles take all rows with k split: a narrow weight whose tiles leave
+// half of the device's places empty, as the o and down products of a small model do beside a prompt portion.)
 extern "C" int llmrs_gemm_norms_whole(int M, int N, int K) {
-    return M > 16 && M <= 256 && N >= 4 && N % 4 == 0 && N <= 16384 && K % 8 == 0 && llmrs_gemm_workspace_floats(M, N, K) > 0;
+    if (!(M > 16 && N >= 4 && N % 4 == 0 && N <= 16384 && K % 8 == 0)) return 0;
+    if (M <= 256) return llmrs_gemm_workspace_floats(M, N, K) > 0;
+    return K % 64 == 0 && (long)ceil_div(M, 256) * ceil_div(N, 256) < 160 && tiled_splits(M, N, K) > 1;
 }
 
 // The product as parts of its sum over k, [parts][M][N] 32-bit in `workspace`, for a caller that adds them up itself
@@ -1361,7 +1365,7 @@ int llmrs_gemm_bf16_mfma(hipStream_t stream, const bf16* A, int lda, const bf16*
                   workspace_bytes >= (size_t)llmrs_gemm_workspace_floats(M, N, K) * sizeof(float) && next->y != nullptr &&
                   next->weight != nullptr && next->ldy >= N && next->ldy % 4 == 0 && ((uintptr_t)next->y & 7) == 0 &&
                   ((uintptr_t)next->weight & 15) == 0 && ldc % 4 == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)workspace & 15) == 0;
-        if (!ok) { llmrs_fail("gemm: a norm finished by a split product needs the += epilogue, 17 to 256 rows of a shape that is split, its workspace and aligned rows, got M=%d N=%d K=%d epilogue %d", M, N, K, epi); return -1; }
+        if (!ok) { llmrs_fail("gemm: a norm finished by a split product needs the += epilogue, 17 rows or more of a shape that is split, its workspace and aligned rows, got M=%d N=%d K=%d epilogue %d", M, N, K, epi); return -1; }
     } else if (scale != nullptr || next != nullptr) {
         bool ok = llmrs_gemm_defers_norm(M, N, K) && (scale == nullptr || (scale->sumsq != nullptr && scale->nparts >= 1 && scale->eps > 0.0f)) &&
                   (next == nullptr || (epi == LLMRS_EPI_ACCUM_F32 && N < 16384 && next->sumsq != nullptr && next->y != nullptr &&

@@ -50,7 +50,7 @@ class NextNorm:
     """What a product that adds into the stream leaves for the norm that follows, see `NormedRows`:
     `y` and `sumsq` to fill, `weight` the following norm's.  With `eps` (and no `sumsq`) the product finishes the
     norm itself: `y` becomes the normed rows, for any product to take as they are (`gemm_norms_whole`: steps of
-    17 to 256 tokens whose product is split over blocks, where the kernel that adds the parts up sees whole rows)."""
+    17 tokens or more whose product is split over blocks, where the kernel that adds the parts up sees whole rows)."""
 
     def __init__(self, y: torch.Tensor, sumsq: Optional[torch.Tensor], weight: torch.Tensor, eps: float = 0.0):
         self.y, self.sumsq, self.weight, self.eps = y, sumsq, weight, float(eps)

@@ -1017,9 +1017,10 @@ def test_a_norm_left_by_one_product_and_finished_by_the_next(M, hidden, inter):
 
 
 @pytest.mark.parametrize("M,N,K", [(64, 4096, 4096), (17, 4096, 14336), (24, 1024, 2048), (33, 2048, 8192), (200, 512, 4096),
-                                   (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192), (45, 4096, 4096)])
+                                   (128, 4096, 4096), (256, 1000, 2048), (40, 6144, 4096), (64, 8192, 8192), (45, 4096, 4096),
+                                   (2030, 2048, 2048), (1900, 2048, 8192), (700, 4096, 4096), (300, 1000, 2048)])
 def test_split_residual_product_finishes_the_next_norm(M, N, K):
-    """17 to 256 rows, a product whose sums are split over blocks: the kernel that adds the parts writes the stream and
+    """17 rows or more, a product whose sums are split over blocks: the kernel that adds the parts writes the stream and
     the normed rows: the stream bit for bit as without, the rows as the norm kernel makes them from that stream."""
     from llm_rs_amd.kernels import NextNorm
     k = kernels()
