@@ -44,6 +44,8 @@ def _lib():
             "llmrs_sched_plan": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
             "llmrs_sched_build": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
             "llmrs_sched_commit": [c_void_p, c_void_p, c_int, c_void_p, c_int],
+            "llmrs_sched_plan_sources": [c_void_p, c_void_p, c_int], "llmrs_sched_launch": [c_void_p],
+            "llmrs_sched_in_flight": [c_void_p],
             "llmrs_request_info": [c_void_p, c_int, c_void_p],
             "llmrs_request_output": [c_void_p, c_int, c_void_p, c_int],
             "llmrs_request_drop": [c_void_p, c_int],
@@ -182,6 +184,20 @@ class HostCore:
         a = [np.zeros(cap, dtype=np.int32) for _ in range(4)]
         n = self._check(self._lib.llmrs_sched_plan(self._h, *(_ptr(x) for x in a), cap))
         return [(int(a[0][i]), int(a[1][i]), int(a[2][i]), bool(a[3][i])) for i in range(n)]
+
+    def plan_sources(self) -> List[int]:
+        """For each entry of the plan: the row of the step in flight whose sample is the entry's one token, or -1."""
+        src = np.zeros(self.max_requests, dtype=np.int32)
+        n = self._check(self._lib.llmrs_sched_plan_sources(self._h, _ptr(src), src.size))
+        return src[:n].tolist()
+
+    def launch(self) -> None:
+        """The planned step has been started: `plan()` may be called for the step after it, before `commit()`
+        lands this one."""
+        self._check(self._lib.llmrs_sched_launch(self._h))
+
+    def in_flight(self) -> bool:
+        return bool(self._lib.llmrs_sched_in_flight(self._h))
 
     def build_planned(self, words: np.ndarray, fixed_widths=None):
         """Flatten the planned step; returns (offsets, n_tokens, n_sampling_rows)."""

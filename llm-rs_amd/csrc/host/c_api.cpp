@@ -165,6 +165,28 @@ int llmrs_sched_plan(void* h, int32_t* slots, int32_t* starts, int32_t* counts, 
     });
 }
 
+// For each entry of the plan the row of the step in flight whose sample is its one token, or -1.  Returns R.
+int llmrs_sched_plan_sources(void* h, int32_t* sources, int cap) {
+    auto c = (Core*)h;
+    return guarded(c, [&] {
+        const auto& plan = c->scheduler->planned();
+        if ((int)plan.size() > cap) throw std::invalid_argument("plan larger than the caller's buffer");
+        for (size_t i = 0; i < plan.size(); ++i) sources[i] = plan[i].pending_src;
+        return (int)plan.size();
+    });
+}
+
+// The planned step has been started on the device; the next one may be planned before it is committed.
+int llmrs_sched_launch(void* h) {
+    auto c = (Core*)h;
+    return guarded(c, [&] {
+        c->scheduler->launch();
+        return 0;
+    });
+}
+
+int llmrs_sched_in_flight(void* h) { return ((Core*)h)->scheduler->in_flight() ? 1 : 0; }
+
 // Writes the planned step's batch.  Returns the words used; n_tokens_out and
 // n_want_out get the step's tokens and the number of rows that sample.
 int llmrs_sched_build(void* h, const int32_t* fixed_widths, int32_t* words, int cap_words, int32_t* offsets_out,

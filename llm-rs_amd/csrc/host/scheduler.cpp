@@ -78,6 +78,7 @@ void Scheduler::preempt_last() {
 }
 
 const std::vector<PlannedEntry>& Scheduler::plan() {
+    const bool ahead = in_flight();
     for (;;) {
         plan_.clear();
         int budget = budget_;
@@ -86,13 +87,19 @@ const std::vector<PlannedEntry>& Scheduler::plan() {
         for (int slot : running_) {
             if (budget == 0) break;
             Request& r = requests_[slot];
-            int n = portion(r, budget);
+            int n = portion(r, budget), src = -1;
+            if (r.pending_row >= 0) {
+                // its next token is being sampled: one token, unless that one is its last
+                if (r.generated() + 1 >= r.max_new) continue;
+                n = 1;
+                src = r.pending_row;
+            }
             if (n <= 0) continue;
             if (!cache_.ensure(slot, r.computed, n)) {
                 starved = true;
                 continue;  // no pages now; it tries again in the next step
             }
-            plan_.push_back({{slot, r.computed, n}, r.computed + n == (int)r.tokens.size()});
+            plan_.push_back({{slot, r.computed, n}, src >= 0 || r.computed + n == (int)r.tokens.size(), src});
             budget -= n;
         }
         // 2. waiting requests, first in first out (scheduler.rs:56-73)
@@ -110,7 +117,7 @@ const std::vector<PlannedEntry>& Scheduler::plan() {
             plan_.push_back({{slot, r.computed, n}, r.computed + n == (int)r.tokens.size()});
             budget -= n;
         }
-        if (!plan_.empty() || !starved) return plan_;
+        if (!plan_.empty() || !starved || ahead) return plan_;   // (ahead of a step in flight nobody is preempted)
         // Nothing can advance and pages are the reason.  With nobody running, the
         // head of the queue found an empty pool too small: add() rules that out.
         if (running_.empty())
@@ -126,7 +133,8 @@ void Scheduler::plan_tokens(std::vector<int32_t>& tokens, std::vector<int32_t>& 
     sampling_words.clear();
     for (const auto& p : plan_) {
         Request& r = requests_[p.entry.slot];
-        tokens.insert(tokens.end(), r.tokens.begin() + p.entry.start, r.tokens.begin() + p.entry.start + p.entry.count);
+        if (p.pending_src >= 0) tokens.push_back(0);     // the device puts the step in flight's sample here
+        else tokens.insert(tokens.end(), r.tokens.begin() + p.entry.start, r.tokens.begin() + p.entry.start + p.entry.count);
         if (!p.samples) continue;
         want_rows.push_back((int32_t)tokens.size() - 1);
         float u = r.sampling.temperature > 0.0f ? r.rng.next_f32() : 0.0f;
@@ -139,15 +147,37 @@ void Scheduler::plan_tokens(std::vector<int32_t>& tokens, std::vector<int32_t>& 
     }
 }
 
-std::vector<int> Scheduler::commit(const int32_t* sampled, int n_sampled) {
-    std::vector<int> finished;
-    int i = 0;
+void Scheduler::launch() {
+    if (in_flight()) throw std::logic_error("a step is in flight already: commit it first");
+    int row = 0;
     for (const auto& p : plan_) {
+        if (p.samples) ++row;
+        if (p.dead) continue;
         Request& r = requests_[p.entry.slot];
         r.computed += p.entry.count;
+        if (p.samples) r.pending_row = row - 1;
+    }
+    flight_.swap(plan_);
+    plan_.clear();
+}
+
+std::vector<int> Scheduler::commit(const int32_t* sampled, int n_sampled) {
+    std::vector<int> finished;
+    const bool launched = in_flight();
+    std::vector<PlannedEntry> step;
+    step.swap(launched ? flight_ : plan_);
+    int i = 0;
+    for (const auto& p : step) {
+        if (p.dead) {
+            if (p.samples) ++i;
+            continue;
+        }
+        Request& r = requests_[p.entry.slot];
+        if (!launched) r.computed += p.entry.count;
         if (!p.samples) continue;  // a portion of a prompt: nothing to sample yet (engine.rs:209)
         if (i >= n_sampled) throw std::invalid_argument("fewer sampled tokens than entries that sample");
         int32_t token = sampled[i++];
+        r.pending_row = -1;
         if (std::find(r.stop.begin(), r.stop.end(), token) != r.stop.end()) {
             r.finish = Finish::Stop;  // the stop token itself is not part of the output (engine.rs:214-216)
         } else {
@@ -159,10 +189,14 @@ std::vector<int> Scheduler::commit(const int32_t* sampled, int n_sampled) {
             cache_.release_pages(p.entry.slot);
             running_.erase(std::remove(running_.begin(), running_.end(), p.entry.slot), running_.end());
             finished.push_back(p.entry.slot);
+            // what the step ahead runs for it (one token past a stop token) is for nothing
+            if (launched)
+                for (auto& q : plan_)
+                    if (q.entry.slot == p.entry.slot) q.dead = true;
         }
     }
     if (i != n_sampled) throw std::invalid_argument("more sampled tokens than entries that sample");
-    plan_.clear();
+    if (!launched) plan_.clear();
     return finished;
 }
 
@@ -173,6 +207,8 @@ void Scheduler::abort(int slot) {
     waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), slot), waiting_.end());
     plan_.erase(std::remove_if(plan_.begin(), plan_.end(), [&](const PlannedEntry& p) { return p.entry.slot == slot; }),
                 plan_.end());
+    for (auto& p : flight_)             // the step in flight keeps its rows: the entry's sample is dropped
+        if (p.entry.slot == slot) p.dead = true;
     requests_[slot] = Request();
     cache_.release_slot(slot);
 }

@@ -15,6 +15,17 @@
 // back and goes to the front of the waiting queue, to be computed again from its
 // prompt and what it has generated.  Its generator state stays, so its output
 // does not change.
+//
+// One step ahead.  A caller that has started a step on the device may say so
+// (launch()) and plan the next one before the first one's sampled tokens are
+// back: a request whose next token is being sampled gets an entry of one token
+// that names the row of the step in flight where that token will stand, and the
+// device hands it over without the host.  What cannot be known yet is left to
+// turn out: a request that ends on a stop token has run one token for nothing,
+// its entry in the step ahead is marked dead and its sample dropped.  Nothing is
+// preempted while a step is in flight; a plan that finds no pages comes back
+// empty and the caller commits the step in flight first.  Tokens, their order
+// and each request's random draws are the same as without.
 #pragma once
 #include <cstdint>
 #include <deque>
@@ -47,12 +58,15 @@ struct Request {
     Phase phase = Phase::Free;
     Finish finish = Finish::None;
     int preemptions = 0;
+    int pending_row = -1;         // >= 0: the step in flight samples its next token, in that row of its samples
     int generated() const { return (int)tokens.size() - prompt_len; }
 };
 
 struct PlannedEntry {
     BatchEntry entry;
-    bool samples;  // the portion ends at the request's last known token
+    bool samples;          // the portion ends at the request's last known token
+    int pending_src = -1;  // >= 0: the entry's one token is the sample in that row of the step in flight
+    bool dead = false;     // its request ended after the step was started: nothing of it counts
 };
 
 class Scheduler {
@@ -77,7 +91,12 @@ public:
                      std::vector<int32_t>& sampling_words);
     // Takes the sampled token of each entry that samples, in plan order; returns
     // the slots that finished (their pages are back; the slot stays until drop()).
+    // (With a step in flight: that step's.)
     std::vector<int> commit(const int32_t* sampled, int n_sampled);
+    // The planned step has been started on the device: plan() may be called for the step after it.
+    // One step can be in flight; commit() lands it.
+    void launch();
+    bool in_flight() const { return !flight_.empty(); }
 
     const Request& request(int slot) const { return requests_[slot]; }
     void drop(int slot);  // forget a finished request, free its slot
@@ -96,6 +115,7 @@ private:
     std::vector<int> running_;       // admission order
     std::deque<int> waiting_;
     std::vector<PlannedEntry> plan_;
+    std::vector<PlannedEntry> flight_;   // the step that was started and has not been committed
     int64_t preemptions_ = 0;
 };
 

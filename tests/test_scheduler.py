@@ -276,3 +276,131 @@ def test_check_request_changes_nothing():
         core.check_request(18, 4)
     core.check_request(10, 4)
     assert core.idle() and core.slots_in_use() == 0 and core.pages_free() == 5
+
+
+class AheadDriver:
+    """The loop of a caller that keeps one step in flight: a step is started (its samples are not known to the
+    scheduler yet), the next one is planned and started, then the first one's samples are committed.  The stand-in
+    device puts a sample of the step in flight where the plan ahead names it."""
+
+    def __init__(self, core):
+        self.core, self.words = core, np.zeros(1 << 16, dtype=np.int32)
+        self.seen = {}            # slot -> tokens fed so far
+        self.flight = None        # samples of the step in flight
+        self.wasted = 0           # tokens run for a request that had ended
+
+    def start(self):
+        """Plans and 'runs' a step; returns its samples, or None when nothing could be planned."""
+        core = self.core
+        plan = core.plan()
+        if not plan:
+            return None
+        sources = core.plan_sources()
+        off, T, n_want = core.build_planned(self.words)
+        toks = self.words[off.tokens:off.tokens + T].tolist()
+        sampled, at = [], 0
+        for (slot, start, count, samples), src in zip(plan, sources):
+            if src >= 0:
+                assert count == 1 and samples and self.flight is not None
+                toks[at] = self.flight[src]                 # what the device does
+            if start == 0:
+                self.seen[slot] = []
+            assert len(self.seen[slot]) == start, "a portion must start where the cache ends"
+            self.seen[slot] = self.seen[slot] + toks[at:at + count]
+            at += count
+            if samples:
+                sampled.append(next_token(self.seen[slot]))
+        return sampled
+
+    def step(self):
+        """One turn of the loop; returns the slots that finished."""
+        core = self.core
+        if self.flight is None:
+            self.flight = self.start()
+            if self.flight is None:
+                return []
+            core.launch()
+        ahead = self.start()                                   # before the step in flight is committed
+        finished = core.commit(self.flight)
+        self.flight = ahead
+        if ahead is not None:
+            core.launch()
+        return finished
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_one_step_ahead_gives_the_same_outputs(seed):
+    """Random load, small pool, stop tokens: with a step in flight while the next is planned every request's output
+    and finish reason are what it gets alone; no page is lost; a request that ends on a stop token costs one token
+    run for nothing and no more."""
+    rng = np.random.default_rng(100 + seed)
+    pages = 16
+    core = HostCore([(4, pages, 0)], max_requests=5, token_budget=int(rng.integers(8, 40)), max_chunk=int(rng.integers(0, 9)))
+    n = 14
+    prompts = [rng.integers(0, 50, int(rng.integers(1, 25))).tolist() for _ in range(n)]
+    news = [int(rng.integers(1, 14)) for _ in prompts]
+    stops = [rng.integers(0, 97, int(rng.integers(0, 12))).tolist() for _ in prompts]
+    d, slots, pending, done = AheadDriver(core), {}, list(range(n)), {}
+    for _ in range(5000):
+        while pending:
+            s = core.add_request(prompts[pending[0]], news[pending[0]], stop=stops[pending[0]])
+            if s < 0:
+                break
+            slots[s] = pending.pop(0)
+        if core.idle() and not pending and d.flight is None:
+            break
+        for s in d.step():
+            info = core.request_info(s)
+            done[slots.pop(s)] = (core.request_output(s), "stop" if info["finish"] == 1 else "length")
+            core.drop_request(s)
+        held = sum(core.pages_held(s) for s in slots)
+        assert held + core.pages_free() == pages
+    assert sorted(done) == list(range(n))
+    for i in range(n):
+        assert done[i] == alone(prompts[i], news[i], stops[i]), f"request {i}"
+    assert core.pages_free() == pages and not core.in_flight()
+
+
+def test_one_step_ahead_plans_the_token_in_flight_and_drops_what_a_stop_wasted():
+    core = HostCore([(4, 20, 0)], max_requests=3, token_budget=16)
+    first = next_token([1, 2, 3])
+    a = core.add_request([1, 2, 3], 5, stop=[next_token([1, 2, 3, first])])      # ends on its second sample
+    b = core.add_request([4, 5], 1)                                              # its first sample is its last
+    assert core.plan() == [(a, 0, 3, True), (b, 0, 2, True)]
+    assert core.plan_sources() == [-1, -1]
+    words = np.zeros(4096, dtype=np.int32)
+    core.build_planned(words)
+    core.launch()
+    assert core.in_flight()
+    # ahead: a's next token is row 0 of the step in flight; b is not planned, the token in flight is its last
+    assert core.plan() == [(a, 3, 1, True)] and core.plan_sources() == [0]
+    off, T, n_want = core.build_planned(words)
+    assert (T, n_want) == (1, 1)
+    assert core.commit([first, 9]) == [b]
+    assert core.request_output(b) == [9]
+    core.drop_request(b)
+    core.launch()
+    # the step after: a's second sample is in flight
+    assert core.plan() == [(a, 4, 1, True)] and core.plan_sources() == [0]
+    core.build_planned(words)
+    assert core.commit([next_token([1, 2, 3, first])]) == [a]                    # the stop token: a ends here
+    assert core.request_output(a) == [first] and core.request_info(a)["finish"] == 1
+    core.drop_request(a)
+    core.launch()                                                                # what was planned for it is dead
+    assert core.plan() == []
+    assert core.commit([55]) == []                                               # its sample is dropped
+    assert core.idle() and core.pages_free() == 20 and core.slots_in_use() == 0 and not core.in_flight()
+
+
+def test_nobody_is_preempted_ahead_of_a_step_in_flight():
+    core = HostCore([(4, 2, 0)], max_requests=2, token_budget=16)
+    a = core.add_request([1, 2, 3, 4], 5)
+    b = core.add_request([5, 6, 7, 8], 5)
+    words = np.zeros(4096, dtype=np.int32)
+    assert core.plan() == [(a, 0, 4, True), (b, 0, 4, True)]
+    core.build_planned(words)
+    core.launch()
+    assert core.plan() == [] and core.preemptions() == 0      # both need a second page and none is free: the caller lands the step first
+    assert core.commit([11, 12]) == []
+    plan = core.plan()                                        # in turn again: the request admitted last gives way
+    assert plan == [(a, 4, 1, True)] and core.preemptions() == 1
