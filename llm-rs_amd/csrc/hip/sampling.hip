@@ -701,3 +701,27 @@ extern "C" int llmrs_sample_rows(hipStream_t stream, const float* logits, int ld
     LLMRS_LAUNCH_CHECK("sample_rows");
     return 0;
 }
+
+// tokens[rows[i]] = ids[sources[i]] for i < n: the ids a step sampled go into the next step's token array on the
+// device, for a caller that starts that step before the ids have reached the host.  rows are places in `tokens`
+// (n_tokens long), sources rows of `ids` (n_ids long); a pair outside either is left alone, and so is an id outside
+// the vocabulary (the token then stays what the host wrote there).
+__global__ void place_ids_kernel(int* __restrict__ tokens, int n_tokens, const int* __restrict__ rows,
+                                 const int* __restrict__ sources, const int* __restrict__ ids, int n_ids, int n, int V) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int row = rows[i], src = sources[i];
+    if (row < 0 || row >= n_tokens || src < 0 || src >= n_ids) return;
+    int id = ids[src];
+    if (id >= 0 && id < V) tokens[row] = id;
+}
+
+extern "C" int llmrs_place_ids(hipStream_t stream, int* tokens, int n_tokens, const int* rows, const int* sources,
+                               const int* ids, int n_ids, int n, int V) {
+    LLMRS_REQUIRE(n >= 0 && n_tokens >= 0 && n_ids >= 0 && V > 0, "place_ids: bad sizes n=%d tokens=%d ids=%d V=%d", n, n_tokens, n_ids, V);
+    if (n == 0) return 0;
+    LLMRS_REQUIRE(tokens && rows && sources && ids, "place_ids: null argument");
+    place_ids_kernel<<<(n + 255) / 256, 256, 0, stream>>>(tokens, n_tokens, rows, sources, ids, n_ids, n, V);
+    LLMRS_LAUNCH_CHECK("place_ids");
+    return 0;
+}

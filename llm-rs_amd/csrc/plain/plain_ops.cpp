@@ -304,6 +304,18 @@ extern "C" int llmrs_plain_argmax_rows(void*, const float* logits, int ld, int n
     return 0;
 }
 
+// tokens[rows[i]] = ids[sources[i]]; a pair outside either array, or an id outside the vocabulary, changes nothing.
+extern "C" int llmrs_plain_place_ids(void*, int* tokens, int n_tokens, const int* rows, const int* sources, const int* ids,
+                                     int n_ids, int n, int V) {
+    if (n < 0 || n_tokens < 0 || n_ids < 0 || V <= 0) return -1;
+    for (int i = 0; i < n; ++i) {
+        if (rows[i] < 0 || rows[i] >= n_tokens || sources[i] < 0 || sources[i] >= n_ids) continue;
+        int id = ids[sources[i]];
+        if (id >= 0 && id < V) tokens[rows[i]] = id;
+    }
+    return 0;
+}
+
 namespace {
 // The probabilities a row is drawn from (src/sampler/mod.rs:84-141): logits / temperature; all but the top_k largest
 // dropped; softmax; the shortest prefix of the descending order whose mass reaches top_p kept and renormalised.  Of

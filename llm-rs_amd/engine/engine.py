@@ -53,6 +53,16 @@ class Emitted:
 
 
 @dataclass
+class _Flight:
+    """A step that was started and whose samples the scheduler has not been told."""
+    owners: List[tuple]              # (slot, request) of the entries that sample, in their order
+    ids: Optional[torch.Tensor]      # their samples on the device (the sampler's buffer: good until the next step samples)
+    host: Optional[torch.Tensor]     # the same on their way to the host
+    landed: object                   # an event behind that copy, or None where copies are synchronous
+    events: Optional[tuple]          # (before the first kernel, after sampling) when device time is measured
+
+
+@dataclass
 class _Submitted:
     prompt: Sequence[int]
     limit: int
@@ -63,7 +73,11 @@ class _Submitted:
 class Engine:
     def __init__(self, config, tensors: Mapping[str, torch.Tensor], *, dtype="bfloat16", device="cuda",
                  page_size: int = 16, num_pages=None, kv_memory_fraction: float = 0.8, max_requests: int = 256,
-                 max_batch_tokens: int = 2048, max_chunk: int = 0, max_seq_len: Optional[int] = None, log: bool = False):
+                 max_batch_tokens: int = 2048, max_chunk: int = 0, max_seq_len: Optional[int] = None, log: bool = False,
+                 overlap: bool = True):
+        """`overlap`: `advance()` starts a step before the samples of the step before it have reached the host (the
+        device hands them over), so that the device does not wait while the host reads samples and plans; outputs
+        are the same.  Without it a step is planned only when the one before has been read."""
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}")
         self.config = config
@@ -90,6 +104,10 @@ class Engine:
         self._waiting: Dict[int, _Submitted] = {}          # submitted, no slot yet (in order of submission)
         self._request_of: Dict[int, int] = {}              # slot -> request, for those the scheduler holds
         self._samples_randomly: set = set()                 # of those, the slots that do not decode greedily
+        self.overlap = bool(overlap)
+        self._flight: Optional[_Flight] = None               # the step in flight (overlap)
+        self._ids_host = [None, None]                        # pinned room for samples on their way to the host, in turns
+        self._ids_turn = 0
         self._steps = 0
         self._step_events: List[tuple] = []                 # (before the first kernel, after sampling) of measured steps
         # A full collection now, while nothing waits for it: building the model has made so many
@@ -212,7 +230,7 @@ class Engine:
         return total
 
     def has_unfinished(self) -> bool:
-        return bool(self._waiting) or bool(self._request_of)
+        return bool(self._waiting) or bool(self._request_of) or self._flight is not None
 
     def cancel(self, request: int) -> None:
         """Ends a request wherever it stands; its pages and its slot go back."""
@@ -240,10 +258,85 @@ class Engine:
             if sub.params.temperature != 0.0:
                 self._samples_randomly.add(slot)
 
+    def _start_step(self, after: Optional[_Flight]) -> Optional[_Flight]:
+        """Plans a step and starts it on the device, sampling included, without waiting for anything.  `after`: the
+        step in flight whose samples this one's tokens may be.  None when nothing could be planned."""
+        logits, n_want, plan = self.runner.run_planned(after.ids if after is not None else None)
+        if not plan:
+            return None
+        ids = host = landed = events = None
+        if n_want:
+            ids = self.sampler.sample(logits, self.runner.ctx.sampling, not self._samples_randomly)
+        if self.runner.time_device and self.runner.started is not None:
+            done = torch.cuda.Event(enable_timing=True)
+            done.record()
+            events = (self.runner.started, done)
+        if n_want:
+            if self.device.type == "cuda":
+                self._ids_turn ^= 1
+                host = self._ids_host[self._ids_turn]
+                if host is None or host.numel() < n_want:
+                    host = self._ids_host[self._ids_turn] = torch.zeros(max(2 * n_want, 256), dtype=torch.int32, pin_memory=True)
+                host = host[:n_want]
+                host.copy_(ids, non_blocking=True)
+                landed = torch.cuda.Event()
+                landed.record()
+            else:
+                host = ids.clone()
+        self._steps += 1
+        return _Flight([(p[0], self._request_of[p[0]]) for p in plan if p[3]], ids, host, landed, events)
+
+    def _land_step(self, flight: _Flight) -> List[Emitted]:
+        """Waits for a started step's samples, tells the scheduler, and returns what each sampling request got."""
+        core = self.cache.core
+        if flight.events is not None:
+            self._step_events.append(flight.events)
+        sampled = []
+        if flight.host is not None:
+            if flight.landed is not None:
+                flight.landed.synchronize()
+            sampled = flight.host.numpy().copy()
+        finished = set(core.commit(sampled))
+        out: List[Emitted] = []
+        for (slot, request), token in zip(flight.owners, sampled):
+            if self._request_of.get(slot) != request:
+                continue                    # it ended while this step was in flight (a stop token, a cancel): dropped
+            if slot in finished:
+                reason = "stop" if core.request_info(slot)["finish"] == 1 else "length"
+                out.append(Emitted(request, None if reason == "stop" else int(token), reason))
+                core.drop_request(slot)
+                self._forget(slot)
+            else:
+                out.append(Emitted(request, int(token)))
+        return out
+
+    def _advance_overlapped(self) -> List[Emitted]:
+        core = self.cache.core
+        self._admit()
+        if self._flight is None:
+            if core.idle():
+                return []
+            self._flight = self._start_step(None)
+            if self._flight is None:
+                raise RuntimeError("the scheduler planned nothing although requests are waiting")
+            core.launch()
+        # the step after it, before this one's samples are known (nothing, when all it could run waits for pages
+        # or for those samples: then the next call starts afresh)
+        ahead = self._start_step(self._flight)
+        out = self._land_step(self._flight)
+        self._flight = ahead
+        if ahead is not None:
+            core.launch()
+        self._admit()
+        return out
+
     def advance(self) -> List[Emitted]:
         """One step of the scheduler: admits what fits, runs the planned batch (prompt portions
         beside decoded tokens), samples, and returns what each sampling request got.  Requests
-        still inside their prompts get nothing in that step."""
+        still inside their prompts get nothing in that step.  (With `overlap` what is returned is
+        the step before the one this call started; the last calls only collect.)"""
+        if self.overlap:
+            return self._advance_overlapped()
         core = self.cache.core
         self._admit()
         if core.idle():
@@ -324,6 +417,9 @@ class Engine:
         except BaseException:
             for r in index_of:                  # leave the engine as it was found
                 self.cancel(r)
+            if self._flight is not None:        # (every entry of the step in flight is dead now: its samples are dropped)
+                flight, self._flight = self._flight, None
+                self.cache.core.commit([0] * len(flight.owners))
             raise
         if self.device.type == "cuda":
             torch.cuda.synchronize(self.device)

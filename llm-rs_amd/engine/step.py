@@ -296,8 +296,10 @@ class StepRunner:
         ctx = self._bind(dev, off, T, R, len(want_rows), list(zip(slots, starts, counts)))
         return self._execute(ctx, widths)
 
-    def run_planned(self):
-        """Runs the step the scheduler planned; returns (logits or None, rows that sample)."""
+    def run_planned(self, samples_in_flight: Optional[torch.Tensor] = None):
+        """Runs the step the scheduler planned; returns (logits or None, rows that sample, the plan).
+        `samples_in_flight`: the ids (on the device) that the step before this one sampled, when the scheduler has
+        not been told them yet: entries whose one token is among them get it there, on the device."""
         core = self.cache.core
         plan = core.plan()
         if not plan:
@@ -305,11 +307,24 @@ class StepRunner:
         T = sum(p[2] for p in plan)
         R = len(plan)
         longest = max(p[1] + p[2] for p in plan)
+        rows, sources, at = [], [], 0
+        if samples_in_flight is not None:
+            for p, src in zip(plan, core.plan_sources()):
+                if src >= 0:
+                    rows.append(at); sources.append(src)
+                at += p[2]
         widths = self._graph_widths([p[2] for p in plan], longest)
-        words = self._staging(self._estimate_words(T, R, R, longest, widths))
+        words = self._staging(self._estimate_words(T, R, R, longest, widths) + 2 * len(rows))
         off, n_tokens, n_want = core.build_planned(words, fixed_widths=widths)
-        dev = self._upload(off.words)
+        n = len(rows)                              # behind the batch: where the samples in flight go, and which
+        words[off.words:off.words + n] = rows
+        words[off.words + n:off.words + 2 * n] = sources
+        dev = self._upload(off.words + 2 * n)
         ctx = self._bind(dev, off, n_tokens, R, n_want, [(p[0], p[1], p[2]) for p in plan])
+        if n:
+            from ..kernels import kernels
+            kernels().place_ids(ctx.tokens, dev[off.words:off.words + n], dev[off.words + n:off.words + 2 * n],
+                                samples_in_flight, self.model.spec.vocab_size)
         return self._execute(ctx, widths), n_want, plan
 
     def _execute(self, ctx: StepContext, graph_widths=None) -> Optional[torch.Tensor]:

@@ -147,6 +147,7 @@ class HipKernels:
             "llmrs_qkv_rope_cache": [V, I, V, I, V, V, I, I, I, V, V, V, I, V, V, I, I, I, I, I, I, V, c_size_t, I, V, I, F],
             "llmrs_argmax_rows": [V, V, I, I, I, V, V, c_size_t],
             "llmrs_sample_rows": [V, V, I, I, I, V, V],
+            "llmrs_place_ids": [V, V, I, V, V, V, I, I, I],
         }
         for name, args in sigs.items():
             fn = getattr(lib, name)
@@ -363,6 +364,13 @@ class HipKernels:
         self._run("argmax", logits.numel() * 4, 0, None,
                   self.lib.llmrs_argmax_rows, self._stream(), _p(logits), logits.stride(0), logits.shape[0],
                   logits.shape[1], _p(out), _p(scratch), 0 if scratch is None else scratch.numel() * scratch.element_size())
+
+    def place_ids(self, tokens: torch.Tensor, rows: torch.Tensor, sources: torch.Tensor, ids: torch.Tensor, vocab: int) -> None:
+        """tokens[rows[i]] = ids[sources[i]]: what a step sampled goes into the next step's tokens on the device."""
+        assert all(t.dtype == torch.int32 and t.is_contiguous() for t in (tokens, rows, sources, ids)) and rows.numel() == sources.numel()
+        self._run("place_ids", rows.numel() * 12, 0, None,
+                  self.lib.llmrs_place_ids, self._stream(), _p(tokens), tokens.numel(), _p(rows), _p(sources), _p(ids),
+                  ids.numel(), rows.numel(), int(vocab))
 
     # words[i] = uniform (float bits), temperature (float bits), top_k, top_p (float bits) of row i
     def sample_rows(self, logits: torch.Tensor, words: torch.Tensor, out: torch.Tensor) -> None:

@@ -136,6 +136,11 @@ class EmulatedKernels:
             best = logits[i].max()
             out[i] = int((logits[i] == best).nonzero()[0])
 
+    def place_ids(self, tokens, rows, sources, ids, vocab):
+        for row, src in zip(rows.tolist(), sources.tolist()):
+            if 0 <= row < tokens.numel() and 0 <= src < ids.numel() and 0 <= int(ids[src]) < vocab:
+                tokens[row] = ids[src]
+
     def sample_rows(self, logits, words, out):
         w = words.cpu()
         for i in range(logits.shape[0]):

@@ -34,6 +34,7 @@ class PlainTwins:
             "llmrs_plain_attention": [V, I, V, I, V, I, V, V, V, I, V, V, V, V, I, I, I, I, I, I, I, I, F, V, S, I, I, ctypes.c_long, I],
             "llmrs_plain_argmax_rows": [V, V, I, I, I, V, V, S],
             "llmrs_plain_sample_rows": [V, V, I, I, I, V, V, V],
+            "llmrs_plain_place_ids": [V, V, I, V, V, V, I, I, I],
             "llmrs_plain_cast": [V, V, I, V, I, S],
             "llmrs_plain_scale_softcap_rows": [V, V, I, I, I, F, F],
         }
@@ -107,6 +108,10 @@ class PlainTwins:
         assert probs is None or (probs.dtype == torch.float64 and probs.is_contiguous() and probs.shape == logits.shape)
         self._check(self.lib.llmrs_plain_sample_rows(None, _p(logits), logits.stride(0), logits.shape[0], logits.shape[1],
                                                      _p(words), _p(out), _p(probs)), "sample_rows")
+
+    def place_ids(self, tokens, rows, sources, ids, vocab: int) -> None:
+        self._check(self.lib.llmrs_plain_place_ids(None, _p(tokens), tokens.numel(), _p(rows), _p(sources), _p(ids),
+                                                   ids.numel(), rows.numel(), int(vocab)), "place_ids")
 
     def cast(self, dst, src) -> None:
         self._check(self.lib.llmrs_plain_cast(None, _p(dst), _CODE[dst.dtype], _p(src), _CODE[src.dtype], src.numel()), "cast")

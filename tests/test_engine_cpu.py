@@ -97,3 +97,60 @@ def test_no_gpu_is_said_before_any_weight_is_read(tmp_path, monkeypatch):
     with pytest.raises(Exception, match="GPU|gfx950|kernel"):
         Engine.from_folder(str(tmp_path))
     assert read == []
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_a_step_started_before_the_last_one_is_read_changes_no_output(which):
+    """`overlap` (a step is planned and started while the step before is in flight, its samples handed over on the
+    device) against stepping in turn: the same tokens and finish reasons, with stop tokens, sampling with a
+    temperature, requests that end at different times and a pool so small that requests give way."""
+    cfg_d = TINY_A if which == "A" else TINY_B
+    cfg = LlamaConfig.from_dict(cfg_d)
+    tensors = random_model_tensors(cfg, 11)
+    rng = np.random.default_rng(5)
+    prompts = [rng.integers(0, cfg.vocab_size, int(n)).tolist() for n in (3, 17, 9, 1, 26, 12, 5)]
+    limits = [16, 14, 1, 16, 6, 2, 15]
+    seeds = [3, 4, 5, 6, 7, 8, 9]
+
+    def run(overlap, temperature, stop):
+        eng = Engine(cfg, tensors, dtype="float32", device="cpu", page_size=4, num_pages=10, max_requests=3,
+                     max_batch_tokens=16, overlap=overlap)
+        got = eng.generate(prompts, limits, temperature=temperature, top_k=20, top_p=0.95, seed=seeds,
+                           stop_token_ids=stop, return_reasons=True)
+        core = eng.cache.core
+        assert core.pages_free() == 10 and core.slots_in_use() == 0 and not core.in_flight() and not eng.has_unfinished()
+        return [(f.tokens, f.reason) for f in got], eng.last_stats
+
+    with use_kernels(EmulatedKernels()):
+        free, stats = run(False, 0.9, [])
+        assert stats.preemptions > 0, "the case itself: the pool is too small for what three requests grow to"
+        assert run(True, 0.9, [])[0] == free
+        assert run(True, 0.0, [])[0] == run(False, 0.0, [])[0]
+        # a stop token that does occur in the middle of an output: a token some request sampled that it had not before
+        i, at = next((i, j) for i, (toks, _) in enumerate(free) for j in range(1, len(toks)) if toks[j] not in toks[:j])
+        stop = [free[i][0][at]]
+        in_turn = run(False, 0.9, stop)[0]
+        assert in_turn[i] == (free[i][0][:at], "stop")
+        assert run(True, 0.9, stop)[0] == in_turn
+
+
+def test_cancel_while_a_step_is_in_flight(engine_a):
+    eng, tensors = engine_a
+    assert eng.overlap
+    a = eng.submit([5, 6, 7], 8)
+    b = eng.submit([9, 1], 8)
+    got = {a: [], b: []}
+    for e in eng.advance():                    # the first call starts two steps and lands the first
+        got[e.request].append(e.token)
+    assert eng.cache.core.in_flight()
+    eng.cancel(a)                              # a has an entry in the step in flight
+    c = eng.submit([3, 3, 3, 3], 4)            # takes a's slot
+    got[c] = []
+    while eng.has_unfinished():
+        for e in eng.advance():
+            got[e.request].append(e.token)
+    assert got[b] == plain_generate(TINY_A, tensors, [9, 1], 8)
+    assert got[c] == plain_generate(TINY_A, tensors, [3, 3, 3, 3], 4), "what a's step in flight sampled is nobody's"
+    assert len(got[a]) == 1
+    core = eng.cache.core
+    assert core.pages_free() == 24 and core.slots_in_use() == 0 and not core.in_flight()

@@ -224,6 +224,28 @@ def test_argmax_and_sample_rows():
             assert tok == int(twin_out[i])
 
 
+def test_place_ids():
+    """Sampled ids into the next step's tokens: pairs out of range and ids outside the vocabulary change nothing."""
+    g = torch.Generator().manual_seed(31)
+    tokens = torch.randint(0, 900, (700,), generator=g).to(torch.int32)
+    ids = torch.randint(0, 900, (300,), generator=g).to(torch.int32)
+    ids[7], ids[8] = -3, 900                                        # not in a vocabulary of 900
+    rows = torch.randperm(700, generator=g)[:300].to(torch.int32)
+    sources = torch.randperm(300, generator=g).to(torch.int32)
+    rows[5], rows[6], sources[9], sources[10] = -1, 700, -1, 300    # outside either array
+    (pair,) = both("place_ids", [tokens.clone(), rows, sources, ids, 900], [0])
+    assert torch.equal(*pair)
+    got = pair[0]
+    changed = 0
+    for i in range(300):
+        r, s_ = int(rows[i]), int(sources[i])
+        if 0 <= r < 700 and 0 <= s_ < 300 and 0 <= int(ids[s_]) < 900:
+            assert int(got[r]) == int(ids[s_]); changed += 1
+    untouched = torch.ones(700, dtype=torch.bool)
+    untouched[rows[(rows >= 0) & (rows < 700)].long()] = False
+    assert torch.equal(got[untouched], tokens[untouched]) and changed >= 290
+
+
 def test_cast_and_softcap():
     src = rnd((100003,), torch.float32, 26, 50.0)
     assert torch.equal(*both("cast", [torch.zeros(100003, dtype=torch.bfloat16), src], [0])[0])
