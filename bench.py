@@ -4,8 +4,9 @@
     python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
-requests, each with 2,048 tokens of context already in the cache, decode K steps
-(one token per request per step, sampled greedily on the device, ids read back),
+requests, each with 2,048 tokens of context in the cache, decode K steps through the
+engine's own loop (submit / advance: one token per request per step, sampled greedily
+on the device, ids read back; the scheduler plans the next step while one is in flight),
 and report decoded tokens a second.  The same line carries a 2,048-token prefill,
 the decode step's share of the HBM roofline, decode at batch 1 and 64, and the
 host's share of a step (wall time minus the device's, from events around the step).
@@ -189,7 +190,9 @@ def prompts_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
 # ---- measurements (need the GPU) -------------------------------------------------------------------------------
 
 class Bench:
-    def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int):
+    def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int, side_by_side: bool = False):
+        """`side_by_side`: a request's portion of a step is capped so that `max_requests` prompts of one length run
+        side by side and end in the same step (for `decode_run`, whose requests then decode over equal contexts)."""
         import torch
         from llm_rs_amd import Engine, LlamaConfig
         self.torch = torch
@@ -199,7 +202,8 @@ class Bench:
         self.config = LlamaConfig.from_dict(d)
         t0 = time.time()
         self.engine = Engine.from_random(self.config, seed=0, dtype=args.dtype, device="cuda:0", page_size=16,
-                                         num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens)
+                                         num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens,
+                                         max_chunk=max(1, max_batch_tokens // max_requests) if side_by_side else 0)
         torch.cuda.synchronize()
         print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         self.gen = torch.Generator().manual_seed(0)
@@ -238,29 +242,29 @@ class Bench:
         return sum(a.elapsed_time(b) for a, b in pairs) * 1e-3 / reps
 
     def decode_run(self, batch, context, steps, warmup, with_device_time=False):
-        from llm_rs_amd import StepEntry
+        """Seconds per decode step of `batch` requests over `context` keys each, through the engine's own loop
+        (submit / advance: the scheduler, one step in flight while the next is planned), and the device's share."""
         engine = self.engine
-        slots = [engine.open_request() for _ in range(batch)]
-        for s in slots:                         # fill each request's cache with `context` tokens
-            self.fill(s, self.prompt(context))
-        pos = [context] * batch
-        state = {"last": [1] * batch}
+        measured = min(steps, 16) if with_device_time else 0
+        requests = [engine.submit(self.prompt(context), max_new_tokens=warmup + steps + measured + 4) for _ in range(batch)]
+        for _ in range(context * batch + 8):        # the prompts, in equal portions side by side: they end in the same step
+            if len(engine.advance()) == batch:
+                break
+        else:
+            raise RuntimeError("the requests did not come to decode together")
 
         def one_step():
-            entries = [StepEntry(s, pos[i], [state["last"][i]], [0]) for i, s in enumerate(slots)]
-            logits = engine.step(entries)
-            ids = engine.sampler.sample(logits, engine.runner.ctx.sampling, True)
-            one_step.after = ids            # (the device-time event is recorded between the launch and the read-back)
-            state["last"] = ids.cpu().tolist()
-            for i in range(batch):
-                pos[i] += 1
+            if len(engine.advance()) != batch:
+                raise RuntimeError("a decode step did not give every request a token")
 
         for _ in range(warmup):
             one_step()
         sec = self.timed(one_step, steps)
-        dev = self.device_seconds(one_step, min(steps, 16)) if with_device_time else None
-        for s in slots:
-            engine.close_request(s)
+        dev = self.device_seconds(one_step, measured) if with_device_time else None
+        for r in requests:
+            engine.cancel(r)
+        while engine.has_unfinished():              # (the step in flight lands; what it sampled is nobody's)
+            engine.advance()
         return sec, dev
 
 
@@ -269,7 +273,7 @@ def run_decode8b(args) -> dict:
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
     ctx_pages = -(-(args.context + args.steps + args.warmup + 24) // 16)
-    b = Bench(args, LLAMA_8B, max_batch * ctx_pages + 8, max(max_batch, 8), max(args.prefill_tokens, 2048))
+    b = Bench(args, LLAMA_8B, max_batch * ctx_pages + 8, max(max_batch, 8), max(args.prefill_tokens, 2048), side_by_side=True)
     engine = b.engine
     toks = b.prompt(args.prefill_tokens)
 
@@ -301,7 +305,7 @@ def run_sizes(args) -> dict:
     small = args.workload == "sizes1b"
     cases = [(1, 2048), (8, 2048), (64, 2048)] if small else [(1, long), (8, long), (64, long), (128, 2048), (256, 2048)]
     pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
-    b = Bench(args, LLAMA_1B if small else LLAMA_8B, pages, 256, 2048)
+    b = Bench(args, LLAMA_1B if small else LLAMA_8B, pages, 256, 2048, side_by_side=True)
     weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
     points, fractions, first_s = {}, {}, None
     for batch, ctx in cases:
@@ -320,7 +324,7 @@ def run_long(args) -> dict:
     shape = dict(LLAMA_8B, max_position_embeddings=131072)
     cases = [(1, 131072 - 64), (4, 32768 - 64)]
     pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
-    b = Bench(args, shape, pages, 8, 2048)
+    b = Bench(args, shape, pages, 8, 2048, side_by_side=True)
     weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
     points, fractions, first_s = {}, {}, None
     for batch, ctx in cases:
