@@ -575,6 +575,162 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 3
         for (int i = 0; i < 16; ++i) pp[2 + o_feature(dt, i, h)] = O[dt][i];
 }
 
+// ---- the same with 16 query columns to a wave (up to 16 heads to a kv head) --
+// A single token brings G query columns; the 32-column products above spend their accumulators on 32 - G columns
+// of nothing.  Here S^T = K Q^T is two 16 x 16 tiles per 32 keys and O^T += V^T P^T one product per 16 features
+// with the 32 keys as its k: a quarter of the accumulators and half of the exponentials, so that a SIMD holds
+// more of these waves, and with them more keys on their way.
+// Which keys a 16-row tile holds is free, as long as the values' operand takes them in the same order: tile t of a
+// 32-key step holds key 8 * (row / 4) + row % 4 + 4 * t in its row, so lane (col, g) ends with the scores of keys
+// 8g .. 8g + 7 in its eight registers (tile 0's four, then tile 1's): the B operand of the second product as it
+// stands, and for the values, [feature][16 keys] per page, one 16-byte load per lane and 16 features.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// The registers would let a SIMD hold three of these waves at head size 128 and four at 64, and with twelve or
+// sixteen to a compute unit the scattered pages come slower than with eight once the device is full (decode steps
+// of the 8B shape, eight waves against twelve: 64 requests over 8128 keys 15.9 against 16.9 ms, 256 over 2048 18.3
+// against 20.7; the 1B serving run 3.03 against 3.10 s with sixteen).  Every block asks for an eighth of a
+// unit's LDS, which it does not use, and that keeps a unit to eight.
+#define SPLIT16_LDS_BYTES (160 * 1024 / 8)
+
+// The value of the lane 16 further on or back (the partner in the neighbouring row of 16 lanes), by the register
+// swap of gfx950: of {x, x} it makes {rows 0, 0, 2, 2 of x; rows 1, 1, 3, 3 of x}.
+__device__ __forceinline__ float other_row(float x) {
+    unsigned u = __float_as_uint(x);
+    auto sw = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return __uint_as_float((threadIdx.x & 16) ? sw[0] : sw[1]);
+}
+__device__ __forceinline__ float across_groups_max(float x) {
+    x = fmaxf(x, other_row(x));
+    return fmaxf(x, other_half(x));
+}
+__device__ __forceinline__ float across_groups_sum(float x) {
+    x += other_row(x);
+    return x + other_half(x);
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict__ q, float* __restrict__ partial,
+                                                          const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                                                          const int* __restrict__ block_table,
+                                                          const int* __restrict__ seq_lens,
+                                                          const int* __restrict__ q_starts, AttnArgs a, int G,
+                                                          int max_chunks, int chunk, int plain) {
+    static_assert(HD % 32 == 0, "the score products take 32 features at a time");
+    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z;
+    int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    bool cvalid = c < G;
+    int head = kvh * G + min(c, G - 1);
+    const int* table = block_table + (size_t)e * a.table_width;
+    bf16x8 qf[HD / 32];
+    int token, pos_t, lo_t, t_begin, pv = 0;
+    auto load_pages = [&](int first) {
+        int pg = table[min(first + lane, a.table_width - 1)];
+        return min(max(pg, 0), a.num_pages - 1);
+    };
+    if (plain) {
+        token = e;
+        lo_t = 0;
+        t_begin = ch * chunk;
+        pv = load_pages(t_begin >> 4);
+        const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + g * 8;
+#pragma unroll
+        for (int j = 0; j < HD / 32; ++j) qf[j] = *(const bf16x8*)(qp + j * 32);
+        pos_t = seq_lens[e] - 1;
+        if (t_begin > pos_t) return;
+    } else {
+        token = q_starts[e];
+        int count = q_starts[e + 1] - token;
+        pos_t = seq_lens[e] - 1;
+        if (count != 1) return;
+        lo_t = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
+        int first_chunk = lo_t / chunk;
+        int n_chunks = pos_t / chunk - first_chunk + 1;
+        if (ch >= n_chunks) return;
+        t_begin = (first_chunk + ch) * chunk;
+        pv = load_pages(t_begin >> 4);
+        const bf16* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + g * 8;
+#pragma unroll
+        for (int j = 0; j < HD / 32; ++j) qf[j] = *(const bf16x8*)(qp + j * 32);
+    }
+    int t_end = min(t_begin + chunk, pos_t + 1);
+    int pv_base = t_begin >> 4;
+    float c2 = a.scale * 1.44269504088896341f;
+    f32x4 O[HD / 16];
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) O[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.0f;                    // m: the same in a column's four lanes; l: this lane's share of the sum
+    // the keys of tile t that this lane's operand row holds, within a 32-key step: 8 * (row / 4) + row % 4 + 4t
+    int krow = 8 * (c >> 2) + (c & 3);
+    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+        int lp = t0 >> 4;
+        if (lp + 1 - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
+        int p0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
+        int p1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : p0;
+        bf16x8 kf[2][HD / 32];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            int key = krow + 4 * t;                                   // 0..31: page key >> 4, row key & 15
+            const bf16* kp = kc + (((size_t)(key < 16 ? p0 : p1) * a.n_kv_heads + kvh) * 16 + (key & 15)) * HD + g * 8;
+#pragma unroll
+            for (int j = 0; j < HD / 32; ++j) kf[t][j] = *(const bf16x8*)(kp + j * 32);
+        }
+        // values: lane (feature row c, g) takes keys 8g .. 8g + 7 of the step: page g / 2, keys 8 * (g % 2) .. of it
+        bf16x8 vf[HD / 16];
+        const bf16* vp = vc + (((size_t)(g < 2 ? p0 : p1) * a.n_kv_heads + kvh) * HD + c) * 16 + (g & 1) * 8;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt) vf[dt] = *(const bf16x8*)(vp + dt * 16 * 16);
+        f32x4 S[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            S[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < HD / 32; ++j) S[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][j], qf[j], S[t], 0, 0, 0);
+        }
+        // this lane's scores: keys t0 + 8g + i, i = 0..7 (tile 0's registers, then tile 1's)
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sc[i] = S[i >> 2][i & 3];
+        if (t0 + 31 > pos_t || t0 < lo_t) {                           // (the same in all lanes)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int key = t0 + 8 * g + i;
+                if (key > pos_t || key < lo_t) sc[i] = -INFINITY;
+            }
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sc[i]);
+        mx = across_groups_max(mx) * c2;
+        bool mine = mx > m + SOFTMAX_SLACK;
+        if (__any(mine)) {
+            float m_new = mine ? mx : m;
+            float alpha = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.0f : m_new));
+            m = m_new;
+            l *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < HD / 16; ++dt) O[dt] *= alpha;
+        }
+        float m_safe = m == -INFINITY ? 0.0f : m;
+        bf16x8 pf;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], c2, -m_safe));
+            l += p;
+            pf[i] = (bf16)p;
+        }
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; ++dt) O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, O[dt], 0, 0, 0);
+    }
+    l = across_groups_sum(l);
+    if (!cvalid) return;
+    float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
+    if (g == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pp[2 + dt * 16 + 4 * g + r] = O[dt][r];
+}
+
 #define MERGE_MAX_CHUNKS 1024
 
 // One block for each (entry, head), a thread for each feature (a wave per 64 of them).  Every wave finds the common
@@ -761,9 +917,10 @@ static SideStream* side_stream() {
     return s.stream != nullptr ? &s : nullptr;
 }
 
-// How many waves of the split a compute unit holds at once: what the registers of the kernel for this head size
-// allow (two to a SIMD at head size 128, three at 64), asked of the runtime once per head size.  Head sizes
-// without a kernel here: 8.
+// How many waves of the split a compute unit holds at once: eight (see SPLIT16_LDS_BYTES), fewer where the registers
+// of the kernel for this head size allow no more (four at head size 256), asked of the runtime once per head size.
+// Head sizes without a kernel here: 8.  (The 32-column kernel, for more than 16 heads to a kv head, holds eight at
+// head size 128 as well and twelve at 64; its chunks are chosen as if it held eight.)
 static int split_waves_to_a_unit(int head_dim) {
     static int known[8] = {0, 0, 0, 0, 0, 0, 0, 0};      // by head_dim / 32 - 1
     static std::mutex mutex;
@@ -774,7 +931,7 @@ static int split_waves_to_a_unit(int head_dim) {
         int blocks = 0;
         hipError_t e = hipErrorInvalidValue;
         switch (head_dim) {
-#define ASK(HD) case HD: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_split_kernel<HD>, 64, 0); break;
+#define ASK(HD) case HD: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, attn_split16_kernel<HD>, 64, SPLIT16_LDS_BYTES); break;
             ASK(32) ASK(64) ASK(96) ASK(128) ASK(192) ASK(256)
 #undef ASK
             default: break;
@@ -877,7 +1034,10 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     if (split) {
         dim3 grid(n_entries, a.n_kv_heads, max_chunks);
         int plain = only_single && a.window == 0;
-        attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk, plain);
+        if (G <= 16)
+            attn_split16_kernel<HD><<<grid, 64, SPLIT16_LDS_BYTES, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk, plain);
+        else
+            attn_split_kernel<HD><<<grid, 64, 0, single_stream>>>(q, scratch, kc, vc, table, seq_lens, q_starts, a, G, max_chunks, chunk, plain);
         if (max_chunks > MERGE_ONE_WALK_CHUNKS && HD <= MERGE_GROUP_THREADS) {
             int threads = (HD / 2) * ((max_chunks + 3) / 4);          // groups of HD / 2 threads, a group for every four chunks
             threads = std::min(MERGE_GROUP_THREADS, std::max(HD, (threads + 63) / 64 * 64));

@@ -248,9 +248,9 @@ def test_a_recording_is_kept_for_the_chunk_it_was_made_with():
         max_position_embeddings=4096, rms_norm_eps=1e-5, tie_word_embeddings=True))
     n_req, steps = 16, 40
     k = kernels()
-    by_len = [k.attention_split_chunk(n_req, 8, 64, 2048, n_req * n) for n in range(1100, 1990)]
-    change = next(1100 + i + 1 for i, (a, b) in enumerate(zip(by_len, by_len[1:])) if a != b)
-    plen = change - 20           # (with the rule as it stands: 1335)
+    by_len = [k.attention_split_chunk(n_req, 8, 64, 2048, n_req * n) for n in range(300, 1990)]
+    change = next(300 + i + 1 for i, (a, b) in enumerate(zip(by_len, by_len[1:])) if a != b)
+    plen = change - 20           # (with the rule as it stands: 902)
     chunks = {k.attention_split_chunk(n_req, 8, 64, 2048, n_req * (plen + 1 + i)) for i in range(steps)}
     assert len(chunks) == 2, "the case itself: the chunk must change on the way"
     prompts = [random_tokens(500, plen + steps + 1, seed=900 + i) for i in range(n_req)]

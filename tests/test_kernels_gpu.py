@@ -448,6 +448,25 @@ def test_attention_decoding_requests_a_few_keys_past_a_chunk(n_req, hd):
                 assert (got[r].float() - ref).abs().max() <= 2e-2, f"request {r}"
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd", [(1, 1, 128), (5, 1, 64), (16, 2, 32), (16, 1, 128), (12, 2, 96), (20, 1, 64), (40, 2, 128),
+                                             (9, 3, 192), (4, 2, 256), (32, 8, 128)])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_decoding_every_group_size(n_heads, n_kv, hd, window):
+    """Decoding requests with a random query for every head, 1 to 20 heads to a kv head (up to 16 a wave of the split
+    takes 16 query columns, beyond that 32), every head size the split has a kernel for, lengths around the edges of
+    32-key steps and of chunks, with and without a window: every head against the plain implementation."""
+    ps = 16
+    lens = [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 200, 257, 500, 777, 1030]
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, ps, seed=hd + n_heads)
+    g = torch.Generator().manual_seed(n_heads * 7 + hd)
+    qs = [torch.randn((1, n_heads, hd), generator=g).to(torch.bfloat16) for _ in lens]
+    pos = [[n - 1] for n in lens]
+    got = case.run(qs, pos, window=window, n_single=len(lens), single_keys=sum(min(n, window) if window else n for n in lens))
+    for r in range(len(lens)):
+        ref = case.reference(r, qs[r], pos[r], window=window)[0].float()
+        assert (got[r].float() - ref).abs().max() <= 2e-2, f"request {r} of length {lens[r]}"
+
+
 @pytest.mark.parametrize("window", [0, 300])
 @pytest.mark.parametrize("n_req", [70, 150])
 def test_attention_many_decoding_requests(n_req, window):
