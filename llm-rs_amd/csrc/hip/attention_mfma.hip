@@ -661,18 +661,42 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
     float m = -INFINITY, l = 0.0f;                    // m: the same in a column's four lanes; l: this lane's share of the sum
     // the keys of tile t that this lane's operand row holds, within a 32-key step: 8 * (row / 4) + row % 4 + 4t
     int krow = 8 * (c >> 2) + (c & 3);
-    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+    // A unit holds eight of these waves whatever they take (see SPLIT16_LDS_BYTES), so up to head size 128 a wave has
+    // the registers for a second set of key operands: the next step's keys are asked for before this step's products.
+    constexpr bool KEYS_AHEAD = HD <= 128;
+    auto pages_of = [&](int t0, int& a0, int& a1) {
         int lp = t0 >> 4;
         if (lp + 1 - pv_base >= 64) { pv_base = lp; pv = load_pages(lp); }
-        int p0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
-        int p1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : p0;
-        bf16x8 kf[2][HD / 32];
+        a0 = __builtin_amdgcn_readlane(pv, lp - pv_base);
+        a1 = (t0 + 16 < t_end) ? __builtin_amdgcn_readlane(pv, lp + 1 - pv_base) : a0;
+    };
+    auto load_keys = [&](bf16x8 (&k)[2][HD / 32], int a0, int a1) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             int key = krow + 4 * t;                                   // 0..31: page key >> 4, row key & 15
-            const bf16* kp = kc + (((size_t)(key < 16 ? p0 : p1) * a.n_kv_heads + kvh) * 16 + (key & 15)) * HD + g * 8;
+            const bf16* kp = kc + (((size_t)(key < 16 ? a0 : a1) * a.n_kv_heads + kvh) * 16 + (key & 15)) * HD + g * 8;
 #pragma unroll
-            for (int j = 0; j < HD / 32; ++j) kf[t][j] = *(const bf16x8*)(kp + j * 32);
+            for (int j = 0; j < HD / 32; ++j) k[t][j] = *(const bf16x8*)(kp + j * 32);
+        }
+    };
+    bf16x8 kf[2][HD / 32];
+    int p0 = 0, p1 = 0;
+    if constexpr (KEYS_AHEAD) {
+        pages_of(t_begin, p0, p1);
+        load_keys(kf, p0, p1);
+    }
+    for (int t0 = t_begin; t0 < t_end; t0 += 32) {
+        bf16x8 kn[2][HD / 32];
+        int n0 = 0, n1 = 0;
+        const bool more = t0 + 32 < t_end;                            // (the same in all lanes)
+        if constexpr (KEYS_AHEAD) {
+            if (more) {
+                pages_of(t0 + 32, n0, n1);
+                load_keys(kn, n0, n1);
+            }
+        } else {
+            pages_of(t0, p0, p1);
+            load_keys(kf, p0, p1);
         }
         // values: lane (feature row c, g) takes keys 8g .. 8g + 7 of the step: page g / 2, keys 8 * (g % 2) .. of it
         bf16x8 vf[HD / 16];
@@ -720,6 +744,15 @@ __global__ __launch_bounds__(64) void attn_split16_kernel(const bf16* __restrict
         }
 #pragma unroll
         for (int dt = 0; dt < HD / 16; ++dt) O[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, O[dt], 0, 0, 0);
+        if constexpr (KEYS_AHEAD) {
+            if (more) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int j = 0; j < HD / 32; ++j) kf[t][j] = kn[t][j];
+                p0 = n0; p1 = n1;
+            }
+        }
     }
     l = across_groups_sum(l);
     if (!cvalid) return;
