@@ -337,35 +337,13 @@ class Engine:
         the step before the one this call started; the last calls only collect.)"""
         if self.overlap:
             return self._advance_overlapped()
-        core = self.cache.core
         self._admit()
-        if core.idle():
+        if self.cache.core.idle():
             return []
-        logits, n_want, plan = self.runner.run_planned()
-        if not plan:
+        step = self._start_step(None)                # in turn: a step is started, and read before anything else happens
+        if step is None:
             raise RuntimeError("the scheduler planned nothing although requests are waiting")
-        sampled = []
-        if n_want:
-            sampled = self.sampler.sample(logits, self.runner.ctx.sampling, not self._samples_randomly)
-        if self.runner.time_device and self.runner.started is not None:
-            done = torch.cuda.Event(enable_timing=True)
-            done.record()
-            self._step_events.append((self.runner.started, done))
-        if n_want:
-            sampled = sampled.cpu().numpy()
-        self._steps += 1
-        sampling_slots = [p[0] for p in plan if p[3]]
-        finished = set(core.commit(sampled))
-        out: List[Emitted] = []
-        for slot, token in zip(sampling_slots, sampled):
-            request = self._request_of[slot]
-            if slot in finished:
-                reason = "stop" if core.request_info(slot)["finish"] == 1 else "length"
-                out.append(Emitted(request, None if reason == "stop" else int(token), reason))
-                core.drop_request(slot)
-                self._forget(slot)
-            else:
-                out.append(Emitted(request, int(token)))
+        out = self._land_step(step)
         self._admit()
         return out
 
