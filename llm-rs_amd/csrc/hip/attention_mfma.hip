@@ -978,14 +978,16 @@ static int split_waves_to_a_unit(int head_dim) {
 // Keys per wave of the split, by what the host knows: the number of single-token entries, the bound on their
 // length, and (when it says so) how many keys they see together.  Measured on the 8B head shape (8 to 256 requests
 // of 520 to 8000 keys, every chunk from 64 to 1024 keys) and on the 1B one: a compute unit holds so many of these
-// waves at once (eight at head size 128, twelve at 64) and works through them in turns of that many.  Waves of one
+// waves at once (eight) and works through them in turns of that many.  Waves of one
 // turn, all of the same length, end together, and the longest chunks that still fill half a turn are the fastest
 // (a wave begins with a chain of trips to memory: lengths, page numbers, then keys); one wave more than a turn
-// costs a second turn.  So: the smallest chunk that gives a unit no more than a turn; and when even chunks of 1024
-// keys give more, 512 if the last turn would be far from full (many short waves share out evenly as they come).
+// costs a second turn.  So: the smallest chunk that gives a unit no more than three quarters of a turn (the next
+// length then still gives it more than a third); and when even chunks of 1024
+// keys give more than a turn, 512 if the last turn would be far from full (many short waves share out evenly as they come).
 // Against the best chunk of each case (also at sizes and lengths between those it was made from, at 4 and 8 heads
-// to a kv head, 2 and 8 kv heads) this rule loses 0.1-0.5 % on average and 9 % at worst; the rule before it (128
-// keys, doubled while the waves kept all units busy, by the bound alone) lost 7.5 % and 19 %.  The chunks of a request are never
+// to a kv head, 2 and 8 kv heads) this rule is within the 3 % that two timings of one case differ by, 6 % at worst;
+// the rule before the first of this kind (128 keys, doubled while the waves kept all units busy, by the bound alone)
+// lost 7.5 % on average and 19 % at worst.  The chunks of a request are never
 // more than a quarter of what the merge takes.
 // The number of keys moves with every step while a recorded graph holds the chunk it was recorded with: callers that
 // record put this function's result into what they key their recordings by.  The scratch is sized by the smallest
@@ -1009,12 +1011,14 @@ extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int hea
             double q = keys / singles / c, whole = floor(q), rest = q - whole;
             return singles * n_kv_heads * (whole + (rest > 0.125 ? 1.0 : 0.0)) / cus;
         };
-        const double full = turn * 1.001;      // (a turn that is exactly full is the best case)
-        // (the shortest chunks are left a little before their turn is full: they gain nothing over the next length
-        // there, and a bound well above the lengths costs them twice the waves that find nothing to do)
+        const double full = turn * 1.001;
+        // With the 16-column kernel a unit does best on about half a turn of waves, one to a SIMD: a full turn of
+        // chunks half as long takes 2-7 % longer, a quarter of a turn of chunks twice as long 15-25 % (8 to 128
+        // requests of 520 to 8000 keys, every chunk forced).  So chunks are doubled while a unit would get more than
+        // three quarters of a turn: the next length still leaves it more than a third.
+        const double enough = 0.75 * turn;
         int c = ATTN_CHUNK / 2;
-        if (to_a_unit(c) >= 0.9 * turn) c *= 2;
-        while (c > ATTN_CHUNK / 2 && c < longest && to_a_unit(c) > full) c *= 2;
+        while (c < longest && to_a_unit(c) > enough) c *= 2;
         if (c == longest && to_a_unit(c) > full) {
             double last = fmod(to_a_unit(c), turn) / turn;
             if (last > 0.006 && last < 0.69) c /= 2;
