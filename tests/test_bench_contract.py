@@ -78,3 +78,23 @@ def test_lines_of_every_workload():
     assert line["config"]["max_context"] == 131072 and set(line["points"]) == set(line["roofline_frac"])
     line = check_line(b.prompts_line(args, 32, {"prefill_2048": 67000.0, "prefill_2049": 60000.0}, {"prefill_2048": 0.39, "prefill_2049": 0.35}, 0.0305))
     assert set(line["points"]) == set(line["peak_frac"]) and line["value"] == 67000.0 and abs(line["ms_per_step"] - 30.5) < 1e-6
+
+
+import pytest
+
+
+@pytest.mark.gpu
+def test_the_default_workload_runs_and_fills_its_line():
+    """The default workload with one layer and a few steps, in this process: decode steps go through the engine's own
+    loop (every call gives every request a token, or the run stops), and the line carries a prefill, a roofline,
+    both points and the host's share."""
+    bench = load_bench()
+    args = SimpleNamespace(gpus=1, steps=6, warmup=4, workload="decode8b", batch=8, context=300, prefill_tokens=256, layers=1,
+                           dtype="bfloat16", points="1,20", only="", requests=0, new_tokens=0, max_batch_tokens=2048)
+    line = check_line(bench.run_decode8b(args))
+    assert line["value"] > 0 and abs(line["value"] - 8 / (line["ms_per_step"] * 1e-3)) <= 1e-3 * line["value"]
+    assert line["config"]["layers_run"] == 1 and line["config"]["layers_of_config"] == 32 and line["config"]["global_batch"] == 8
+    assert set(line["points"]) == {"decode_b1", "decode_b20"} and all(v > 0 for v in line["points"].values())
+    assert line["prefill"]["tokens"] == 256 and 0 < line["prefill"]["frac"] < 1
+    assert line["roofline"]["bound"] == "hbm" and 0 < line["roofline"]["frac"] < 1
+    assert 0 <= line["host"]["overhead_frac"] < 0.5 and line["host"]["device_ms_per_step"] > 0
