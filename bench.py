@@ -107,8 +107,8 @@ def decode_line(args, layers, step_s, weight_bytes, cache_bytes_per_token, prefi
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     T = args.prefill_tokens
     line = base_line(
-        f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens and batch "
-        f"{'/'.join(p.split('_b')[1] for p in points)} alongside",
+        f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens"
+        + (f" and batch {'/'.join(p.split('_b')[1] for p in points)}" if points else "") + " alongside",
         args.batch / step_s, args.steps, args.warmup, step_s, args.dtype,
         flat_config("Llama-3.1-8B shape", layers, args.batch, args.context, 16, prefill_tokens=T))
     line["prefill"] = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
