@@ -190,8 +190,16 @@ class StepRunner:
     def _drop_graphs(self) -> None:
         """Forgets every recorded graph.  Destroying a graph frees device objects, so never during a recording."""
         assert not self._recording, "recorded graphs must not be destroyed while a stream is being captured"
+        self._settle()
         self._graphs.clear()
         self._seen.clear()
+
+    def _settle(self) -> None:
+        """Waits for what has been started on the device, before a recorded graph is destroyed: with a step in flight
+        while the next is planned, the graph being destroyed may be the one that is running.  (Rare: buffers grow a
+        few times in an engine's life, and recordings are dropped when a new one takes the oldest one's place.)"""
+        if self._graphs and self._pinned:
+            torch.cuda.current_stream(self.device).synchronize()
 
     # -- staging -----------------------------------------------------------------
     def _staging(self, words_needed: int) -> np.ndarray:
@@ -375,6 +383,7 @@ class StepRunner:
             self._seen.pop(key, None)
             return self.model.forward(ctx, self.cache.views)
         while len(self._graphs) >= self.max_graphs:
+            self._settle()
             self._graphs.popitem(last=False)
         self._graphs[key] = (graph, logits)
         graph.replay()                  # recording does not run the kernels
