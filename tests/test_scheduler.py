@@ -404,3 +404,43 @@ def test_nobody_is_preempted_ahead_of_a_step_in_flight():
     assert core.commit([11, 12]) == []
     plan = core.plan()                                        # in turn again: the request admitted last gives way
     assert plan == [(a, 4, 1, True)] and core.preemptions() == 1
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_one_step_ahead_with_requests_aborted_at_any_time(seed):
+    """Requests are aborted between the turns of the loop, also while the step in flight holds an entry of theirs and
+    after the step ahead was planned with one: what they sampled is dropped, their slot may go to the next request
+    at once, no page is lost, and every request that was not aborted gets the output it gets alone."""
+    rng = np.random.default_rng(500 + seed)
+    pages = 18
+    core = HostCore([(4, pages, 0)], max_requests=4, token_budget=int(rng.integers(6, 30)), max_chunk=int(rng.integers(0, 7)))
+    n = 16
+    prompts = [rng.integers(0, 50, int(rng.integers(1, 20))).tolist() for _ in range(n)]
+    news = [int(rng.integers(1, 12)) for _ in prompts]
+    stops = [rng.integers(0, 97, int(rng.integers(0, 6))).tolist() for _ in prompts]
+    doomed = {int(i): int(rng.integers(0, 8)) for i in rng.choice(n, 5, replace=False)}     # request -> turns it lives
+    d, slots, pending, done, age, aborted = AheadDriver(core), {}, list(range(n)), {}, {}, set()
+    for _ in range(5000):
+        while pending:
+            s = core.add_request(prompts[pending[0]], news[pending[0]], stop=stops[pending[0]])
+            if s < 0:
+                break
+            slots[s] = pending.pop(0)
+            age[slots[s]] = 0
+        if core.idle() and not pending and d.flight is None:
+            break
+        for s in d.step():
+            info = core.request_info(s)
+            done[slots.pop(s)] = (core.request_output(s), "stop" if info["finish"] == 1 else "length")
+            core.drop_request(s)
+        for s, r in list(slots.items()):
+            age[r] += 1
+            if r in doomed and age[r] > doomed[r]:
+                core.abort_request(s)
+                aborted.add(slots.pop(s))
+        held = sum(core.pages_held(s) for s in slots)
+        assert held + core.pages_free() == pages
+    assert sorted(list(done) + list(aborted)) == list(range(n)) and aborted
+    for i in done:
+        assert done[i] == alone(prompts[i], news[i], stops[i]), f"request {i}"
+    assert core.pages_free() == pages and core.slots_in_use() == 0 and not core.in_flight()
