@@ -298,6 +298,21 @@ def test_toy_architecture_with_a_stateful_mixer(dtype):
             assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), (cuts, i)
             eng.close_request(slots[i])
     assert eng.generate([seqs[1][:5]], max_new_tokens=4)[0] == eng.generate([seqs[1][:5]], max_new_tokens=4)[0]
+    # Through the scheduler, two slots for five requests, one step in flight while the next is planned against
+    # stepping in turn: a request that ends on a stop token has run one token more on the device (its state moved
+    # once more), and the request that takes its slot must find that state reset.
+    prompts = [seqs[0][:7], seqs[1][:3], seqs[0][10:31], seqs[1][5:6], seqs[0][40:44]]
+    outs = {}
+    for overlap in (False, True):
+        small = Engine(cfg, ws, dtype=dtype, page_size=16, num_pages=16, max_requests=2, overlap=overlap)
+        free = small.generate(prompts, max_new_tokens=12, temperature=0.8, seed=[1, 2, 3, 4, 5])
+        stop = next(t for toks in free for j, t in enumerate(toks) if j >= 2 and t not in toks[:j])
+        outs[overlap] = (free, small.generate(prompts, max_new_tokens=12, temperature=0.8, seed=[1, 2, 3, 4, 5],
+                                              stop_token_ids=[stop], return_reasons=True))
+        assert any(f.reason == "stop" and f.tokens for f in outs[overlap][1]), "the case itself"
+    if dtype == "float32":
+        assert outs[True][0] == outs[False][0]
+        assert [(f.tokens, f.reason) for f in outs[True][1]] == [(f.tokens, f.reason) for f in outs[False][1]]
 
 
 class RoutedLinear(FeedForward):
