@@ -116,10 +116,11 @@ class Model:
         for i, run in enumerate(self.spec.schedule):
             ctx.run_index = i
             block = self.blocks[run.layer]
-            # the norm that reads the stream after this block: the next block's first (the final norm reads
-            # gathered rows and runs as a kernel of its own)
+            # the norm that reads the stream after this block: the next block's first; after the last block the
+            # final norm, where it reads every row (else it reads gathered rows and runs as a kernel of its own)
             later = self.spec.schedule[i + 1] if i + 1 < len(self.spec.schedule) else None
-            ctx.norm_after_block = self.blocks[later.layer].first_norm() if later is not None else None
+            ctx.norm_after_block = (self.blocks[later.layer].first_norm() if later is not None
+                                    else self.final_norm if ctx.wants_every_row else None)
             block.forward(ctx, h, cache_views[i])
             if not block.keeps_left_current:
                 ctx.note_left(h, None)
@@ -128,8 +129,12 @@ class Model:
             return None
         # Norm only the wanted rows, then the output matrix: the reference norms all
         # rows and gathers after (src/arch/llama.rs:135-139), which is the same numbers.
-        x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
-        self.final_norm.forward(ctx, h, x, ctx.want_rows)
+        # (A step of few single tokens that wants them all: the last product has prepared the final norm, and the
+        # output matrix's product finishes it; no norm kernel runs.)
+        x = self.final_norm.deferred(ctx, h) if ctx.wants_every_row else None
+        if x is None:
+            x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
+            self.final_norm.forward(ctx, h, x, ctx.want_rows)
         logits = ctx.workspace("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
         k.gemm(x, self.head, logits, EPI_STORE_F32, ctx.gemm_workspace(x, self.head))
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:

@@ -78,6 +78,7 @@ class StepContext:
         # the part that runs now (its block says so); `norm_after_block` the one after the block (the model says so).
         self.upcoming_norm = None
         self.norm_after_block = None
+        self.wants_every_row = False
         self._left = None               # kernels.NextNorm that describes the stream as it stands, or None
         self._left_of = 0               # the stream it describes
         self._last_y = 0                # where the rows left last lie
@@ -247,10 +248,11 @@ class StepRunner:
             widths.append(cap)
         return widths
 
-    def _bind(self, dev: torch.Tensor, off, T: int, R: int, n_want: int, entries) -> StepContext:
+    def _bind(self, dev: torch.Tensor, off, T: int, R: int, n_want: int, entries, wants_all: bool = False) -> StepContext:
         c = self.ctx
         c.n_tokens, c.n_entries, c.n_want = T, R, n_want
         c.entries = entries
+        c.wants_every_row = bool(wants_all)       # the wanted rows are the step's rows, each once and in order
         c.max_seq_len = max(start + count for _, start, count in entries)
         c.single_lens = [start + 1 for _, start, count in entries if count == 1]
         c.n_single = len(c.single_lens)
@@ -301,7 +303,7 @@ class StepRunner:
         words = self._staging(self._estimate_words(T, R, len(want_rows), longest, widths))
         off = core.build_batch(slots, starts, counts, tokens, want_rows, words, fixed_widths=widths)
         dev = self._upload(off.words)
-        ctx = self._bind(dev, off, T, R, len(want_rows), list(zip(slots, starts, counts)))
+        ctx = self._bind(dev, off, T, R, len(want_rows), list(zip(slots, starts, counts)), want_rows == list(range(T)))
         return self._execute(ctx, widths)
 
     def run_planned(self, samples_in_flight: Optional[torch.Tensor] = None):
@@ -328,7 +330,8 @@ class StepRunner:
         words[off.words:off.words + n] = rows
         words[off.words + n:off.words + 2 * n] = sources
         dev = self._upload(off.words + 2 * n)
-        ctx = self._bind(dev, off, n_tokens, R, n_want, [(p[0], p[1], p[2]) for p in plan])
+        ctx = self._bind(dev, off, n_tokens, R, n_want, [(p[0], p[1], p[2]) for p in plan],
+                         all(p[2] == 1 and p[3] for p in plan))
         if n:
             from ..kernels import kernels
             kernels().place_ids(ctx.tokens, dev[off.words:off.words + n], dev[off.words + n:off.words + 2 * n],
