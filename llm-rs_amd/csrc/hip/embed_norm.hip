@@ -1,6 +1,24 @@
 // Token embedding into the 32-bit residual stream, and RMSNorm out of it.
 #include "common.h"
 
+typedef float embed_f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 embed_bf16x8 __attribute__((ext_vector_type(8)));
+
+// Eight values of a 16-bit row as one 16-byte load, widened and scaled (rows of a multiple of 8 values, 16-byte aligned).
+__device__ __forceinline__ void load8_scaled(const bf16* src, float scale, float (&v)[8]) {
+    embed_bf16x8 raw = *(const embed_bf16x8*)src;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = (float)raw[j] * scale;
+}
+__device__ __forceinline__ void store8(float* dst, const float (&v)[8]) {
+    *(embed_f32x4*)dst = embed_f32x4{v[0], v[1], v[2], v[3]};
+    *(embed_f32x4*)(dst + 4) = embed_f32x4{v[4], v[5], v[6], v[7]};
+}
+template <class T>
+__device__ __forceinline__ bool rows_by_eights(const T* table, const float* out, int D) {
+    return sizeof(T) == 2 && D % 8 == 0 && ((uintptr_t)table & 15) == 0 && ((uintptr_t)out & 15) == 0;
+}
+
 // out[t, :] = float(table[tokens[t], :]) * scale   (reference: embed_batch_*, shaders/ops.metal:878-915,
 // which has no scale: 1 there and for every architecture that does not ask for one)
 template <class T>
@@ -11,6 +29,16 @@ __global__ void embed_rows_kernel(float* __restrict__ out, const T* __restrict__
     row = row < 0 ? 0 : (row >= V ? V - 1 : row);  // the host has checked ids; never read outside the table
     const T* src = table + (size_t)row * D;
     float* dst = out + (size_t)t * D;
+    if constexpr (sizeof(T) == 2) {
+        if (rows_by_eights(table, out, D)) {           // (the same in all threads)
+            for (int d = threadIdx.x * 8; d < D; d += blockDim.x * 8) {
+                float v[8];
+                load8_scaled((const bf16*)src + d, scale, v);
+                store8(dst + d, v);
+            }
+            return;
+        }
+    }
     for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = to_f32(src[d]) * scale;
 }
 

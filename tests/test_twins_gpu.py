@@ -51,10 +51,11 @@ def close(pair, floor=1e-6, sums_of=0):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_embed_rows(dtype):
-    table = rnd((1001, 328), dtype, 1)
+@pytest.mark.parametrize("D", [328, 35, 4096])
+def test_embed_rows(dtype, D):
+    table = rnd((1001, D), dtype, 1)
     tokens = torch.randint(0, 1001, (37,), generator=torch.Generator().manual_seed(2)).to(torch.int32)
-    (pair,) = both("embed_rows", [torch.zeros((37, 328)), table, tokens, 0.7], [0])
+    (pair,) = both("embed_rows", [torch.zeros((37, D)), table, tokens, 0.7], [0])
     assert torch.equal(*pair)
 
 
