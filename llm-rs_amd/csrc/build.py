@@ -30,6 +30,15 @@ HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={GPU_ARCH}",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-pthread", "-ffp-contract=off"]
+# LLMRS_SANITIZE=1 in the environment: the two g++ libraries (raw-pointer C interfaces fed through ctypes) are built
+# with the address and undefined-behaviour sanitizers, under names of their own beside the ordinary ones.  A Python
+# that loads them needs the address sanitizer's runtime loaded first: `sanitizer_env()` gives the variables to start
+# it with.  The kernel library is never built this way (there is no sanitizer for the device on these machines).
+SANITIZE = os.environ.get("LLMRS_SANITIZE", "") not in ("", "0")
+SANITIZE_FLAGS = ["-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer", "-g", "-O1"]
+if SANITIZE:
+    HOST_FLAGS = HOST_FLAGS + SANITIZE_FLAGS
+_SUFFIX = "_san" if SANITIZE else ""
 
 
 class BuildError(RuntimeError):
@@ -47,7 +56,7 @@ def _digest(sub: str) -> str:
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIP_FLAGS + HOST_FLAGS).encode())
+    h.update(" ".join(HIP_FLAGS if sub == "hip" else HOST_FLAGS).encode())
     return h.hexdigest()
 
 
@@ -92,7 +101,7 @@ def _finish(lib: str, tmp: str, sub: str) -> None:
 
 def build_host(force: bool = False) -> str:
     d = _build_dir()
-    lib = os.path.join(d, "libllmrs_host.so")
+    lib = os.path.join(d, f"libllmrs_host{_SUFFIX}.so")
     if not force and _is_current(lib, "host"):
         return lib
     cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
@@ -108,7 +117,7 @@ def build_host(force: bool = False) -> str:
 def build_plain(force: bool = False) -> str:
     """The kernels' plain C++ twins (test equipment: the package has no CPU path and never loads them)."""
     d = _build_dir()
-    lib = os.path.join(d, "libllmrs_plain.so")
+    lib = os.path.join(d, f"libllmrs_plain{_SUFFIX}.so")
     if not force and _is_current(lib, "plain"):
         return lib
     cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("clang++")
@@ -119,6 +128,28 @@ def build_plain(force: bool = False) -> str:
     _run([cxx, *HOST_FLAGS, "-shared", "-o", tmp, *_sources("plain", (".cpp",))], "plain twins build")
     _finish(lib, tmp, "plain")
     return lib
+
+
+def sanitizer_env(env=None) -> dict:
+    """The environment to start a Python in that is to load the sanitized host libraries: LLMRS_SANITIZE set, the
+    address sanitizer's runtime first among the preloaded libraries (whatever was there stays behind it), and no
+    leak report at exit (the interpreter itself never frees much of what it allocates)."""
+    env = dict(os.environ if env is None else env)
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise BuildError("no g++ to ask for the sanitizer's runtime")
+    runtime = subprocess.run([cxx, "-print-file-name=libasan.so"], capture_output=True, text=True).stdout.strip()
+    if not os.path.isabs(runtime) or not os.path.exists(runtime):
+        raise BuildError("this compiler has no address sanitizer runtime (libasan.so)")
+    # (the C++ runtime too: the sanitizer looks up the real `__cxa_throw` when it starts, and an interpreter that is
+    # not itself linked against libstdc++ has none to show then, so the first exception inside a library would abort)
+    cxxlib = subprocess.run([cxx, "-print-file-name=libstdc++.so.6"], capture_output=True, text=True).stdout.strip()
+    env["LLMRS_SANITIZE"] = "1"
+    env["LD_PRELOAD"] = ":".join(x for x in (os.path.realpath(runtime), os.path.realpath(cxxlib) if os.path.isabs(cxxlib) else "",
+                                             env.get("LD_PRELOAD", "")) if x)
+    env["ASAN_OPTIONS"] = "detect_leaks=0:abort_on_error=1:" + env.get("ASAN_OPTIONS", "")
+    env["UBSAN_OPTIONS"] = "print_stacktrace=1:halt_on_error=1:" + env.get("UBSAN_OPTIONS", "")
+    return env
 
 
 def _hipcc() -> Optional[str]:

@@ -341,7 +341,7 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (a.head_dim + 2) * sizeof(float);
     bool split = max_chunks > 0 && scratch != nullptr && q_starts != nullptr && seq_lens != nullptr &&
                  scratch_bytes >= need && n_single != 0 && n_entries <= 65535 && max_chunks <= 65535;
-    bool only_single = split && a.n_tokens == n_entries;     // every entry brings one token
+    bool only_single = split && n_single == n_entries && a.n_tokens == n_entries;     // every entry brings one token: the caller says so
     const int G = a.n_heads / a.n_kv_heads;
     const bool groupable = a.head_dim <= GROUP_MAX_HEAD_DIM && (G == 2 || G == 4 || G == 8);
     bool tiles_took = false;
@@ -405,7 +405,8 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
 // scratch: device memory for the partial results of single-token entries, which
 // are split over waves by key range (may be null: then they are not split);
 // max_seq_len: an upper bound of seq_lens that the host knows (0: unknown, no split);
-// n_single: how many entries bring one token, if the host knows (-1: it does not);
+// n_single: how many entries bring one token, if the host knows (-1: it does not); n_single == n_entries is the
+// caller's word that every entry brings exactly one token (then token t is entry t, and q_starts is not read);
 // single_keys: how many keys those entries see together (windows counted), if the host knows (0: it does not):
 // the matrix-core kernels choose the keys per wave by it.
 extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int q_stride, void* out, int out_stride,
@@ -422,6 +423,9 @@ extern "C" int llmrs_attention(hipStream_t stream, int dtype, const void* q, int
     LLMRS_REQUIRE(q_stride >= n_heads * head_dim && out_stride >= n_heads * head_dim, "attention: row stride too short");
     LLMRS_REQUIRE(window >= 0, "attention: negative window");
     LLMRS_REQUIRE(n_heads <= 65535, "attention: too many heads for one launch");
+    LLMRS_REQUIRE(n_single <= n_entries, "attention: %d single-token entries among %d entries", n_single, n_entries);
+    LLMRS_REQUIRE(n_single != n_entries || n_tokens == n_entries,
+                  "attention: every entry is said to bring one token, but %d entries bring %d tokens", n_entries, n_tokens);
     if (n_tokens == 0) return 0;
     AttnArgs a{n_tokens, n_heads, n_kv_heads, head_dim, page_size, table_width, num_pages, q_stride, out_stride, window, scale};
     if (dtype == LLMRS_BF16 && allow_mfma) {

@@ -1043,7 +1043,9 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     size_t need = (size_t)n_entries * a.n_heads * max_chunks * (HD + 2) * sizeof(float);
     // Split the single-token entries when the caller gave room for their partial results.
     int split = max_chunks > 0 && scratch != nullptr && seq_lens != nullptr && scratch_bytes >= need && max_chunks <= MERGE_MAX_CHUNKS && n_single != 0;
-    int only_single = split && a.n_tokens == n_entries;   // every entry brings one token: no tile work
+    // every entry brings one token, on the caller's word (n_single == n_entries): no tile work.  It is not read off
+    // n_tokens == n_entries, which entries of two tokens and of none would satisfy as well.
+    int only_single = split && n_single == n_entries && a.n_tokens == n_entries;
     // both kinds of work: the single tokens' kernels on the second stream, beside the tiles
     hipStream_t single_stream = stream;
     SideStream* side = nullptr;

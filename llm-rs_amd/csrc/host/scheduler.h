@@ -24,8 +24,13 @@
 // turn out: a request that ends on a stop token has run one token for nothing,
 // its entry in the step ahead is marked dead and its sample dropped.  Nothing is
 // preempted while a step is in flight; a plan that finds no pages comes back
-// empty and the caller commits the step in flight first.  Tokens, their order
-// and each request's random draws are the same as without.
+// empty and the caller commits the step in flight first.  Which tokens run in
+// which order, and each request's random draws, are the same as without.  The
+// logits are the same up to what the kernels make of a step's row count: a dead
+// row makes the step one row larger than the step taken in turn, and where that
+// crosses a boundary between kernels (16 to 17 rows, say) the live rows are
+// rounded in another order, so that in bfloat16 a greedy near-tie can fall the
+// other way.
 #pragma once
 #include <cstdint>
 #include <deque>

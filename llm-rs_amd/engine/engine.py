@@ -296,6 +296,10 @@ class Engine:
             if flight.landed is not None:
                 flight.landed.synchronize()
             sampled = flight.host.numpy().copy()
+            # A sampler or hand-over fault must not go on as "the request decodes from token 0": fail here.
+            vocab = self.model.spec.vocab_size
+            if len(sampled) and (int(sampled.min()) < 0 or int(sampled.max()) >= vocab):
+                raise RuntimeError(f"a step sampled token ids outside [0, {vocab}): {int(sampled.min())}..{int(sampled.max())}")
         finished = set(core.commit(sampled))
         out: List[Emitted] = []
         for (slot, request), token in zip(flight.owners, sampled):
@@ -322,11 +326,17 @@ class Engine:
             core.launch()
         # the step after it, before this one's samples are known (nothing, when all it could run waits for pages
         # or for those samples: then the next call starts afresh)
-        ahead = self._start_step(self._flight)
-        out = self._land_step(self._flight)
-        self._flight = ahead
-        if ahead is not None:
-            core.launch()
+        landing, ahead = self._flight, self._start_step(self._flight)
+        try:
+            out = self._land_step(landing)
+        finally:
+            # Whatever happens while the first step lands (an interrupt included), engine and scheduler go on
+            # agreeing about which step is in flight: the one that was started ahead, once the scheduler has
+            # taken the landed one (commit), or still the first one if it has not.
+            if not core.in_flight():
+                self._flight = ahead
+                if ahead is not None:
+                    core.launch()
         self._admit()
         return out
 
@@ -395,8 +405,9 @@ class Engine:
         except BaseException:
             for r in index_of:                  # leave the engine as it was found
                 self.cancel(r)
-            if self._flight is not None:        # (every entry of the step in flight is dead now: its samples are dropped)
-                flight, self._flight = self._flight, None
+            flight, self._flight = self._flight, None
+            if flight is not None and self.cache.core.in_flight():
+                # (every entry of the step in flight is dead now: its samples are dropped)
                 self.cache.core.commit([0] * len(flight.owners))
             raise
         if self.device.type == "cuda":

@@ -73,16 +73,22 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold at any time, each rounded up to a multiple of 64")
     ap.add_argument("--page-size", type=int, default=16)
     args = ap.parse_args(argv)
-    os.makedirs(args.out, exist_ok=True)
     replayer = TraceReplayer(args.model, args.dtype, args.max_tokens, page_size=args.page_size)
-    for line in sys.stdin:
+    return replay_lines(replayer, sys.stdin, args.out)
+
+
+def replay_lines(replayer: TraceReplayer, lines, out_dir: str) -> int:
+    """Steps as JSON objects, one a line; `<step>.f32` into `out_dir` for every step that wants rows, and a line
+    `done <step>` on standard output after every step."""
+    os.makedirs(out_dir, exist_ok=True)
+    for line in lines:
         line = line.strip()
         if not line:
             continue
         record = json.loads(line)
         logits = replayer.step(record)
         if logits is not None and logits.shape[0] > 0:
-            logits.tofile(os.path.join(args.out, f"{record['step']}.f32"))
+            logits.tofile(os.path.join(out_dir, f"{record['step']}.f32"))
         elif torch.cuda.is_available():
             torch.cuda.synchronize()
         print(f"done {record['step']}", flush=True)

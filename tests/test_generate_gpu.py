@@ -202,6 +202,42 @@ def test_steps_started_ahead_change_no_output(folders, which, dtype):
     assert run(True, 0.8, [], **tight_kw)[0] == in_turn
 
 
+def test_a_dead_row_beside_sixteen_live_ones_moves_logits_by_rounding_only():
+    """A step started ahead carries a row for a request that a stop token has just ended, so sixteen live requests
+    run as a step of seventeen rows where stepping in turn runs sixteen; and the kernels choose by the row count (up to
+    sixteen rows the norms are finished by the neighbouring products, from seventeen on by a norm kernel or by the
+    product that is split over blocks).  The live rows' logits may differ between the two by rounding, not more:
+    both are compared with the plain implementation and with each other, in bfloat16 and in float32."""
+    from llm_rs_amd import LlamaConfig
+    cfg = LlamaConfig.from_dict(dict(
+        architectures=["LlamaForCausalLM"], num_hidden_layers=2, hidden_size=2048, num_attention_heads=16,
+        num_key_value_heads=4, head_dim=128, intermediate_size=4096, vocab_size=1000, rope_theta=500000.0,
+        max_position_embeddings=512, rms_norm_eps=1e-5, tie_word_embeddings=False))
+    plen, n_live = 40, 16
+    prompts = [random_tokens(1000, plen + 1, seed=500 + i) for i in range(n_live + 1)]
+    weights = None
+    for dtype in ("bfloat16", "float32"):
+        eng = Engine.from_random(cfg, 9, dtype=dtype, page_size=16, num_pages=128, max_requests=32)
+        if weights is None:
+            weights = eng.weights()
+        slots = [eng.open_request() for _ in prompts]
+        for s, p in zip(slots, prompts):
+            eng.step([StepEntry(s, 0, p[:plen], [])])
+        decode = lambda n: [StepEntry(slots[i], plen, [prompts[i][plen]], [0]) for i in range(n)]
+        in_turn = eng.step(decode(n_live)).double().cpu().clone()
+        # the dead row stands in the middle, as a request that ended does, not at the end
+        order = list(range(8)) + [n_live] + list(range(8, n_live))
+        with_dead = eng.step([decode(n_live + 1)[i] for i in order]).double().cpu().clone()
+        with_dead = with_dead[[order.index(i) for i in range(n_live)]]
+        plain = torch.stack([plain_forward(cfg.to_dict(), {n: t.double() for n, t in weights.items()}, p)[-1] for p in prompts[:n_live]])
+        allowed = tolerance_for(dtype, cfg.to_dict(), weights, prompts[:3])
+        scale = logit_scale(plain)
+        for name, a, b in (("in turn", in_turn, plain), ("with a dead row", with_dead, plain), ("one against the other", in_turn, with_dead)):
+            err = float((a - b).abs().max()) / scale
+            assert err <= allowed, f"{dtype}, {name}: {err:.3e} of the largest logit, allowed {allowed:.3e}"
+            note(dtype, err)
+
+
 @pytest.mark.parametrize("which,dtype", [("B", "bfloat16"), ("A", "float32")])
 def test_recorded_decode_steps_equal_eager_ones(folders, which, dtype):
     """Decode steps are recorded into a HIP graph and replayed.  Every replay is compared

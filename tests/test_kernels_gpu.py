@@ -6,7 +6,7 @@ import math
 import pytest
 import torch
 
-from llm_rs_amd.kernels import EPI_ACCUM_F32, EPI_STORE, EPI_STORE_F32, EPI_SWIGLU, kernels
+from llm_rs_amd.kernels import EPI_ACCUM_F32, EPI_STORE, EPI_STORE_F32, EPI_SWIGLU, KernelError, kernels
 from plain_llama import plain_attention, plain_inv_freq, plain_rmsnorm, plain_rope, plain_silu
 
 pytestmark = pytest.mark.gpu
@@ -250,14 +250,15 @@ class PagedCase:
         T = q.shape[0]
         entry = torch.cat([torch.full((len(p),), r, dtype=torch.int32) for r, p in enumerate(q_pos_list)]).to(DEV)
         pos = torch.cat([torch.tensor(p, dtype=torch.int32) for p in q_pos_list]).to(DEV)
+        lens_now = [max(p) + 1 if len(p) else 1 for p in q_pos_list]      # (an entry without tokens: any length will do)
         counts = [len(p) for p in q_pos_list]
         q_starts = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
-        seq_lens = torch.tensor([max(p) + 1 for p in q_pos_list], dtype=torch.int32, device=DEV)
+        seq_lens = torch.tensor(lens_now, dtype=torch.int32, device=DEV)
         out = torch.zeros((T, self.n_heads * self.hd), dtype=self.dtype, device=DEV)
         scratch = torch.empty(scratch_floats, dtype=torch.float32, device=DEV)
         kernels().attention(q, out, self.kc.to(DEV), self.vc.to(DEV), self.tables.to(DEV), entry, pos, q_starts, seq_lens,
                             self.n_heads, self.n_kv, self.hd, self.ps, self.num_pages, window, scale, scratch,
-                            max(max(p) + 1 for p in q_pos_list) if bound is None else bound, n_single, single_keys)
+                            max(lens_now) if bound is None else bound, n_single, single_keys)
         return out.cpu().view(T, self.n_heads, self.hd)
 
     def reference(self, r, q, positions, window=0, scale=None):
@@ -279,6 +280,31 @@ class PagedCase:
             o = plain_attention(qq, self.k[r][:n].double(), self.v[r][:n].double(), scale, window)
             outs.append(o[-1])
         return torch.stack(outs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps", [(8, 2, 128, 16), (6, 3, 48, 8)])
+def test_attention_as_many_tokens_as_entries_but_not_one_each(dtype, n_heads, n_kv, hd, ps):
+    """Entries of two tokens and of none come to as many tokens as entries, as single tokens would: the kernels
+    treat a batch as single tokens only on the caller's word (n_single == n_entries), never by that count, and a
+    caller that claims it for such a batch is refused."""
+    lens = [40, 25, 9, 33]
+    case = PagedCase(dtype, lens, n_heads, n_kv, hd, ps, seed=3)
+    g = torch.Generator().manual_seed(2)
+    q_pos = [[38, 39], [], [7, 8], []]
+    qs = [torch.randn((len(p), n_heads, hd), generator=g).to(dtype) for p in q_pos]
+    floor = 2e-6 if dtype == torch.float32 else 4e-3
+    for n_single in (-1, 0):
+        got = case.run(qs, q_pos, n_single=n_single)
+        at = 0
+        for r, p in enumerate(q_pos):
+            if p:
+                ref = case.reference(r, qs[r], p)
+                err = (got[at:at + len(p)].double() - ref).abs()
+                assert (err <= out_tol(ref, dtype, floor)).all(), f"n_single {n_single}, entry {r}: max err {float(err.max())}"
+                at += len(p)
+    with pytest.raises(KernelError, match="every entry is said to bring one token"):
+        case.run([qs[0], qs[2]], [q_pos[0], q_pos[2]] , n_single=2)      # two entries, four tokens
 
 
 ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 16), (8, 8, 64, 16), (8, 2, 128, 16), (6, 3, 48, 8), (5, 1, 80, 16),

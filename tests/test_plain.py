@@ -167,3 +167,45 @@ def test_xorshift_constants():
     assert g.state == 0xDEADBEEFCAFE                      # src/sampler/mod.rs:10
     g = PlainXorshift(1)
     assert g.next_u64() == 1082269761 and 0.0 <= g.next_f32() < 1.0   # 1 ^ 1<<13 -> ^ >>7 -> ^ <<17
+
+
+# Figures that were not made by this repository's code.  A reviewer computed them in float64 with an independent
+# implementation of the Llama decoder (files in the HF layout: split-half rotation pairs, llama3 frequency scaling)
+# from the tensors `random_model_tensors(cfg, 3)` and the tokens [(7 i + 3) mod vocab for i < 40], and handed over
+# the numbers alone.  They pin the two things the reference's own files do not contain: the pairing of rotation
+# under HF tensor names (the reference runs files converted to neighbouring pairs, src/arch/llama.rs:156,
+# src/tensor/mod.rs:133-139) and the llama3 scaling of the frequencies (the reference scales nothing,
+# shaders/ops.metal:1030).  Rotating neighbouring pairs on these files, or blending along the wavelength, fails them.
+OUTSIDE_LOGITS = {
+    "A": (TINY_A, {0: 0.101146, 1: -0.197046, 2: 0.007545, 128: -0.116913, 255: -0.016560}, 20, 109),
+    "B": (TINY_B, {0: -0.182026, 1: 0.096695, 2: -0.054555, 192: -0.153350, 383: -0.267057}, 123, 325),
+}
+OUTSIDE_INV_FREQ = [     # (rotary width, factor, original length) -> {pair: frequency}; theta 5e5, low 1, high 4
+    (32, 8.0, 64, {4: 0.004700753837823868, 8: 0.00017677668074611574, 12: 6.647869668086059e-06, 15: 5.677088097399974e-07}),
+    (128, 8.0, 8192, {16: 0.03760603070259094, 32: 0.0005248460220173001, 48: 6.647869668086059e-06, 63: 3.068925877869333e-07}),
+    (64, 32.0, 8192, {16: 0.000429556705057621, 24: 1.6619674170215148e-06, 31: 9.418306490260875e-08}),
+]
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_logits_computed_outside_this_repository(which):
+    cfg, last_row, last_argmax, first_argmax = OUTSIDE_LOGITS[which]
+    weights = random_model_tensors(LlamaConfig.from_dict(cfg), 3)
+    tokens = [(7 * i + 3) % cfg["vocab_size"] for i in range(40)]
+    logits = plain_forward(cfg, weights, tokens)
+    for i, want in last_row.items():
+        assert abs(float(logits[-1, i]) - want) < 2e-6, (i, float(logits[-1, i]), want)
+    assert int(logits[-1].argmax()) == last_argmax and int(logits[0].argmax()) == first_argmax
+    # the mistakes these figures are there to catch do move them
+    wrong = plain_forward(cfg, weights, tokens, layout="interleaved")
+    assert max(abs(float(wrong[-1, i]) - want) for i, want in last_row.items()) > 1e-4
+
+
+@pytest.mark.parametrize("width,factor,length,want", OUTSIDE_INV_FREQ)
+def test_llama3_frequencies_computed_outside_this_repository(width, factor, length, want):
+    from llm_rs_amd.parts import rope_inv_freq
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=length)
+    for table in (plain_inv_freq(width, 5e5, sc), rope_inv_freq(width, 5e5, sc)):
+        for i, f in want.items():
+            assert abs(float(table[i]) / f - 1) < 1e-6, (i, float(table[i]), f)

@@ -46,14 +46,44 @@ def test_argmax_rows_static_follows_argmax_rows():
                                    caller_scratch.data_ptr(), caller_scratch.numel())
         assert rc == 0, lib.llmrs_hip_error().decode()
         torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated()
+        # the driver's own figure of free memory: it moves with any hipMalloc or hipFree, whoever calls it
+        # (torch's counters see only what goes through torch's allocator)
+        before = torch.cuda.mem_get_info()[0]
         rc = lib.llmrs_argmax_rows_static(stream, x.data_ptr(), x.stride(0), rows, V, got.data_ptr())
         assert rc == 0, lib.llmrs_hip_error().decode()
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert torch.cuda.mem_get_info()[0] == before
         assert torch.equal(got, want), (rows, V)
         first_max = (x == x.max(dim=1, keepdim=True).values).int().argmax(dim=1).to(torch.int32)
         assert torch.equal(got, first_max)
+
+
+def test_argmax_rows_static_inside_a_recorded_graph():
+    """The use the entry point is there for: one call with no rows before the recording (it looks the array's
+    address up), then calls while a stream is being captured, where any allocation would end the capture with an
+    error.  The graph is replayed on new logits, with other work and synchronisations between the replays, and
+    every replay compared with the existing entry point."""
+    lib = _lib()
+    rows, V = 19, 50000
+    x = _logits(rows, V, 5)
+    got = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
+    want = torch.empty(rows, dtype=torch.int32, device="cuda")
+    caller_scratch = torch.empty(rows * 32 * 8, dtype=torch.uint8, device="cuda")
+    assert lib.llmrs_argmax_rows_static(torch.cuda.current_stream().cuda_stream, None, V, 0, V, None) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = lib.llmrs_argmax_rows_static(torch.cuda.current_stream().cuda_stream, x.data_ptr(), x.stride(0), rows, V, got.data_ptr())
+    assert rc == 0, lib.llmrs_hip_error().decode()
+    for replay in range(4):
+        x.copy_(_logits(rows, V, 10 + replay))
+        rc = lib.llmrs_argmax_rows(torch.cuda.current_stream().cuda_stream, x.data_ptr(), x.stride(0), rows, V, want.data_ptr(),
+                                   caller_scratch.data_ptr(), caller_scratch.numel())
+        assert rc == 0, lib.llmrs_hip_error().decode()
+        got.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {replay}"
 
 
 def test_argmax_rows_static_refuses_more_rows_than_its_array_holds():
