@@ -108,7 +108,7 @@ def decode_line(args, layers, step_s, weight_bytes, cache_bytes_per_token, prefi
     T = args.prefill_tokens
     line = base_line(
         f"decode tok/s at batch {args.batch} (8B {short}); prefill tok/s at {T} tokens"
-        + (f" and batch {'/'.join(p.split('_b')[1] for p in points)}" if points else "") + " alongside",
+        + (f" and batch {'/'.join(p.split('_b')[1] for p in points if '_ctx' not in p and p != 'decode_b256')}" if points else "") + " alongside",
         args.batch / step_s, args.steps, args.warmup, step_s, args.dtype,
         flat_config("Llama-3.1-8B shape", layers, args.batch, args.context, 16, prefill_tokens=T))
     line["prefill"] = {"value": round(T / prefill_s, 1), "tokens": T, "ms": round(prefill_s * 1e3, 3),
@@ -190,9 +190,7 @@ def prompts_line(args, layers, points, fractions, first_step_s=0.0) -> dict:
 # ---- measurements (need the GPU) -------------------------------------------------------------------------------
 
 class Bench:
-    def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int, side_by_side: bool = False):
-        """`side_by_side`: a request's portion of a step is capped so that `max_requests` prompts of one length run
-        side by side and end in the same step (for `decode_run`, whose requests then decode over equal contexts)."""
+    def __init__(self, args, shape: dict, num_pages: int, max_requests: int, max_batch_tokens: int):
         import torch
         from llm_rs_amd import Engine, LlamaConfig
         self.torch = torch
@@ -202,8 +200,8 @@ class Bench:
         self.config = LlamaConfig.from_dict(d)
         t0 = time.time()
         self.engine = Engine.from_random(self.config, seed=0, dtype=args.dtype, device="cuda:0", page_size=16,
-                                         num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens,
-                                         max_chunk=max(1, max_batch_tokens // max_requests) if side_by_side else 0)
+                                         num_pages=num_pages, max_requests=max_requests, max_batch_tokens=max_batch_tokens)
+        self.max_batch_tokens = max_batch_tokens
         torch.cuda.synchronize()
         print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
         self.gen = torch.Generator().manual_seed(0)
@@ -246,6 +244,9 @@ class Bench:
         (submit / advance: the scheduler, one step in flight while the next is planned), and the device's share."""
         engine = self.engine
         measured = min(steps, 16) if with_device_time else 0
+        # a request's portion of a step is capped so that the `batch` prompts, all of one length, run side by side
+        # and end in the same step: the requests then decode over equal contexts
+        engine.cache.core.set_max_chunk(max(1, self.max_batch_tokens // batch))
         requests = [engine.submit(self.prompt(context), max_new_tokens=warmup + steps + measured + 4) for _ in range(batch)]
         for _ in range(context * batch + 8):        # the prompts, in equal portions side by side: they end in the same step
             if len(engine.advance()) == batch:
@@ -265,15 +266,18 @@ class Bench:
             engine.cancel(r)
         while engine.has_unfinished():              # (the step in flight lands; what it sampled is nobody's)
             engine.advance()
+        engine.cache.core.set_max_chunk(0)
         return sec, dev
 
 
 def run_decode8b(args) -> dict:
     from llm_rs_amd import StepEntry
-    points = [int(p) for p in args.points.split(",") if p]
-    max_batch = max([args.batch] + points)
-    ctx_pages = -(-(args.context + args.steps + args.warmup + 24) // 16)
-    b = Bench(args, LLAMA_8B, max_batch * ctx_pages + 8, max(max_batch, 8), max(args.prefill_tokens, 2048), side_by_side=True)
+    # further points: "batch" (at --context) or "batch@context"
+    points = [(int(p.split("@")[0]), int(p.split("@")[1]) if "@" in p else args.context) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + [bt for bt, _ in points])
+    pages_for = lambda bt, ctx: bt * (-(-(ctx + args.steps + args.warmup + 24) // 16))
+    b = Bench(args, LLAMA_8B, max([pages_for(args.batch, args.context)] + [pages_for(bt, ctx) for bt, ctx in points]) + 8,
+              max(max_batch, 8), max(args.prefill_tokens, 2048))
     engine = b.engine
     toks = b.prompt(args.prefill_tokens)
 
@@ -289,13 +293,19 @@ def run_decode8b(args) -> dict:
         return {"prefill_ms": round(prefill_s * 1e3, 3), "tokens": args.prefill_tokens}
     step_s, dev_s = b.decode_run(args.batch, args.context, args.steps, args.warmup, with_device_time=True)
     print(f"[bench] decode batch {args.batch}: {step_s * 1e3:.3f} ms/step (device {dev_s * 1e3:.3f})", file=sys.stderr, flush=True)
-    point_values = {}
-    for p in points:
-        s, _ = b.decode_run(p, args.context, max(args.steps // 2, 8), max(args.warmup // 2, 2))
-        point_values[f"decode_b{p}"] = round(p / s, 1)
-        print(f"[bench] decode batch {p}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
-    return decode_line(args, b.config.num_hidden_layers, step_s, engine.model.weight_bytes_per_step(),
-                       engine.cache.bytes_per_token(), prefill_s, point_values, host_share(step_s, dev_s))
+    point_values, point_fracs = {}, {}
+    weight_bytes, per_token = engine.model.weight_bytes_per_step(), engine.cache.bytes_per_token()
+    for bt, ctx in points:
+        steps, warmup = max(args.steps // 2, 8), max(args.warmup // 2, 2)
+        s, _ = b.decode_run(bt, ctx, steps, warmup)
+        key = f"decode_b{bt}" + (f"_ctx{ctx}" if ctx != args.context else "")
+        point_values[key] = round(bt / s, 1)
+        point_fracs[key] = round((weight_bytes + bt * (ctx + warmup + steps // 2) * per_token) / s / PEAK_HBM, 4)
+        print(f"[bench] decode batch {bt} at context {ctx}: {s * 1e3:.3f} ms/step, {point_fracs[key] * 100:.1f}% of the HBM roofline",
+              file=sys.stderr, flush=True)
+    line = decode_line(args, b.config.num_hidden_layers, step_s, weight_bytes, per_token, prefill_s, point_values, host_share(step_s, dev_s))
+    line["points_frac"] = point_fracs
+    return line
 
 
 def run_sizes(args) -> dict:
@@ -305,7 +315,7 @@ def run_sizes(args) -> dict:
     small = args.workload == "sizes1b"
     cases = [(1, 2048), (8, 2048), (64, 2048)] if small else [(1, long), (8, long), (64, long), (128, 2048), (256, 2048)]
     pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
-    b = Bench(args, LLAMA_1B if small else LLAMA_8B, pages, 256, 2048, side_by_side=True)
+    b = Bench(args, LLAMA_1B if small else LLAMA_8B, pages, 256, 2048)
     weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
     points, fractions, first_s = {}, {}, None
     for batch, ctx in cases:
@@ -324,7 +334,7 @@ def run_long(args) -> dict:
     shape = dict(LLAMA_8B, max_position_embeddings=131072)
     cases = [(1, 131072 - 64), (4, 32768 - 64)]
     pages = max(bt * (-(-(ctx + steps + warmup + 24) // 16)) for bt, ctx in cases) + 8
-    b = Bench(args, shape, pages, 8, 2048, side_by_side=True)
+    b = Bench(args, shape, pages, 8, 2048)
     weight_bytes, per_token = b.engine.model.weight_bytes_per_step(), b.engine.cache.bytes_per_token()
     points, fractions, first_s = {}, {}, None
     for batch, ctx in cases:
@@ -423,7 +433,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--points", default="1,64", help="other decode batch sizes to report (decode8b)")
+    ap.add_argument("--points", default="1,64,256,1@8128,64@8128",
+                    help="other decode points to report (decode8b): batch sizes at --context, or batch@context")
     ap.add_argument("--only", default="", choices=["", "prefill", "decode"], help="for profiling: time one phase only (decode8b)")
     ap.add_argument("--requests", type=int, default=256, help="serve1b: requests submitted at once")
     ap.add_argument("--new-tokens", type=int, default=256, help="serve1b: tokens generated for each request")

@@ -1,53 +1,67 @@
 """The cache a model's runs need, on the device, and the host core that hands
 out its pages.
 
-Every run of the schedule whose mixer asks for `PagedKV` gets a cache layer;
-layers with equal needs (kv heads, head size, window) form a group that shares a
-page pool and block tables, so one page id names the same slots in every layer
+Every run of the schedule whose mixer asks for a paged need (`PagedKV`, or any class
+registered as a paged kind) gets a cache layer; layers with equal needs form a group that
+shares a page pool and block tables, so one page id names the same slots in every layer
 of its group (as one block id does in all layers of the reference's pool,
 src/kv_pool.rs:37-42).  A run that reads another run's cache shares that run's
-layer and writes nothing.  `FixedState` needs become one tensor per run with a
-row for every request slot.
-
-Layout of a group (csrc/hip/cache_layout.h):
-  keys   [layer][page][kv_head][slot][head_dim]
-  values [layer][page][kv_head][head_dim][slot]
+layer and writes nothing.  Per-request needs (`FixedState`) become memory with a
+row for every request slot.  How a need is laid out is its kind's business (cache/spec.py).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Optional, Sequence, Tuple, Union
+from typing import Any, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from .native import HostCore
-from .spec import FixedState, PagedKV
-
-
-@dataclass
-class CacheView:
-    """What one run's mixer sees of the cache."""
-    kind: str                       # "paged", "state" or "none"
-    group: int = -1                 # index into the step's slot maps and block tables
-    k: Optional[torch.Tensor] = None
-    v: Optional[torch.Tensor] = None
-    page_size: int = 0
-    num_pages: int = 0
-    writes: bool = True
-    state: Optional[torch.Tensor] = None   # [max_requests, *shape]
+from .spec import CacheKind, CacheView, cache_kind
 
 
 @dataclass
 class PagedGroup:
-    need: PagedKV
+    need: Any
+    kind: CacheKind
     page_size: int
     num_pages: int
     n_layers: int
-    k: torch.Tensor
-    v: torch.Tensor
+    storage: Any
+    dtype: torch.dtype
 
     def bytes_per_token(self) -> int:
-        return 2 * self.n_layers * self.need.kv_heads * self.need.head_dim * self.k.element_size()
+        return self.n_layers * self.kind.bytes_per_token(self.need, self.dtype)
+
+
+def _group_runs(needs: Sequence[Tuple[object, Optional[int]]]):
+    """(the distinct paged needs, layers in each, (group, layer) of every run or None, the runs with per-request needs)."""
+    group_needs: List[Any] = []
+    layers_in_group: List[int] = []
+    layer_of_run: List[Optional[Tuple[int, int]]] = []
+    per_request: List[int] = []
+    for i, (need, cache_of) in enumerate(needs):
+        paged = need is not None and cache_kind(need).paged
+        if not paged:
+            if cache_of is not None:
+                raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no paged cache")
+            layer_of_run.append(None)
+            if need is not None:
+                per_request.append(i)
+            continue
+        if cache_of is not None:
+            src_need = needs[cache_of][0]
+            if src_need != need or layer_of_run[cache_of] is None:
+                raise ValueError(f"run {i} reads the cache of run {cache_of}, whose cache has other sizes: {src_need} vs {need}")
+            layer_of_run.append(layer_of_run[cache_of])
+            continue
+        if need not in group_needs:
+            group_needs.append(need)
+            layers_in_group.append(0)
+        g = group_needs.index(need)
+        layer_of_run.append((g, layers_in_group[g]))
+        layers_in_group[g] += 1
+    return group_needs, layers_in_group, layer_of_run, per_request
 
 
 class CacheManager:
@@ -57,62 +71,58 @@ class CacheManager:
         """`needs[i]` = (what run i's mixer asks for, index of the run whose cache it reads or None)."""
         self.dtype, self.device = dtype, device
         self.page_size, self.max_requests = page_size, max_requests
-        group_needs: List[PagedKV] = []
-        layer_of_run: List[Optional[Tuple[int, int]]] = []
-        layers_in_group: List[int] = []
-        for i, (need, cache_of) in enumerate(needs):
-            if not isinstance(need, PagedKV):
-                if cache_of is not None:
-                    raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no paged cache")
-                layer_of_run.append(None)
-                continue
-            if cache_of is not None:
-                src_need = needs[cache_of][0]
-                if src_need != need or layer_of_run[cache_of] is None:
-                    raise ValueError(f"run {i} reads the cache of run {cache_of}, whose cache has other sizes: {src_need} vs {need}")
-                layer_of_run.append(layer_of_run[cache_of])
-                continue
-            if need not in group_needs:
-                group_needs.append(need)
-                layers_in_group.append(0)
-            g = group_needs.index(need)
-            layer_of_run.append((g, layers_in_group[g]))
-            layers_in_group[g] += 1
+        group_needs, layers_in_group, layer_of_run, per_request = _group_runs(needs)
         pages = [int(num_pages)] * len(group_needs) if isinstance(num_pages, int) else [int(n) for n in num_pages]
         if len(pages) != len(group_needs):
             raise ValueError(f"num_pages names {len(pages)} groups, the model has {len(group_needs)}")
         self.groups: List[PagedGroup] = []
         for need, n_layers, n_pages in zip(group_needs, layers_in_group, pages):
-            shape_k = (n_layers, n_pages, need.kv_heads, page_size, need.head_dim)
-            shape_v = (n_layers, n_pages, need.kv_heads, need.head_dim, page_size)
-            self.groups.append(PagedGroup(need, page_size, n_pages, n_layers,
-                                          torch.zeros(shape_k, dtype=dtype, device=device),
-                                          torch.zeros(shape_v, dtype=dtype, device=device)))
+            kind = cache_kind(need)
+            self.groups.append(PagedGroup(need, kind, page_size, n_pages, n_layers,
+                                          kind.allocate_pages(need, n_layers, n_pages, page_size, dtype, device), dtype))
         self.views: List[CacheView] = []
-        self.state_tensors: List[torch.Tensor] = []
+        self._per_request: List[Tuple[CacheKind, Any, Any]] = []      # (kind, need, storage) of the runs with such needs
         for i, (need, cache_of) in enumerate(needs):
-            if isinstance(need, PagedKV):
+            if need is None:
+                self.views.append(CacheView("none"))
+            elif layer_of_run[i] is not None:
                 g, layer = layer_of_run[i]
                 grp = self.groups[g]
-                self.views.append(CacheView("paged", g, grp.k[layer], grp.v[layer], page_size, grp.num_pages,
-                                            writes=cache_of is None))
-            elif isinstance(need, FixedState):
-                state = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
-                self.state_tensors.append(state)
-                self.views.append(CacheView("state", state=state))
-            elif need is None:
-                self.views.append(CacheView("none"))
+                self.views.append(grp.kind.page_view(grp.storage, need, layer, g, page_size, grp.num_pages, cache_of is None))
             else:
-                raise TypeError(f"run {i}: a mixer's cache need must be PagedKV, FixedState or None, got {need!r}")
-        self.core = HostCore([(page_size, g.num_pages, g.need.window) for g in self.groups], max_requests,
+                kind = cache_kind(need)
+                storage = kind.allocate_slots(need, max_requests, device)
+                self._per_request.append((kind, need, storage))
+                self.views.append(kind.slot_view(storage, need))
+        self.core = HostCore([(page_size, g.num_pages, g.kind.window(g.need)) for g in self.groups], max_requests,
                              token_budget, max_chunk, max_positions)
+
+    @staticmethod
+    def pages_that_fit(needs: Sequence[Tuple[object, Optional[int]]], dtype: torch.dtype, page_size: int, free_bytes: int,
+                       fraction: float, max_requests: int, max_seq_len: int) -> List[int]:
+        """Pages for each group such that all of them take `fraction` of `free_bytes` less what the per-request
+        needs take, and no more than `max_requests` requests of `max_seq_len` tokens could ever fill
+        (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
+        group_needs, layers_in_group, _, per_request = _group_runs(needs)
+        if not group_needs:
+            return []
+        fixed = sum(cache_kind(needs[i][0]).bytes_per_request(needs[i][0]) for i in per_request) * max_requests
+        per_token = sum(n * cache_kind(need).bytes_per_token(need, dtype) for need, n in zip(group_needs, layers_in_group))
+        tokens = int(max(free_bytes - fixed, 0) * fraction) // max(per_token, 1)
+        tokens = min(tokens, max_requests * max_seq_len)
+        return [max(tokens // page_size, 1)] * len(group_needs)
 
     def bytes_per_token(self) -> int:
         return sum(g.bytes_per_token() for g in self.groups)
 
+    @property
+    def state_tensors(self) -> List[Any]:
+        """What the per-request needs were given, in the order of their runs."""
+        return [storage for _, _, storage in self._per_request]
+
     def reset_state(self, slots: Sequence[int]) -> None:
-        """Fixed-size state starts from zero when a request starts (or starts again) at position 0."""
-        if self.state_tensors and len(slots):
+        """Per-request memory starts afresh when a request starts (or starts again) at position 0."""
+        if self._per_request and len(slots):
             idx = torch.as_tensor(list(slots), dtype=torch.long, device=self.device)
-            for s in self.state_tensors:
-                s.index_fill_(0, idx, 0)
+            for kind, need, storage in self._per_request:
+                kind.reset_slots(storage, need, idx)

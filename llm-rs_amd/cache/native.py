@@ -45,7 +45,7 @@ def _lib():
             "llmrs_sched_build": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
             "llmrs_sched_commit": [c_void_p, c_void_p, c_int, c_void_p, c_int],
             "llmrs_sched_plan_sources": [c_void_p, c_void_p, c_int], "llmrs_sched_launch": [c_void_p],
-            "llmrs_sched_in_flight": [c_void_p],
+            "llmrs_sched_in_flight": [c_void_p], "llmrs_sched_set_max_chunk": [c_void_p, c_int],
             "llmrs_request_info": [c_void_p, c_int, c_void_p],
             "llmrs_request_output": [c_void_p, c_int, c_void_p, c_int],
             "llmrs_request_drop": [c_void_p, c_int],
@@ -198,6 +198,10 @@ class HostCore:
 
     def in_flight(self) -> bool:
         return bool(self._lib.llmrs_sched_in_flight(self._h))
+
+    def set_max_chunk(self, max_chunk: int) -> None:
+        """The most tokens of one request in a step from now on (0: the step's whole budget)."""
+        self._check(self._lib.llmrs_sched_set_max_chunk(self._h, int(max_chunk)))
 
     def build_planned(self, words: np.ndarray, fixed_widths=None):
         """Flatten the planned step; returns (offsets, n_tokens, n_sampling_rows)."""

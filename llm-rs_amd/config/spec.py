@@ -23,13 +23,10 @@ class PartSpec:
     params: Dict[str, Any] = field(default_factory=dict)
 
 
-PART_FAMILIES = ("mixer", "feed_forward", "norm")
-
-
 @dataclass(frozen=True)
 class ExtraPart:
     name: str                       # what the block arrangement calls it, e.g. "post_mixer_norm"
-    family: str                     # one of PART_FAMILIES: which registry builds it
+    family: str                     # which registry builds it: "mixer", "feed_forward", "norm", or a family registered with the parts
     spec: PartSpec
 
 
@@ -56,7 +53,7 @@ class ModelSpec:
     max_positions: int
     layers: List[LayerSpec]
     schedule: List[RunSpec]
-    final_norm: PartSpec
+    final_norm: Optional[PartSpec]  # the norm between the last block and the output matrix; None: the stream's rows as they are
     embedding_name: str             # tensor name of the token table
     head_name: Optional[str]        # tensor name of the output matrix; None = tied to the table
     # patterns (fnmatch) of tensor names this architecture's files may hold although the model reads none of them
@@ -71,8 +68,6 @@ class ModelSpec:
         for i, layer in enumerate(self.layers):
             names = [e.name for e in layer.extra]
             for e in layer.extra:
-                if e.family not in PART_FAMILIES:
-                    raise ValueError(f"layer {i}: part {e.name!r} is of family {e.family!r}, known: {', '.join(PART_FAMILIES)}")
                 if e.name in ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm") or names.count(e.name) > 1:
                     raise ValueError(f"layer {i}: two parts are called {e.name!r}")
         for i, run in enumerate(self.schedule):

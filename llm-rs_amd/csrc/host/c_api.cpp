@@ -186,6 +186,7 @@ int llmrs_sched_launch(void* h) {
 }
 
 int llmrs_sched_in_flight(void* h) { return ((Core*)h)->scheduler->in_flight() ? 1 : 0; }
+int llmrs_sched_set_max_chunk(void* h, int max_chunk) { auto c = (Core*)h; return guarded(c, [&] { c->scheduler->set_max_chunk(max_chunk); return 0; }); }
 
 // Writes the planned step's batch.  Returns the words used; n_tokens_out and
 // n_want_out get the step's tokens and the number of rows that sample.

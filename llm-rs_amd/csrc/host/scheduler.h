@@ -102,6 +102,8 @@ public:
     // One step can be in flight; commit() lands it.
     void launch();
     bool in_flight() const { return !flight_.empty(); }
+    // The most tokens of one request in a step from now on (0 or less: the step's whole budget).
+    void set_max_chunk(int max_chunk) { max_chunk_ = max_chunk > 0 ? max_chunk : budget_; }
 
     const Request& request(int slot) const { return requests_[slot]; }
     void drop(int slot);  // forget a finished request, free its slot

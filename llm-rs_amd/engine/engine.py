@@ -14,7 +14,7 @@ from typing import Dict, List, Mapping, Optional, Sequence, Union
 import numpy as np
 import torch
 
-from ..cache import CacheManager, CoreError
+from ..cache import CacheManager, CoreError, cache_kind
 from ..config import load_config
 from ..sampling import Sampler, SamplingParams
 from ..weights import RandomTensors, load_tensors, random_tensors
@@ -152,30 +152,14 @@ class Engine:
         return self.model.weights()
 
     def _pages_from_memory(self, needs, page_size, fraction, max_requests):
-        """Pages that fit `fraction` of the memory still free after the weights and after the
-        fixed-size state every request slot gets (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
-        from ..cache.spec import FixedState, PagedKV
-        groups: Dict[PagedKV, int] = {}
-        state_bytes = 0
-        for need, cache_of in needs:
-            if isinstance(need, PagedKV) and cache_of is None:
-                groups[need] = groups.get(need, 0) + 1
-            elif isinstance(need, FixedState):
-                n = need.dtype.itemsize
-                for s in need.shape:
-                    n *= int(s)
-                state_bytes += n * max_requests
-        if not groups:
-            return []
+        """Pages that fit `fraction` of the memory still free after the weights and after what every request
+        slot gets of fixed size; what a token and a slot cost is the cache kinds' to say."""
         if self.device.type != "cuda":
-            raise ValueError("num_pages must be given when the engine is not on a GPU")
+            if any(need is not None and cache_kind(need).paged for need, _ in needs):
+                raise ValueError("num_pages must be given when the engine is not on a GPU")
+            return []
         free, _ = torch.cuda.mem_get_info(self.device)
-        free = max(free - state_bytes, 0)
-        per_token = sum(2 * n * need.kv_heads * need.head_dim * self.dtype.itemsize for need, n in groups.items())
-        tokens = int(free * fraction) // per_token
-        tokens = min(tokens, max_requests * self.max_seq_len)
-        pages = max(tokens // page_size, 1)
-        return [pages] * len(groups)
+        return CacheManager.pages_that_fit(needs, self.dtype, page_size, free, fraction, max_requests, self.max_seq_len)
 
     # -- manual stepping (trace replay, tests) -----------------------------------
     def open_request(self) -> int:

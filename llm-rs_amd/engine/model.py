@@ -21,7 +21,7 @@ class Model:
             raise ValueError(f"the engine computes in float32 or bfloat16, not {dtype}")
         self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
         self.blocks = [build_block(layer, dtype) for layer in spec.layers]
-        self.final_norm = build_norm(spec.final_norm, dtype)
+        self.final_norm = build_norm(spec.final_norm, dtype) if spec.final_norm is not None else None
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
         keyed = {}
@@ -40,7 +40,8 @@ class Model:
         for block in self.blocks:
             for part in block.parts():
                 out.update(part.tensors())
-        out.update(self.final_norm.tensors())
+        if self.final_norm is not None:
+            out.update(self.final_norm.tensors())
         return out
 
     def load(self, tensors: Mapping[str, torch.Tensor]) -> None:
@@ -57,7 +58,8 @@ class Model:
         for block in self.blocks:
             for part in block.parts():
                 part.load(tensors, self.device)
-        self.final_norm.load(tensors, self.device)
+        if self.final_norm is not None:
+            self.final_norm.load(tensors, self.device)
 
     def weights(self) -> Dict[str, torch.Tensor]:
         """Every tensor of the model on the host, under its file name and in the file's layout
@@ -70,31 +72,25 @@ class Model:
         for block in self.blocks:
             for part in block.parts():
                 out.update(part.export())
-        out.update(self.final_norm.export())
+        if self.final_norm is not None:
+            out.update(self.final_norm.export())
         return out
 
     def weight_bytes_per_step(self) -> int:
         """Bytes of weights one step reads when it uses each once (the table's rows aside):
         every tensor a part of the schedule's layers holds, the final norm's, and the output matrix."""
         seen = set()
-
-        def held(part) -> int:
-            total = 0
-            for v in vars(part).values():
-                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
-                    seen.add(v.data_ptr())
-                    total += v.numel() * v.element_size()
-            return total
-
-        total = sum(held(part) for run in self.spec.schedule for part in self.blocks[run.layer].parts())
-        total += held(self.final_norm)
+        total = sum(part.step_weight_bytes(seen) for run in self.spec.schedule for part in self.blocks[run.layer].parts())
+        if self.final_norm is not None:
+            total += self.final_norm.step_weight_bytes(seen)
         if self.head.data_ptr() not in seen:
             total += self.head.numel() * self.head.element_size()
         return total
 
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph (every part says so)."""
-        return all(part.graph_safe for block in self.blocks for part in block.parts()) and self.final_norm.graph_safe
+        return (all(part.graph_safe for block in self.blocks for part in block.parts())
+                and (self.final_norm is None or self.final_norm.graph_safe))
 
     def recording_key(self, ctx) -> tuple:
         """What a recording of this step depends on beyond its sizes (its parts say)."""
@@ -120,7 +116,7 @@ class Model:
             # final norm, where it reads every row (else it reads gathered rows and runs as a kernel of its own)
             later = self.spec.schedule[i + 1] if i + 1 < len(self.spec.schedule) else None
             ctx.norm_after_block = (self.blocks[later.layer].first_norm() if later is not None
-                                    else self.final_norm if ctx.wants_every_row else None)
+                                    else self.final_norm if ctx.wants_every_row else None)      # (None too without a final norm)
             block.forward(ctx, h, cache_views[i])
             if not block.keeps_left_current:
                 ctx.note_left(h, None)
@@ -131,10 +127,16 @@ class Model:
         # rows and gathers after (src/arch/llama.rs:135-139), which is the same numbers.
         # (A step of few single tokens that wants them all: the last product has prepared the final norm, and the
         # output matrix's product finishes it; no norm kernel runs.)
-        x = self.final_norm.deferred(ctx, h) if ctx.wants_every_row else None
+        x = self.final_norm.deferred(ctx, h) if ctx.wants_every_row and self.final_norm is not None else None
         if x is None:
             x = ctx.workspace("model.head_in", (ctx.n_want, self.spec.hidden_size), self.dtype)
-            self.final_norm.forward(ctx, h, x, ctx.want_rows)
+            if self.final_norm is not None:
+                self.final_norm.forward(ctx, h, x, ctx.want_rows)
+            else:       # no norm before the output matrix: the wanted rows of the stream, in the activation type
+                rows = x if self.dtype == torch.float32 else ctx.workspace("model.head_rows", x.shape, torch.float32)
+                k.embed_rows(rows, h, ctx.want_rows, 1.0)
+                if rows is not x:
+                    k.cast(x, rows)
         logits = ctx.workspace("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
         k.gemm(x, self.head, logits, EPI_STORE_F32, ctx.gemm_workspace(x, self.head))
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:

@@ -99,21 +99,18 @@ class StepContext:
         product to fill (`kernels().gemm(..., leave=...)`; then `note_left(h, it)`), or None when the norm that
         follows cannot be left to the next product (no such norm, other dtype, too many rows)."""
         from ..kernels import NextNorm, kernels
-        k = kernels()
         norm = self.upcoming_norm
         weight = norm.deferred_weight() if norm is not None else None
-        defers = getattr(k, "gemm_defers_norm", None)
         T, N = h.shape[0], w.shape[0]
-        if weight is None or defers is None or w.dtype != torch.bfloat16 or N != h.shape[1] or weight.shape[0] != N:
+        if weight is None or N != h.shape[1] or weight.shape[0] != N:
             return None
-        if N < 16384 and defers(T, N, w.shape[1]):
-            parts = k.gemm_next_parts(T, N, w.shape[1]) if hasattr(k, "gemm_next_parts") else -(-N // 16)
-            return NextNorm(self._prenormed(T, N), self.workspace("model.sumsq", (T, parts), torch.float32), weight)
-        # more rows: a product that is split over blocks finishes the norm where its parts are added up
-        whole, eps = getattr(k, "gemm_norms_whole", None), norm.deferred_eps()
-        if whole is not None and eps is not None and eps > 0 and whole(T, N, w.shape[1]):
-            return NextNorm(self._prenormed(T, N), None, weight, eps)
-        return None
+        plan = kernels().norm_left_by_product(T, N, w.shape[1], w.dtype)
+        if plan is None:
+            return None
+        if not plan.whole:
+            return NextNorm(self._prenormed(T, N), self.workspace("model.sumsq", (T, plan.parts), torch.float32), weight)
+        eps = norm.deferred_eps()
+        return NextNorm(self._prenormed(T, N), None, weight, eps) if eps is not None and eps > 0 else None
 
     def _prenormed(self, T: int, N: int) -> torch.Tensor:
         """Room for the rows a product leaves: not the rows that were left last, which the part at work may

@@ -15,7 +15,7 @@ import ctypes
 import os
 import sys
 from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
-from typing import Dict, List, Optional
+from typing import Dict, List, NamedTuple, Optional
 
 import torch
 
@@ -122,7 +122,47 @@ def _p(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
 
-class HipKernels:
+class NormPlan(NamedTuple):
+    """How a product that adds into the stream serves the norm that follows it (`Kernels.norm_left_by_product`)."""
+    whole: bool          # True: the product finishes the norm itself (a `NextNorm` with eps, and the product's workspace)
+    parts: int           # else: partial sums of squares it leaves per row, the second dimension of `NextNorm.sumsq`
+
+
+class Kernels:
+    """What the engine asks of its device operations beyond the operations themselves: how much room a call needs and
+    which of the optional hand-overs between kernels a call can take.  An implementation answers for itself; the
+    answers here are those of one that splits nothing and hands nothing over, so that parts never have to probe the
+    object they were given."""
+
+    allow_mfma = False
+    times: Optional[KernelTimes] = None
+
+    def gemm_workspace_floats(self, M: int, N: int, K: int) -> int:
+        """Room (floats) that lets the product of M rows with an [N, K] weight split K over blocks; 0: none needed."""
+        return 0
+
+    def product_norms_its_rows(self, M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+        """Whether the product of M rows with an [N, K] weight takes `NormedRows` (rows still to be scaled by
+        their norm) in place of normed rows."""
+        return False
+
+    def norm_left_by_product(self, M: int, N: int, K: int, dtype: torch.dtype) -> Optional[NormPlan]:
+        """What the product of M rows with an [N, K] weight, adding into the stream, can leave for the norm that
+        reads the stream next (`NextNorm`), or None: then a norm kernel runs."""
+        return None
+
+    def attention_scratch_floats(self, n_entries: int, n_heads: int, head_dim: int, max_seq_len: int,
+                                 n_kv_heads: Optional[int] = None, n_single: int = 0) -> int:
+        """Room (floats) for the partial results of single-token entries whose keys are shared out over waves."""
+        return 0
+
+    def attention_split_chunk(self, n_single: int, n_kv_heads: int, head_dim: int, max_seq_len: int, single_keys: int = 0) -> int:
+        """Keys per wave that a call with these figures splits its single-token entries by (0: it does not split):
+        what a caller that records steps has to key its recordings by."""
+        return 0
+
+
+class HipKernels(Kernels):
     """Launches on the current torch stream of the tensors' device."""
 
     def __init__(self):
@@ -174,6 +214,20 @@ class HipKernels:
     def gemm_workspace_floats(self, M: int, N: int, K: int) -> int:
         """Room that lets a product with too few blocks split K over blocks (the kernels' own rule)."""
         return int(self.lib.llmrs_gemm_workspace_floats(int(M), int(N), int(K)))
+
+    def product_norms_its_rows(self, M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+        return dtype == torch.bfloat16 and self.gemm_defers_norm(M, N, K)
+
+    def norm_left_by_product(self, M: int, N: int, K: int, dtype: torch.dtype) -> Optional[NormPlan]:
+        if dtype != torch.bfloat16:
+            return None
+        # up to a few rows: partial sums of squares, for the next product to finish (the kernels keep at most 1024
+        # of them a row); more rows: a product that is split over blocks finishes the norm where its parts are added up
+        if N < 16384 and self.gemm_defers_norm(M, N, K):
+            return NormPlan(False, self.gemm_next_parts(M, N, K))
+        if self.gemm_norms_whole(M, N, K):
+            return NormPlan(True, 0)
+        return None
 
     def gemm_defers_norm(self, M: int, N: int, K: int) -> bool:
         """Whether the bfloat16 product of M rows with an [N, K] weight takes `NormedRows` as its rows and, adding

@@ -99,9 +99,7 @@ class Attention(Mixer):
     def takes_normed_rows(self, ctx, rows):
         # the q/k/v product norms its rows itself where it is the fused kernel: a rotation it applies (or none)
         fused = self.position is None or self.position.rotary() is not None
-        k = kernels()
-        return (fused and self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
-                and k.gemm_defers_norm(rows, self.w_qkv.shape[0], self.hidden))
+        return fused and kernels().product_norms_its_rows(rows, self.w_qkv.shape[0], self.hidden, self.dtype)
 
     # The kernel library shares the decoding requests' keys out over waves in chunks whose length it chooses by
     # how many keys the step sees (`single_keys`).  A recorded step holds the chunk it was recorded with, so the
@@ -112,7 +110,7 @@ class Attention(Mixer):
 
     def recording_key(self, ctx):
         k = kernels()
-        if not ctx.n_single or not hasattr(k, "attention_split_chunk"):
+        if not ctx.n_single:
             return 0
         keys = ctx.single_keys(self.window)
         want = k.attention_split_chunk(ctx.n_single, self.kv_heads, self.head_dim, ctx.max_seq_len, keys)

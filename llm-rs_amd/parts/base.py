@@ -70,6 +70,17 @@ class Part:
     def load(self, tensors: Mapping[str, torch.Tensor], device) -> None:
         pass
 
+    def step_weight_bytes(self, seen: set) -> int:
+        """Bytes of this part's tensors that a step has to read when it uses each once: every tensor the part
+        holds (`seen`: addresses already counted, for tensors that parts share).  A part that reads only some of
+        what it holds in a step (the experts a router chose) answers with what a step reads."""
+        total = 0
+        for v in vars(self).values():
+            if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                seen.add(v.data_ptr())
+                total += v.numel() * v.element_size()
+        return total
+
     def takes_normed_rows(self, ctx, rows: int) -> bool:
         """Whether `forward` may be given `kernels.NormedRows` (rows still to be normed, which the part's
         first product norms itself) in place of the normed input `x`, for a step of `rows` tokens."""
@@ -240,7 +251,23 @@ def build_position(params: Optional[Mapping], dtype) -> Optional[PositionEncodin
     return _build(POSITIONS, "position encoding", params["kind"], params, dtype)
 
 
-_BUILDERS = {"mixer": build_mixer, "feed_forward": build_feed_forward, "norm": build_norm}
+# Families of parts that a layer's `extra` list may name: family -> the table of its kinds.  The three below are
+# what the four usual places of a layer are built from; an arrangement that needs parts of another nature (a router
+# shared by two feed-forwards, a gate) registers a family for them.
+FAMILIES: Dict[str, Dict[str, Callable]] = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+
+
+def register_part_family(family: str) -> Callable:
+    """Makes `family` a family of parts that `LayerSpec.extra` may name; returns the function that registers its
+    kinds, `register(kind, factory)` with `factory(spec, dtype)` as for the other families."""
+    table = FAMILIES.setdefault(family, {})
+    return _register(table, family)
+
+
+def build_part(family: str, spec: PartSpec, dtype) -> Part:
+    if family not in FAMILIES:
+        raise KeyError(f"unknown family of parts {family!r} (registered: {', '.join(sorted(FAMILIES))})")
+    return _build(FAMILIES[family], family, spec.kind, spec, dtype)
 
 
 def build_block(layer_spec, dtype) -> Block:
@@ -249,5 +276,5 @@ def build_block(layer_spec, dtype) -> Block:
              "feed_forward_norm": opt(build_norm, layer_spec.feed_forward_norm),
              "feed_forward": opt(build_feed_forward, layer_spec.feed_forward)}
     for extra in layer_spec.extra:
-        named[extra.name] = _BUILDERS[extra.family](extra.spec, dtype)
+        named[extra.name] = build_part(extra.family, extra.spec, dtype)
     return _build(BLOCKS, "block arrangement", layer_spec.block, named)

@@ -39,9 +39,7 @@ class SwiGLU(FeedForward):
                 self.name("down_proj.weight"): self.w_down.cpu()}
 
     def takes_normed_rows(self, ctx, rows):
-        k = kernels()
-        return (self.dtype == torch.bfloat16 and hasattr(k, "gemm_defers_norm")
-                and k.gemm_defers_norm(rows, 2 * self.inter, self.hidden))
+        return kernels().product_norms_its_rows(rows, 2 * self.inter, self.hidden, self.dtype)
 
     def forward(self, ctx, x, h):
         k = kernels()

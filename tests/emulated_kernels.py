@@ -9,14 +9,13 @@ import math
 
 import torch
 
+from llm_rs_amd.kernels import Kernels, NormPlan
+
 EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU = 0, 1, 2, 3
 
 
-class EmulatedKernels:
-    allow_mfma = False
-
-    def attention_scratch_floats(self, n_entries, n_heads, head_dim, max_seq_len, n_kv_heads=None, n_single=0):
-        return 0
+class EmulatedKernels(Kernels):
+    """(What `Kernels` answers by itself stays: no workspace, no scratch, nothing split.)"""
 
     def embed_rows(self, out, table, tokens, scale=1.0):
         out.copy_(table[tokens.long()].float() * scale)
@@ -35,13 +34,12 @@ class EmulatedKernels:
         inv = 1.0 / torch.sqrt(ss / src.shape[-1] + eps)
         out.copy_((src * inv * weight).to(out.dtype))
 
-    @staticmethod
-    def gemm_workspace_floats(M, N, K):
-        return 0
+    # as the device: steps of up to 16 tokens in bfloat16 leave their norms to the products around them
+    def product_norms_its_rows(self, M, N, K, dtype):
+        return dtype == torch.bfloat16 and 1 <= M <= 16
 
-    @staticmethod
-    def gemm_defers_norm(M, N, K):
-        return 1 <= M <= 16            # as the device: steps of up to 16 tokens leave their norms to the products
+    def norm_left_by_product(self, M, N, K, dtype):
+        return NormPlan(False, -(-N // 16)) if dtype == torch.bfloat16 and 1 <= M <= 16 else None
 
     def gemm(self, a, w, out, epilogue=EPI_STORE, workspace=None, leave=None):
         inv = None

@@ -41,7 +41,7 @@ def read_model_folder(folder: str):
 
 def plain_embedding(table: torch.Tensor, tokens: Sequence[int]) -> torch.Tensor:
     """x[t, :] = table[tok[t], :], no scaling (src/arch/llama.rs:150, shaders/ops.metal:878-902)."""
-    return table[torch.tensor(list(tokens), dtype=torch.long)]
+    return table[torch.tensor(list(tokens), dtype=torch.long, device=table.device)]
 
 
 def plain_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
@@ -76,7 +76,7 @@ def plain_rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
     is (i, i + d/2) for "split_half", (2i, 2i+1) for "interleaved"
     (src/tensor/mod.rs:133-139).  Features past the rotary width are unchanged."""
     rot = 2 * inv_freq.shape[0]
-    angle = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).to(x.dtype)   # [T, rot/2]
+    angle = (positions.to(torch.float32)[:, None] * inv_freq[None, :]).to(device=x.device, dtype=x.dtype)   # [T, rot/2]
     cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
     out = x.clone()
     if layout == "split_half":
@@ -93,16 +93,17 @@ def plain_rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
 
 
 def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
-                    window: int = 0, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    window: int = 0, positions: Optional[torch.Tensor] = None, rounded=lambda t: t) -> torch.Tensor:
     """q: [T, heads, d]; k, v: [T, kv_heads, d]; one sequence, causal.
     Head h uses kv head h / (heads / kv_heads); s_j = (q . k_j) * rsqrt(d), the scale
     after the dot; keys j <= the query's place (and > place - window if a window is
-    given); softmax over j; o = sum_j p_j v_j (shaders/ops.metal:658-757)."""
+    given); softmax over j; o = sum_j p_j v_j (shaders/ops.metal:658-757).
+    (`rounded`: see `plain_forward_streamed`; applied to the probabilities.)"""
     T, H, d = q.shape
     KV = k.shape[1]
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     out = torch.zeros_like(q)
-    place = torch.arange(T) if positions is None else positions
+    place = (torch.arange(T) if positions is None else positions).to(q.device)
     for h in range(H):
         g = h // (H // KV)
         scores = (q[:, h, :] @ k[:, g, :].T) * scale                      # [T, T]
@@ -110,7 +111,7 @@ def plain_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Op
         if window > 0:
             visible &= place[None, :] > place[:, None] - window
         scores = scores.masked_fill(~visible, float("-inf"))
-        out[:, h, :] = torch.softmax(scores, dim=-1) @ v[:, g, :]
+        out[:, h, :] = rounded(torch.softmax(scores, dim=-1)) @ v[:, g, :]
     return out
 
 
@@ -119,32 +120,34 @@ def plain_silu(x: torch.Tensor) -> torch.Tensor:
     return x / (1.0 + torch.exp(-x))
 
 
-def plain_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
-    """(silu(x Wg^T) * (x Wu^T)) Wd^T (src/arch/llama.rs:165-169)."""
-    return (plain_silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+def plain_swiglu(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, rounded=lambda t: t) -> torch.Tensor:
+    """(silu(x Wg^T) * (x Wu^T)) Wd^T (src/arch/llama.rs:165-169).  (`rounded`: see `plain_forward_streamed`.)"""
+    return rounded(plain_silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
 
 
 # ---- the model -----------------------------------------------------------------
 
 def plain_layer(cfg: dict, W: Dict[str, torch.Tensor], prefix: str, x: torch.Tensor, pos: torch.Tensor,
-                inv_freq: torch.Tensor, layout: str = "split_half") -> torch.Tensor:
+                inv_freq: torch.Tensor, layout: str = "split_half", rounded=lambda t: t) -> torch.Tensor:
     """One layer on one whole sequence x [T, hidden]: x += attention(norm(x)); x += swiglu(norm(x))
-    (src/arch/llama.rs:151-170).  `W` holds the layer's tensors under `prefix` + their names."""
+    (src/arch/llama.rs:151-170).  `W` holds the layer's tensors under `prefix` + their names.
+    (`rounded`: see `plain_forward_streamed`.)"""
     H, D = cfg["num_attention_heads"], cfg["hidden_size"]
     KV = cfg.get("num_key_value_heads") or H
     d = cfg.get("head_dim") or D // H
     eps = cfg.get("rms_norm_eps", 1e-5)
     T = x.shape[0]
     p = prefix
-    xn = plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps)
+    r = rounded
+    xn = r(plain_rmsnorm(x, W[p + "input_layernorm.weight"], eps))
     q = (xn @ W[p + "self_attn.q_proj.weight"].T).view(T, H, d)
     k = (xn @ W[p + "self_attn.k_proj.weight"].T).view(T, KV, d)
-    v = (xn @ W[p + "self_attn.v_proj.weight"].T).view(T, KV, d)
-    q, k = plain_rope(q, pos, inv_freq, layout), plain_rope(k, pos, inv_freq, layout)
-    o = plain_attention(q, k, v).reshape(T, H * d)
+    v = r((xn @ W[p + "self_attn.v_proj.weight"].T).view(T, KV, d))
+    q, k = r(plain_rope(q, pos, inv_freq, layout)), r(plain_rope(k, pos, inv_freq, layout))
+    o = r(plain_attention(q, k, v, rounded=r).reshape(T, H * d))
     x = x + o @ W[p + "self_attn.o_proj.weight"].T
-    xn = plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps)
-    return x + plain_swiglu(xn, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+    xn = r(plain_rmsnorm(x, W[p + "post_attention_layernorm.weight"], eps))
+    return x + plain_swiglu(xn, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"], r)
 
 
 def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[int],
@@ -157,28 +160,56 @@ def plain_forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: Sequence[
 
 
 def plain_forward_streamed(cfg: dict, tensor_of, sequences: Sequence[Sequence[int]], compute: torch.dtype = torch.float64,
-                           layout: str = "split_half", position_offset: int = 0) -> List[torch.Tensor]:
+                           layout: str = "split_half", position_offset: int = 0, rows: Optional[Sequence[Sequence[int]]] = None,
+                           rounding: Optional[torch.dtype] = None, device="cpu", also_in: Optional[torch.dtype] = None):
     """The same for several whole sequences, one after the other through each layer, with the
     tensors asked for by name through `tensor_of(name)` when their layer is reached and dropped
-    after it: a model too large to hold in `compute` precision needs one layer's worth of room."""
+    after it: a model too large to hold in `compute` precision needs one layer's worth of room.
+    `rows[i]`: the places of sequence i whose logits are wanted (default: all).  `device`: where the
+    tensor operations run (the same plain operations; a long sequence through a deep model takes
+    minutes on the host).
+    `rounding`: a second pass beside the first in which every activation that a kernel of an engine
+    computing in that type hands to the next kernel through memory is rounded to it (the normed rows,
+    q, k and v, the probabilities, the attention's output, silu(gate) * up, the output matrix's input;
+    never the residual stream, never a sum).  It says how far rounding alone takes this model on these
+    sequences from the exact result; the return value is then (logits, logits of the rounded pass)."""
     H, D = cfg["num_attention_heads"], cfg["hidden_size"]
     d = cfg.get("head_dim") or D // H
     inv_freq = plain_inv_freq(d, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
-    table = tensor_of("model.embed_tokens.weight")
+    get = lambda name: tensor_of(name).to(device)
+    rounded = (lambda t: t.to(rounding).to(t.dtype)) if rounding is not None else None
+    table = get("model.embed_tokens.weight")
     xs = [plain_embedding(table, tokens).to(compute) for tokens in sequences]
+    ys = [x.clone() for x in xs] if rounded else None
+    zs = [x.to(also_in) for x in xs] if also_in is not None else None
     positions = [torch.arange(len(tokens)) + position_offset for tokens in sequences]
     leaves = ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight",
               "self_attn.o_proj.weight", "post_attention_layernorm.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight",
               "mlp.down_proj.weight")
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        W = {p + leaf: tensor_of(p + leaf).to(compute) for leaf in leaves}
+        W = {p + leaf: get(p + leaf).to(compute) for leaf in leaves}
         xs = [plain_layer(cfg, W, p, x, pos, inv_freq, layout) for x, pos in zip(xs, positions)]
+        if rounded:
+            ys = [plain_layer(cfg, W, p, y, pos, inv_freq, layout, rounded) for y, pos in zip(ys, positions)]
+        if zs is not None:
+            W = {n: t.to(also_in) for n, t in W.items()}
+            zs = [plain_layer(cfg, W, p, z, pos, inv_freq, layout) for z, pos in zip(zs, positions)]
         del W
-    norm = tensor_of("model.norm.weight").to(compute)
-    head = (table if cfg.get("tie_word_embeddings", False) else tensor_of("lm_head.weight")).to(compute)
+    norm = get("model.norm.weight").to(compute)
+    head = (table if cfg.get("tie_word_embeddings", False) else get("lm_head.weight")).to(compute)
     eps = cfg.get("rms_norm_eps", 1e-5)
-    return [plain_rmsnorm(x, norm, eps) @ head.T for x in xs]
+    pick = lambda x, i: x if rows is None else x[torch.tensor(list(rows[i]), dtype=torch.long, device=x.device)]
+    exact = [plain_rmsnorm(pick(x, i), norm, eps) @ head.T for i, x in enumerate(xs)]
+    if not rounded and zs is None:
+        return exact
+    out = [exact]
+    if rounded:
+        out.append([rounded(plain_rmsnorm(pick(y, i), norm, eps)) @ head.T for i, y in enumerate(ys)])
+    if zs is not None:
+        norm, head = norm.to(also_in), head.to(also_in)
+        out.append([plain_rmsnorm(pick(z, i), norm, eps) @ head.T for i, z in enumerate(zs)])
+    return tuple(out)
 
 
 # ---- sampling ------------------------------------------------------------------

@@ -90,11 +90,13 @@ def test_the_default_workload_runs_and_fills_its_line():
     both points and the host's share."""
     bench = load_bench()
     args = SimpleNamespace(gpus=1, steps=6, warmup=4, workload="decode8b", batch=8, context=300, prefill_tokens=256, layers=1,
-                           dtype="bfloat16", points="1,20", only="", requests=0, new_tokens=0, max_batch_tokens=2048)
+                           dtype="bfloat16", points="1,20,3@700", only="", requests=0, new_tokens=0, max_batch_tokens=2048)
     line = check_line(bench.run_decode8b(args))
     assert line["value"] > 0 and abs(line["value"] - 8 / (line["ms_per_step"] * 1e-3)) <= 1e-3 * line["value"]
     assert line["config"]["layers_run"] == 1 and line["config"]["layers_of_config"] == 32 and line["config"]["global_batch"] == 8
-    assert set(line["points"]) == {"decode_b1", "decode_b20"} and all(v > 0 for v in line["points"].values())
+    assert set(line["points"]) == {"decode_b1", "decode_b20", "decode_b3_ctx700"} and all(v > 0 for v in line["points"].values())
+    assert set(line["points_frac"]) == set(line["points"]) and all(0 < v < 1 for v in line["points_frac"].values())
+    assert line["metric"].endswith("prefill tok/s at 256 tokens and batch 1/20 alongside")
     assert line["prefill"]["tokens"] == 256 and 0 < line["prefill"]["frac"] < 1
     assert line["roofline"]["bound"] == "hbm" and 0 < line["roofline"]["frac"] < 1
     assert 0 <= line["host"]["overhead_frac"] < 0.5 and line["host"]["device_ms_per_step"] > 0

@@ -167,6 +167,7 @@ def test_bench_subcommand_and_the_table_by_kernel(tmp_path):
             assert "TOTAL" in timed.stderr
             assert all(calls > 0 and t > 0 for calls, t, _, _ in rows.values())
             gemms = {n: r for n, r in rows.items() if n.startswith("gemm")}
-            assert all(r[2] > 0 and r[3] != "-" for r in gemms.values()), "a product has bytes and operations"
+            # (a kernel's first call waits for its code to reach the device, so a label that ran once may show 0 GB/s)
+            assert all(r[3] != "-" for r in gemms.values()) and any(r[2] > 0 for r in gemms.values()), "a product has bytes and operations"
             # 13 steps (one prompt step, 12 decode steps less the last) of 3 layers: each layer's products are counted
             assert sum(r[0] for r in gemms.values()) >= 12 * (3 * 4 + 1)

@@ -303,8 +303,10 @@ def test_attention_as_many_tokens_as_entries_but_not_one_each(dtype, n_heads, n_
                 err = (got[at:at + len(p)].double() - ref).abs()
                 assert (err <= out_tol(ref, dtype, floor)).all(), f"n_single {n_single}, entry {r}: max err {float(err.max())}"
                 at += len(p)
+    q_pos = [[38, 39], [5], [7, 8], [3]]                                  # four entries, six tokens
+    qs = [torch.randn((len(p), n_heads, hd), generator=g).to(dtype) for p in q_pos]
     with pytest.raises(KernelError, match="every entry is said to bring one token"):
-        case.run([qs[0], qs[2]], [q_pos[0], q_pos[2]] , n_single=2)      # two entries, four tokens
+        case.run(qs, q_pos, n_single=4)
 
 
 ATTN_SHAPES = [(4, 2, 16, 4), (3, 1, 32, 16), (8, 8, 64, 16), (8, 2, 128, 16), (6, 3, 48, 8), (5, 1, 80, 16),
@@ -353,6 +355,31 @@ def test_attention_finds_a_far_key(dtype, hd, ps, n):
         assert (ref[0].float() - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
         tol = 1e-4 if dtype == torch.float32 else 2e-2
         assert (got[0].float() - ref[0].float()).abs().max() <= tol, f"far key {far}"
+
+
+def test_attention_at_131008_keys():
+    """One request decoding over 131,008 keys at head size 128 in bfloat16 (134 MB of cache, 8,188 pages scattered
+    over the pool, a block table that wide, the most chunks the merge takes): a key that matches the query strongly is
+    found wherever it lies (the first and last keys, the edges of pages, of every chunk length and of 65,536), and random
+    queries agree with the plain formula."""
+    n, n_heads, n_kv, hd, ps = 131008, 8, 2, 128, 16
+    case = PagedCase(torch.bfloat16, [n], n_heads, n_kv, hd, ps, seed=23)
+    assert case.width == 8188
+    fars = (0, 15, 16, 511, 512, 1023, 1024, 32767, 65535, 65536, 65537, 100003, n - 1025, n - 1024, n - 513, n - 17, n - 2, n - 1)
+    for far in fars:
+        q = (case.k[0][far].float().repeat_interleave(n_heads // n_kv, dim=0) * 8.0).unsqueeze(0).to(torch.bfloat16)
+        got = case.run([q], [[n - 1]], n_single=1, single_keys=n)
+        want = case.v[0][far].float().repeat_interleave(n_heads // n_kv, dim=0)
+        ref = case.reference(0, q, [n - 1])[0].float()
+        assert (ref - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
+        assert (got[0].float() - ref).abs().max() <= 2e-2, f"far key {far}"
+    g = torch.Generator().manual_seed(9)
+    for i in range(3):
+        # queries of growing length: from nearly uniform weights over all keys to a handful of keys that count
+        q = (torch.randn((1, n_heads, hd), generator=g) * (0.5, 1.5, 3.0)[i]).to(torch.bfloat16)
+        got = case.run([q], [[n - 1]], n_single=1, single_keys=n)
+        ref = case.reference(0, q, [n - 1])[0].float()
+        assert (got[0].float() - ref).abs().max() <= 4e-3 + 2e-2 * float(ref.abs().max()), f"random query {i}"
 
 
 def test_attention_chunk_rule_and_its_scratch():

@@ -636,3 +636,199 @@ def test_toy_architecture_with_other_block_arrangements_scaled_embedding_and_ben
         got = torch.cat(rows)
         assert float((got - ref).abs().max()) <= tol * max(float(ref.abs().max()), 1.0), cuts
         eng.close_request(slot)
+
+
+# ---- a mixer with a cache kind of its own, a family of parts of its own, and no final norm -------------------------
+
+from dataclasses import dataclass  # noqa: E402
+
+from llm_rs_amd.cache import CacheKind, CacheView, register_cache_kind  # noqa: E402
+from llm_rs_amd.parts import Part, register_part_family  # noqa: E402
+
+
+@dataclass(frozen=True)
+class PagedLatent:
+    """One vector of `width` numbers per token, in pages."""
+    width: int
+    window: int = 0
+
+
+class PagedLatentKind(CacheKind):
+    """[layer][page][slot][width] in 32-bit, whatever the engine computes in."""
+    paged = True
+
+    def window(self, need):
+        return need.window
+
+    def bytes_per_token(self, need, dtype):
+        return 4 * need.width
+
+    def allocate_pages(self, need, n_layers, num_pages, page_size, dtype, device):
+        return torch.zeros((n_layers, num_pages, page_size, need.width), dtype=torch.float32, device=device)
+
+    def page_view(self, storage, need, layer, group, page_size, num_pages, writes):
+        return CacheView("latent", group, page_size=page_size, num_pages=num_pages, writes=writes, data=storage[layer])
+
+
+class LatentMixer(Mixer):
+    """c_t = x_t Wc^T is what a token leaves in the cache; y_t = (sum_j<=t softmax_j((x_t Wq^T) . c_j / sqrt(L)) c_j) Wo^T:
+    attention whose keys and values are the same latent vector."""
+
+    def __init__(self, spec, dtype):
+        super().__init__(spec, dtype)
+        self.hidden, self.width = spec.params["hidden_size"], spec.params["latent"]
+
+    def tensors(self):
+        return {self.name("c"): TensorSpec((self.width, self.hidden)), self.name("q"): TensorSpec((self.width, self.hidden)),
+                self.name("o"): TensorSpec((self.hidden, self.width))}
+
+    def load(self, tensors, device):
+        self.wc, self.wq, self.wo = (tensors[self.name(n)].to(device=device, dtype=torch.float32) for n in "cqo")
+
+    def export(self):
+        return {self.name(n): w.cpu() for n, w in zip("cqo", (self.wc, self.wq, self.wo))}
+
+    def cache_need(self):
+        return PagedLatent(self.width)
+
+    def forward(self, ctx, x, h, cache):
+        assert cache.kind == "latent" and cache.data.shape[1:] == (cache.page_size, self.width)
+        g, L = cache.group, self.width
+        xf = x.float()
+        cache.data.view(-1, L)[ctx.slot_maps[g].long()] = xf @ self.wc.T       # this step's latents into their pages
+        at = 0
+        for e, (slot, start, count) in enumerate(ctx.entries):
+            n = start + count
+            pages = ctx.block_tables[g][e, :-(-n // cache.page_size)].long()
+            lat = cache.data[pages].reshape(-1, L)[:n]                          # the request's latents, in order
+            s = (xf[at:at + count] @ self.wq.T) @ lat.T / math.sqrt(L)
+            seen = torch.arange(n, device=s.device)[None, :] <= (start + torch.arange(count, device=s.device))[:, None]
+            p = torch.softmax(s.masked_fill(~seen, -math.inf), dim=-1)
+            h[at:at + count] += (p @ lat) @ self.wo.T
+            at += count
+
+
+class VectorGate(Part):
+    """A part that is neither mixer, feed-forward nor norm: one number per feature."""
+
+    def tensors(self):
+        return {self.name("g"): TensorSpec((self.spec.params["size"],))}
+
+    def load(self, tensors, device):
+        self.g = tensors[self.name("g")].to(device=device, dtype=torch.float32)
+
+    def export(self):
+        return {self.name("g"): self.g.cpu()}
+
+
+class GatedBlock(Block):
+    """h += mixer(norm(h)); h += gate * feed_forward(norm(h)), the gate a part of a family of its own."""
+    needs = ("mixer", "feed_forward", "mixer_norm", "feed_forward_norm", "gate")
+
+    def forward(self, ctx, h, cache):
+        self.mixer.forward(ctx, self.normed_input(ctx, h, self.mixer_norm, self.mixer, None), h, cache)
+        x = self.normed_input(ctx, h, self.feed_forward_norm, self.feed_forward, None)
+        y = torch.zeros_like(h)
+        self.feed_forward.forward(ctx, x, y)
+        h += y * self.named["gate"].g
+        ctx.note_left(h, None)
+
+
+class ToyLatentConfig:
+    """Two layers: the latent mixer in a gated block, then grouped-query attention in the usual block; no norm
+    between the last block and the output matrix."""
+
+    def __init__(self, d):
+        self.d = d
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def model_spec(self):
+        H, V = self.d["hidden_size"], self.d["vocab_size"]
+        norm = lambda p: PartSpec("rmsnorm", p, {"size": H, "eps": 1e-5})
+        ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": H, "intermediate_size": 2 * H})
+        rope = {"kind": "rope", "head_dim": 32, "rotary_dim": 32, "theta": 1e4, "layout": "split_half"}
+        att = PartSpec("attention", "l1.att", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 32, "window": None, "position": rope})
+        layers = [LayerSpec("test_gated", PartSpec("test_latent", "l0.mix", {"hidden_size": H, "latent": 24}), ffn("l0.mlp"), norm("l0.n1"), norm("l0.n2"),
+                            extra=(ExtraPart("gate", "test_gate", PartSpec("vector", "l0.gate", {"size": H})),)),
+                  LayerSpec("prenorm", att, ffn("l1.mlp"), norm("l1.n1"), norm("l1.n2"))]
+        return ModelSpec(H, V, 512, layers, [RunSpec(0), RunSpec(1)], None, "embed", "head")
+
+
+def toy_latent_reference(ws, tokens, r=lambda t: t):
+    """`r`: applied to what one kernel hands the next (the identity for the exact result; rounding to bfloat16 to see
+    what rounding alone does to these logits)."""
+    w = {k: v.double() for k, v in ws.items()}
+    T = len(tokens)
+    x = w["embed"][torch.tensor(tokens)]
+    mlp = lambda xn, p: plain_swiglu(xn, w[f"{p}.gate_proj.weight"], w[f"{p}.up_proj.weight"], w[f"{p}.down_proj.weight"], r)
+    xn = r(plain_rmsnorm(x, w["l0.n1.weight"], 1e-5))
+    c, q = xn @ w["l0.mix.c"].T, xn @ w["l0.mix.q"].T             # (the toy mixer computes in 32-bit from the normed rows)
+    s = (q @ c.T / math.sqrt(24)).masked_fill(torch.ones(T, T).triu(1).bool(), -math.inf)
+    x = x + (torch.softmax(s, dim=-1) @ c) @ w["l0.mix.o"].T
+    x = x + w["l0.gate.g"] * mlp(r(plain_rmsnorm(x, w["l0.n2.weight"], 1e-5)), "l0.mlp")
+    xn = r(plain_rmsnorm(x, w["l1.n1.weight"], 1e-5))
+    pos, inv = torch.arange(T), plain_inv_freq(32, 1e4, None)
+    qq = r(plain_rope((xn @ w["l1.att.q_proj.weight"].T).view(T, 2, 32), pos, inv))
+    kk = r(plain_rope((xn @ w["l1.att.k_proj.weight"].T).view(T, 1, 32), pos, inv))
+    vv = r((xn @ w["l1.att.v_proj.weight"].T).view(T, 1, 32))
+    x = x + r(plain_attention(qq, kk, vv, rounded=r).reshape(T, 64)) @ w["l1.att.o_proj.weight"].T
+    x = x + mlp(r(plain_rmsnorm(x, w["l1.n2.weight"], 1e-5)), "l1.mlp")
+    return r(x) @ w["head"].T                                      # no final norm
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_with_a_cache_kind_of_its_own(dtype):
+    """A need of a class the package has never seen (one latent vector per token, paged), a family of parts it has
+    never seen, and a stack without a final norm: registered here, sized, paged, given back and replayed in the four
+    cuts (whole, the tail token by token, portions, mixed with so few pages that they are used again) by the cache
+    manager, step function and trace replay as they are."""
+    from llm_rs_amd.engine import Model
+    from llm_rs_amd.engine.trace import TraceReplayer
+    from replay_cases import live_token_need, mixed, portions, tail_decoded, whole
+    from replay_checks import check_rows, run_trace
+    register_cache_kind(PagedLatent, PagedLatentKind())
+    register_mixer("test_latent", LatentMixer)
+    register_part_family("test_gate")("vector", VectorGate)
+    register_block("test_gated", GatedBlock)
+    register_architecture("TestToyLatentForCausalLM", ToyLatentConfig)
+    H, V = 48, 83
+    cfg = ToyLatentConfig({"architectures": ["TestToyLatentForCausalLM"], "hidden_size": H, "vocab_size": V})
+    names = Model(cfg.model_spec(), torch.float32, "cpu").tensors()
+    assert {"l0.gate.g", "l0.mix.c", "head"} <= set(names) and "final.weight" not in names
+    ws = {n: ((rnd(s.shape, i) * 0.1 + 1) if s.kind == "norm" else rnd(s.shape, i, 0.2)).bfloat16()
+          for i, (n, s) in enumerate(sorted(names.items()))}
+    with pytest.raises(TypeError, match="registered class"):
+        CacheManager([(("keys", 3), None)], torch.float32, DEV, 16, 4, max_requests=2)
+    # what the pool is sized by is the kinds' to say: 24 floats a token for the latents, 2 x 32 values for the keys and values
+    per_token = 4 * 24 + 2 * 32 * (4 if dtype == "float32" else 2)
+    needs = Model(cfg.model_spec(), torch.float32, "cpu").cache_needs()
+    assert needs[0][0] == PagedLatent(24)
+    assert CacheManager.pages_that_fit(needs, torch.float32 if dtype == "float32" else torch.bfloat16, 16, 10_000_000, 0.5, 64, 512) \
+        == [min(5_000_000 // per_token, 64 * 512) // 16] * 2
+    requests = {f"r{i}": torch.randint(0, V, (n,), generator=torch.Generator().manual_seed(30 + i)).tolist()
+                for i, n in enumerate((70, 41, 100, 33, 57))}
+    reference = {rid: toy_latent_reference(ws, toks) for rid, toks in requests.items()}
+    # bfloat16: as for the real models, the bound is made from what rounding between kernels alone does to these logits
+    to_bf16 = lambda t: t.to(torch.bfloat16).to(t.dtype)
+    by_rounding = max(float((toy_latent_reference(ws, toks, to_bf16) - reference[rid]).abs().max()) / float(reference[rid].abs().max())
+                      for rid, toks in requests.items())
+    allowed = 3e-5 if dtype == "float32" else 1.5 * by_rounding
+    for name, steps in (("whole", whole(requests)), ("tail", tail_decoded(requests, 32)), ("portions", portions(requests)),
+                        ("mixed", mixed(requests, live=3))):
+        need = live_token_need(steps)
+        eng = Engine(cfg, ws, dtype=dtype, page_size=16, num_pages=need // 16, max_requests=8)
+        assert len(eng.cache.groups) == 2 and eng.cache.bytes_per_token() == per_token
+        assert eng.cache.views[0].kind == "latent" and eng.cache.views[1].kind == "paged" and eng.model.final_norm is None
+        rows, _ = run_trace(lambda n: TraceReplayer.for_engine(eng), steps)
+        check_rows(rows, reference, dtype, requests, allowed)
+        core = eng.cache.core
+        assert all(core.pages_free(g) == core.pages_total(g) for g in range(2)) and core.slots_in_use() == 0, name
+    back = eng.weights()
+    assert all(torch.equal(back[n].float(), t.float()) for n, t in ws.items())
+    out = eng.generate([requests["r1"][:9]], max_new_tokens=5)[0]
+    assert len(out) == 5
+    if dtype == "float32":
+        full = toy_latent_reference(ws, requests["r1"][:9] + out)
+        assert out == [int(full[8 + i].argmax()) for i in range(5)]
