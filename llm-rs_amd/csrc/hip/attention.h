@@ -71,3 +71,9 @@ extern "C" int llmrs_attention_split_chunk(long singles, int n_kv_heads, int hea
 int llmrs_attention_f32_mfma(hipStream_t stream, const float* q, float* out, const float* k_cache, const float* v_cache,
                              const int* block_table, const int* positions, const int* q_starts, int n_entries,
                              int skip_single, const AttnArgs& a);
+// The same for entries with one token, split into chunks of F32_SPLIT_CHUNK keys whose partial results go to `partial`
+// in the layout of attention_generic.hip's split, for that file's merge.
+#define F32_SPLIT_CHUNK 128
+int llmrs_attention_f32_mfma_split(hipStream_t stream, const float* q, float* partial, const float* k_cache, const float* v_cache,
+                                   const int* block_table, const int* q_starts, const int* seq_lens, int n_entries,
+                                   int max_chunks, const AttnArgs& a);

@@ -18,6 +18,8 @@
 // [feature][slot], so a lane reads four consecutive keys of its feature at a time.
 // Needs head_dim % 32 == 0 (up to 256), page_size % 4 == 0, at most 32 heads per kv head,
 // 16-byte aligned rows; otherwise the caller keeps to the walk.
+// Entries with one token are shared out over waves by key range on the same products (attn_f32_split_kernel): a
+// decode step in 32-bit reads its keys and values once for all heads of a kv head, 16 bytes a lane.
 // Formulas: shaders/ops.metal:636-758 (scale after the dot, causal bound, softmax, weighted sum).
 #include "attention.h"
 #include "cache_layout.h"
@@ -31,47 +33,15 @@ __device__ __forceinline__ float swap_halves(float x) {
     return __uint_as_float((threadIdx.x & 32) ? sw[0] : sw[1]);
 }
 
+// One wave's walk over the keys [t_begin, t_end) (t_begin a multiple of 32) for its 32 columns: column c of this lane
+// sees the keys lo..pos (pos < 0: a column that is not there).  Adds to the running maximum m (base 2, scale applied),
+// the sum l and the sums O^T as they stand.
 template <int HD>
-__global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __restrict__ q, float* __restrict__ out,
-                                                             const float* __restrict__ kc, const float* __restrict__ vc,
-                                                             const int* __restrict__ block_table,
-                                                             const int* __restrict__ positions,
-                                                             const int* __restrict__ q_starts, int n_entries,
-                                                             AttnArgs a, int G, int tpt, int skip_single) {
-    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int c = lane & 31, h = lane >> 5;
-    int task = blockIdx.x * 4 + wave;
-    int kvh = (task >> 2) % a.n_kv_heads;
-    int tile = (task / (4 * a.n_kv_heads)) * 4 + (task & 3);
-    int e = 0, rem = 0;
-    if (!locate_tile(q_starts, n_entries, tpt, skip_single, tile, e, rem)) return;
-    int tok0 = q_starts[e] + rem * tpt;
-    int ntok = min(tpt, q_starts[e + 1] - tok0);
-    int tq = c / G, hg = c - tq * G;
-    bool cvalid = tq < ntok;
-    int token = tok0 + min(tq, ntok - 1);
-    int head = kvh * G + hg;
-    int pos = cvalid ? positions[token] : -1;
-    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-    int last = positions[tok0 + ntok - 1], first = positions[tok0];
-    int t_end = last + 1;
-    int t_begin = ((a.window > 0 && first + 1 > a.window) ? first + 1 - a.window : 0) & ~31;
-    const int* table = block_table + (size_t)e * a.table_width;
+__device__ __forceinline__ void f32_walk(const f32x4 (&qf)[HD / 8], const float* __restrict__ kc, const float* __restrict__ vc,
+                                         const int* __restrict__ table, const AttnArgs& a, int kvh, int c, int h, int pos, int lo,
+                                         int t_begin, int t_end, f32x16 (&O)[HD / 32], float& m, float& l) {
     const int ps = a.page_size;
-
-    // this lane's part of its column's query: values 8j + 4h .. 8j + 4h + 3
-    f32x4 qf[HD / 8];
-    const float* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + 4 * h;
-#pragma unroll
-    for (int j = 0; j < HD / 8; ++j) qf[j] = *(const f32x4*)(qp + 8 * j);
-    f32x16 O[HD / 32];
-#pragma unroll
-    for (int dt = 0; dt < HD / 32; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
-    float m = -INFINITY, l = 0.0f;
     const float scale_log2e = a.scale * 1.44269504088896341f;     // exponentials in base 2: one multiply-add and one v_exp_f32
-
     auto page_of = [&](int key) {
         int pg = table[min(key / ps, a.table_width - 1)];
         return min(max(pg, 0), a.num_pages - 1);                   // stay inside the cache whatever the table holds
@@ -143,6 +113,47 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
                 O[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[V_AHEAD ? dt : 0][s >> 2][s & 3], S[s], O[dt], 0, 0, 0);
         }
     }
+}
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __restrict__ q, float* __restrict__ out,
+                                                             const float* __restrict__ kc, const float* __restrict__ vc,
+                                                             const int* __restrict__ block_table,
+                                                             const int* __restrict__ positions,
+                                                             const int* __restrict__ q_starts, int n_entries,
+                                                             AttnArgs a, int G, int tpt, int skip_single) {
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int c = lane & 31, h = lane >> 5;
+    int task = blockIdx.x * 4 + wave;
+    int kvh = (task >> 2) % a.n_kv_heads;
+    int tile = (task / (4 * a.n_kv_heads)) * 4 + (task & 3);
+    int e = 0, rem = 0;
+    if (!locate_tile(q_starts, n_entries, tpt, skip_single, tile, e, rem)) return;
+    int tok0 = q_starts[e] + rem * tpt;
+    int ntok = min(tpt, q_starts[e + 1] - tok0);
+    int tq = c / G, hg = c - tq * G;
+    bool cvalid = tq < ntok;
+    int token = tok0 + min(tq, ntok - 1);
+    int head = kvh * G + hg;
+    int pos = cvalid ? positions[token] : -1;
+    int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+    int last = positions[tok0 + ntok - 1], first = positions[tok0];
+    int t_end = last + 1;
+    int t_begin = ((a.window > 0 && first + 1 > a.window) ? first + 1 - a.window : 0) & ~31;
+    const int* table = block_table + (size_t)e * a.table_width;
+
+    // this lane's part of its column's query: values 8j + 4h .. 8j + 4h + 3
+    f32x4 qf[HD / 8];
+    const float* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + 4 * h;
+#pragma unroll
+    for (int j = 0; j < HD / 8; ++j) qf[j] = *(const f32x4*)(qp + 8 * j);
+    f32x16 O[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, t_begin, t_end, O, m, l);
     if (!cvalid) return;
     float inv = 1.0f / l;
     float* op = out + (size_t)token * a.out_stride + (size_t)head * HD + 4 * h;
@@ -155,6 +166,56 @@ __global__ __launch_bounds__(256) void attn_f32_tiles_kernel(const float* __rest
             for (int j = 0; j < 4; ++j) v[j] = O[dt][4 * g + j] * inv;
             *(f32x4*)(op + dt * 32 + 8 * g) = v;
         }
+}
+
+// Entries with one token: a wave for each (entry, kv head, chunk of F32_SPLIT_CHUNK keys, aligned to absolute positions):
+// its columns are the heads of the kv head (the other columns of the 32 multiply zeros: the keys and values are read
+// once for all of them, 16 bytes a lane, which is what this step is bound by).  It leaves what the walk of
+// attention_generic.hip leaves for such a chunk, where that file's merge finds it: the maximum (natural logarithm's
+// scale), the sum and the weighted values of each head, [entry][head][chunk][2 + head_dim].
+template <int HD>
+__global__ __launch_bounds__(64) void attn_f32_split_kernel(const float* __restrict__ q, float* __restrict__ partial,
+                                                            const float* __restrict__ kc, const float* __restrict__ vc,
+                                                            const int* __restrict__ block_table,
+                                                            const int* __restrict__ q_starts, const int* __restrict__ seq_lens,
+                                                            int max_chunks, AttnArgs a, int G) {
+    int lane = threadIdx.x, c = lane & 31, h = lane >> 5;
+    int e = blockIdx.x, kvh = blockIdx.y, ch = blockIdx.z;
+    int token = q_starts[e];
+    if (q_starts[e + 1] - token != 1) return;
+    int pos_t = seq_lens[e] - 1;                  // an entry with one token: its position is its length less one
+    int lo = (a.window > 0 && pos_t + 1 > a.window) ? pos_t + 1 - a.window : 0;
+    int first = lo / F32_SPLIT_CHUNK;
+    if (ch > pos_t / F32_SPLIT_CHUNK - first) return;
+    int begin = max(lo, (first + ch) * F32_SPLIT_CHUNK), end = min(pos_t + 1, (first + ch + 1) * F32_SPLIT_CHUNK);
+    bool cvalid = c < G;
+    int head = kvh * G + min(c, G - 1);
+    int pos = cvalid ? pos_t : -1;
+    const int* table = block_table + (size_t)e * a.table_width;
+    f32x4 qf[HD / 8];
+    const float* qp = q + (size_t)token * a.q_stride + (size_t)head * HD + 4 * h;
+#pragma unroll
+    for (int j = 0; j < HD / 8; ++j) qf[j] = *(const f32x4*)(qp + 8 * j);
+    f32x16 O[HD / 32];
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[dt][i] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+    f32_walk<HD>(qf, kc, vc, table, a, kvh, c, h, pos, lo, begin & ~31, end, O, m, l);
+    if (!cvalid) return;
+    float* pp = partial + ((size_t)(e * a.n_heads + head) * max_chunks + ch) * (HD + 2);
+    if (h == 0) { pp[0] = m * 0.69314718055994531f; pp[1] = l; }
+    // this lane holds features dt * 32 + 8 g + 4 h + j of its column (rows of 2 + head_dim floats: 8-byte aligned)
+#pragma unroll
+    for (int dt = 0; dt < HD / 32; ++dt)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+                float2 v = make_float2(O[dt][4 * g + j], O[dt][4 * g + j + 1]);
+                *(float2*)(pp + 2 + dt * 32 + 8 * g + 4 * h + j) = v;
+            }
 }
 
 // Takes the entries with several tokens (all entries when skip_single is 0).  Returns 1 when it took them,
@@ -180,6 +241,31 @@ int llmrs_attention_f32_mfma(hipStream_t stream, const float* q, float* out, con
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         llmrs_fail("attention (32-bit tiles): launch failed: %s", hipGetErrorString(err));
+        return -1;
+    }
+    return 1;
+}
+
+// Takes the entries with one token, split by key range into `partial` (max_chunks chunks of F32_SPLIT_CHUNK keys an
+// entry; the caller merges them).  Returns 1 when it took them, 0 when the shape is not its own, -1 on error.
+int llmrs_attention_f32_mfma_split(hipStream_t stream, const float* q, float* partial, const float* k_cache, const float* v_cache,
+                                   const int* block_table, const int* q_starts, const int* seq_lens, int n_entries,
+                                   int max_chunks, const AttnArgs& a) {
+    int G = a.n_heads / a.n_kv_heads;
+    if (a.head_dim % 32 || a.head_dim > 256 || a.page_size % 4 || G > 32 || q_starts == nullptr || seq_lens == nullptr) return 0;
+    if (a.q_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)k_cache & 15) || ((uintptr_t)v_cache & 15) || ((uintptr_t)partial & 7))
+        return 0;
+    if (n_entries > 65535 || a.n_kv_heads > 65535 || max_chunks > 65535 || max_chunks < 1) return 0;
+    dim3 grid(n_entries, a.n_kv_heads, max_chunks);
+    switch (a.head_dim) {
+#define CASE(HD) case HD: attn_f32_split_kernel<HD><<<grid, 64, 0, stream>>>(q, partial, k_cache, v_cache, block_table, q_starts, seq_lens, max_chunks, a, G); break;
+        CASE(32) CASE(64) CASE(96) CASE(128) CASE(160) CASE(192) CASE(224) CASE(256)
+#undef CASE
+        default: return 0;
+    }
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        llmrs_fail("attention (32-bit split): launch failed: %s", hipGetErrorString(err));
         return -1;
     }
     return 1;

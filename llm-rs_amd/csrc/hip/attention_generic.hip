@@ -287,7 +287,8 @@ __global__ __launch_bounds__(64) void attention_generic_group_kernel(
     }
 }
 
-// One wave for each (entry, head) adds the chunks up, in ascending order.
+// One wave for each (entry, head) adds the chunks up.  The chunks' maxima and sums are read 64 at a time, a lane
+// each; the weighted values are added chunk by chunk in ascending order, four chunks' rows asked for at a time.
 template <class T>
 __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
     const float* __restrict__ partial, T* __restrict__ out, const int* __restrict__ q_starts,
@@ -299,18 +300,42 @@ __global__ __launch_bounds__(64) void attention_generic_merge_kernel(
     int lo = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
     int n_chunks = pos / GENERIC_CHUNK - lo / GENERIC_CHUNK + 1;
     const float* pp = partial + (size_t)(e * a.n_heads + h) * max_chunks * (hd + 2);
-    int stride = hd + 2;
+    const size_t stride = hd + 2;
     float M = -INFINITY;
-    for (int ch = 0; ch < n_chunks; ++ch) M = fmaxf(M, pp[(size_t)ch * stride]);
+    for (int ch = lane; ch < n_chunks; ch += 64) M = fmaxf(M, pp[(size_t)ch * stride]);
+    M = wave_max(M);
     float L = 0.0f;
     float o[MAX_HEAD_DIM / 64] = {};
-    for (int ch = 0; ch < n_chunks; ++ch) {
-        float w = expf(pp[(size_t)ch * stride] - M);
-        L = fmaf(pp[(size_t)ch * stride + 1], w, L);
+    for (int base = 0; base < n_chunks; base += 64) {
+        int mine = base + lane;
+        float w_mine = mine < n_chunks ? expf(pp[(size_t)mine * stride] - M) : 0.0f;
+        float l_mine = mine < n_chunks ? pp[(size_t)mine * stride + 1] * w_mine : 0.0f;
+        L += wave_sum(l_mine);
+        int n = min(64, n_chunks - base);
+        int j = 0;
+        for (; j + 4 <= n; j += 4) {
+            float v[4][MAX_HEAD_DIM / 64];
 #pragma unroll
-        for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
-            int d = lane + 64 * i;
-            if (d < hd) o[i] = fmaf(pp[(size_t)ch * stride + 2 + d], w, o[i]);
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
+                    int d = lane + 64 * i;
+                    v[u][i] = d < hd ? pp[(size_t)(base + j + u) * stride + 2 + d] : 0.0f;
+                }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                float w = __shfl(w_mine, j + u, 64);
+#pragma unroll
+                for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) o[i] = fmaf(v[u][i], w, o[i]);
+            }
+        }
+        for (; j < n; ++j) {
+            float w = __shfl(w_mine, j, 64);
+#pragma unroll
+            for (int i = 0; i < MAX_HEAD_DIM / 64; ++i) {
+                int d = lane + 64 * i;
+                if (d < hd) o[i] = fmaf(pp[(size_t)(base + j) * stride + 2 + d], w, o[i]);
+            }
         }
     }
     T* orow = out + (size_t)t * a.out_stride + (size_t)h * hd;
@@ -374,10 +399,23 @@ static int launch_generic(hipStream_t stream, const T* q, T* out, const T* k_cac
         }
     }
     if (split) {
+        static_assert(F32_SPLIT_CHUNK == GENERIC_CHUNK, "the matrix-core split leaves its chunks where this file's merge looks for them");
+        bool mfma_took = false;
+        if constexpr (std::is_same<T, float>::value) {
+            // 32-bit: the single tokens' chunks on the matrix cores where the shape allows (one wave reads a chunk's keys
+            // and values once for all heads of a kv head)
+            if (allow_mfma) {
+                int took = llmrs_attention_f32_mfma_split(stream, q, scratch, k_cache, v_cache, block_table, q_starts, seq_lens,
+                                                          n_entries, max_chunks, a);
+                if (took < 0) return -1;
+                mfma_took = took == 1;
+            }
+        }
         // a wave for all heads of a kv head when that still leaves two waves or more for each compute unit
         // (measured in 32-bit at the 8B shape, 2048 keys: 8 requests 174 -> 88 us; one request alone is faster with a wave per head)
         long group_waves = (long)(n_single > 0 ? n_single : n_entries) * a.n_kv_heads * max_chunks;
-        if (groupable && group_waves >= 2L * llmrs_compute_units()) {
+        if (mfma_took) {
+        } else if (groupable && group_waves >= 2L * llmrs_compute_units()) {
             dim3 grid(n_entries, a.n_kv_heads, max_chunks);
 #define GROUP(V, GG) attention_generic_group_kernel<T, V, GG><<<grid, 64, 0, stream>>>(q, scratch, k_cache, v_cache, block_table, q_starts, seq_lens, max_chunks, a)
             if (G == 8) { if (vec) GROUP(true, 8); else GROUP(false, 8); }
