@@ -27,6 +27,10 @@ The other workloads print one line of the same form each:
             tiles: tokens a second and the share of the matrix cores' peak for each; value = the 2,048-token one.
   long      the 8B shape with the 131,072 positions of Llama 3.1: one request decoding over 131,000 keys and four over
             32,700 each, with their shares of the HBM roofline (filling the caches takes about ten seconds).
+  widths    the four products of a layer alone, at widths that are none of the three Llama shapes the kernels' choices
+            were timed on (hidden 1536 to 6144, odd intermediates), at 1, 8, 64, 256 and 2048 rows: GB/s of weights or
+            TFLOP/s for each, so that a width that falls into a poor choice shows; value = the worst share of the best
+            share seen at the same number of rows.
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -57,7 +61,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -422,6 +426,65 @@ def run_mixed70b(args) -> dict:
                       host_share(step_s, dev_s))
 
 
+def run_widths(args) -> dict:
+    """The products q/k/v, o, gate/up and down of one layer at other widths, in a HIP graph, back to back over
+    different weights (so that no weight is read twice in a row)."""
+    import torch
+    from llm_rs_amd.kernels import EPI_ACCUM_F32, EPI_STORE, EPI_SWIGLU, kernels
+    k, dev = kernels(), "cuda:0"
+    # (hidden, heads x head size of q, kv heads x head size, intermediate)
+    shapes = [(1536, 1536, 256, 8960), (2560, 2560, 640, 6912), (3072, 3072, 1024, 8192), (3584, 3584, 512, 18944),
+              (5120, 5120, 1024, 13824), (6144, 6144, 1024, 16384), (4096, 4096, 1024, 11008)]
+    rows_list = (1, 8, 64, 256, 2048)
+    points, best = {}, {}
+    for hidden, qd, kvd, inter in shapes:
+        products = {"qkv": (qd + 2 * kvd, hidden, EPI_STORE), "o": (hidden, qd, EPI_ACCUM_F32),
+                    "gate_up": (2 * inter, hidden, EPI_SWIGLU), "down": (hidden, inter, EPI_ACCUM_F32)}
+        for name, (N, K, epi) in products.items():
+            copies = max(2, min(8, int(600e6 // (N * K * 2))))          # enough different weights to pass the caches
+            ws = [(torch.randn(N, K, device=dev) * 0.02).bfloat16() for _ in range(copies)]
+            for M in rows_list:
+                x = torch.randn(M, K, device=dev).bfloat16()
+                out = torch.zeros(M, N // 2 if epi == EPI_SWIGLU else N, device=dev,
+                                  dtype=torch.float32 if epi == EPI_ACCUM_F32 else torch.bfloat16)
+                n_ws = k.gemm_workspace_floats(M, N, K)
+                wsp = torch.empty(max(n_ws, 1), dtype=torch.float32, device=dev) if n_ws else None
+                for w in ws:
+                    k.gemm(x, w, out, epi, wsp)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for _ in range(4):
+                        for w in ws:
+                            k.gemm(x, w, out, epi, wsp)
+                graph.replay()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(5):
+                    graph.replay()
+                torch.cuda.synchronize()
+                sec = (time.perf_counter() - t0) / (5 * 4 * copies)
+                hbm = N * K * 2 / sec / PEAK_HBM
+                mfma = 2.0 * M * N * K / sec / PEAK_FLOPS["bfloat16"]
+                share = max(hbm, mfma)              # of whichever roof the product is nearer to
+                key = f"{name}_{N}x{K}_m{M}"
+                points[key] = round(share, 4)
+                best[M] = max(best.get(M, 0.0), share)
+                print(f"[bench] {key}: {sec * 1e6:8.1f} us  {hbm * 100:5.1f}% of HBM  {mfma * 100:5.1f}% of the matrix peak", file=sys.stderr, flush=True)
+                del graph
+            del ws
+    worst = min(points, key=lambda kk: points[kk] / best[int(kk.rsplit("_m", 1)[1])])
+    rel = points[worst] / best[int(worst.rsplit("_m", 1)[1])]
+    line = base_line("the worst product's share of its roof (HBM for few rows, matrix cores for many) against the best seen at the same "
+                     "number of rows, over the four products of a layer at seven other widths", rel, 20, 0, 0.0, "bfloat16",
+                     {"model": "other widths", "global_batch": 0, "seq_len": 0, "parallelism": "single GPU"})
+    line["unit"] = "ratio"
+    line["worst"] = worst
+    line["best_share_by_rows"] = {str(m): round(v, 4) for m, v in best.items()}
+    line["points"] = points
+    return line
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -447,7 +510,7 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts, "long": run_long}[args.workload](args)
+            "prompts": run_prompts, "long": run_long, "widths": run_widths}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()

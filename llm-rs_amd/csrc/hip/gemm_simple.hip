@@ -236,6 +236,106 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const T* __restrict__ A,
     }
 }
 
+// Up to 16 tokens in 32-bit on the matrix cores: v_mfma_f32_16x16x4_f32 multiplies and adds in 32-bit (no
+// reduced-precision mode).  The weight's rows are the A operand, read once, 16 bytes a lane (lane l: feature
+// l % 16 of a tile, the four k-values 4 (l / 16) .. + 3 of a group of 16); the tokens' rows are the B operand, read
+// the same way once for all of a block's NT feature tiles, so that the tokens cost a load for every NT loads of
+// weights where the walk above asks for every token's row again for every two or four rows of the weight.  An MFMA
+// contracts the four k-values that the four lane groups hold in the same place of their loads.  A block's NW waves
+// take the 32-wide k-blocks in turn, U of them with all loads asked for before the first product, and add their sums
+// through LDS in wave order: an output's sum depends on K (and on the weight's shape, which chooses NW) only.
+// C: lane l holds token l % 16 and features 4 (l / 16) + r.  Needs K % 32 == 0 and 16-byte aligned rows.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <int NT, int NW, int U>
+__global__ __launch_bounds__(NW * 64) void gemm_f32_skinny_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W,
+                                                                  void* __restrict__ out, int ldc, int M, int N, int K, int epi) {
+    extern __shared__ __attribute__((aligned(16))) float f32_skinny_red[];       // [NW][NT][4][64]
+    float* red = f32_skinny_red;
+    int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int row = lane & 15, g = lane >> 4;
+    int n0 = blockIdx.x * NT * 16;
+    const float* wp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) wp[nt] = W + (size_t)min(n0 + nt * 16 + row, N - 1) * K + 4 * g;
+    const float* xp = A + (size_t)min(row, M - 1) * lda + 4 * g;
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int nkb = K / 32;
+    auto products = [&](const f32x4_t (&w)[NT][2], const f32x4_t (&x)[2]) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[nt][half][j], x[half][j], acc[nt], 0, 0, 0);
+    };
+    int kb = wave;
+    for (; kb + (U - 1) * NW < nkb; kb += U * NW) {
+        f32x4_t w[U][NT][2], x[U][2];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            int k = (kb + u * NW) * 32;
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) { w[u][nt][0] = *(const f32x4_t*)(wp[nt] + k); w[u][nt][1] = *(const f32x4_t*)(wp[nt] + k + 16); }
+            x[u][0] = *(const f32x4_t*)(xp + k);
+            x[u][1] = *(const f32x4_t*)(xp + k + 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // keep the round's loads together, ahead of its products
+#pragma unroll
+        for (int u = 0; u < U; ++u) products(w[u], x[u]);
+    }
+    for (; kb < nkb; kb += NW) {
+        f32x4_t w[NT][2], x[2];
+        int k = kb * 32;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) { w[nt][0] = *(const f32x4_t*)(wp[nt] + k); w[nt][1] = *(const f32x4_t*)(wp[nt] + k + 16); }
+        x[0] = *(const f32x4_t*)(xp + k);
+        x[1] = *(const f32x4_t*)(xp + k + 16);
+        products(w, x);
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[((wave * NT + nt) * 4 + r) * 64 + lane] = acc[nt][r];
+    __syncthreads();
+    // the block's feature tiles are shared out over its waves; each is summed over the waves in order
+    for (int nt = wave; nt < NT; nt += NW) {
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float s = 0.0f;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) s += red[((w2 * NT + nt) * 4 + r) * 64 + lane];
+            v[r] = s;
+        }
+        int m = row, n = n0 + nt * 16 + 4 * g;
+        if (m >= M) continue;
+        if (epi == LLMRS_EPI_SWIGLU) {
+#pragma unroll
+            for (int r = 0; r < 4; r += 2)
+                if (n + r + 1 < N) ((float*)out)[(size_t)m * ldc + (n + r) / 2] = silu_f32(v[r]) * v[r + 1];
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (n + r < N) epilogue_store<float>(epi, out, ldc, m, n + r, v[r]);
+        }
+    }
+}
+
+template <int NT, int NW, int U>
+static void launch_f32_skinny(hipStream_t stream, const float* A, int lda, const float* W, void* out, int ldc, int M, int N, int K, int epi) {
+    size_t bytes = (size_t)NW * NT * 4 * 64 * sizeof(float);
+    static_assert((size_t)NW * NT * 4 * 64 * sizeof(float) <= 64 * 1024, "the waves' sums must fit in the LDS a block may ask for");
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)gemm_f32_skinny_kernel<NT, NW, U>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        configured = true;
+    }
+    gemm_f32_skinny_kernel<NT, NW, U><<<ceil_div(N, NT * 16), NW * 64, bytes, stream>>>(A, lda, W, out, ldc, M, N, K, epi);
+}
+
 // A: [M, K] with row stride lda; W: [N, K] dense; out: row stride ldc (elements of
 // its own type; for SWIGLU the output has N/2 columns).  workspace: optional device
 // memory (16 * 64 * N * 4 bytes is always enough) for products that split K over blocks.
@@ -265,6 +365,25 @@ extern "C" int llmrs_gemm(hipStream_t stream, int dtype, const void* A, int lda,
         if (took != 0) return took < 0 ? -1 : 0;
     }
     LLMRS_REQUIRE(scale_sumsq == nullptr && next_y == nullptr, "gemm: a deferred norm needs the bfloat16 matrix-core kernels (M=%d N=%d K=%d)", M, N, K);
+    // (one or two tokens are better off with the walk below, which then asks for little beside the weights:
+    // a decode step of the 8B shape at one request 7.1 against 7.8 ms)
+    if (dtype == LLMRS_F32 && allow_mfma && M > 2 && M <= 16 && K % 32 == 0 && lda % 4 == 0 && ((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0) {
+        // (the waves per block follow the weight's shape alone, so a row's sums do not depend on the batch)
+        const float* a = (const float*)A;
+        const float* w = (const float*)W;
+        // (blocks of 7 tiles with one wave a SIMD and one k-block in flight took 92 us for the 8B shape's gate/up
+        // weight: a 32-bit MFMA is long, and the wave's loads and products took turns; two waves a SIMD, two k-blocks each)
+        int cus = llmrs_compute_units();
+        if (N >= 16384) {
+            if (N % 112 == 0) launch_f32_skinny<7, 8, 2>(stream, a, lda, w, out, ldc, M, N, K, epi);
+            else launch_f32_skinny<4, 4, 2>(stream, a, lda, w, out, ldc, M, N, K, epi);
+        } else if (K >= 2048 && (ceil_div(N, 16) <= cus || ceil_div(N, 16) > 2 * cus)) launch_f32_skinny<1, 8, 4>(stream, a, lda, w, out, ldc, M, N, K, epi);
+        // between one and two blocks a unit: blocks of four waves, two of which a unit holds side by side, make it one round
+        else if (K >= 2048) launch_f32_skinny<1, 4, 8>(stream, a, lda, w, out, ldc, M, N, K, epi);
+        else launch_f32_skinny<1, 4, 4>(stream, a, lda, w, out, ldc, M, N, K, epi);
+        LLMRS_LAUNCH_CHECK("gemm");
+        return 0;
+    }
     if (M <= GEMV_MAX_M) {
         size_t elt = dtype == LLMRS_F32 ? sizeof(float) : sizeof(bf16);
         bool vec = K % 4 == 0 && lda % 4 == 0 && (uintptr_t)A % (4 * elt) == 0 && (uintptr_t)W % (4 * elt) == 0;
