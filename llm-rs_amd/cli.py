@@ -40,7 +40,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--config", help="a config.json; with --random-weights in place of --model")
     ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
                     help="weights drawn from this seed for the configuration of --config (or of --model's folder)")
-    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32", "bf16", "f32"],
+                    type=lambda d: {"bf16": "bfloat16", "f32": "float32", "fp32": "float32"}.get(d, d))
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--num-pages", type=int, default=None, help="KV pages (default: sized from free memory)")
     ap.add_argument("--max-batch-tokens", type=int, default=2048,

@@ -50,6 +50,8 @@ def test_argument_errors(tmp_path, capsys):
     assert (args.config, args.random_weights, args.prompt, args.prompt_len) == ("c.json", 5, "1,2", None)
     args = cli.build_parser().parse_args(["-m", "x", "replay", "--out", "o", "--max-tokens", "128"])
     assert (args.command, args.out, args.max_tokens) == ("replay", "o", 128)
+    assert cli.build_parser().parse_args(["-m", "x", "--dtype", "f32", "bench"]).dtype == "float32"
+    assert cli.build_parser().parse_args(["-m", "x", "--dtype", "bf16", "bench"]).dtype == "bfloat16"
     args = cli.build_parser().parse_args(["-m", "x", "bench"])
     assert (args.prompt_len, args.batch, args.context) == (2048, 8, 2048)
     with pytest.raises(SystemExit, match="token ids"):

@@ -382,6 +382,77 @@ def test_attention_at_131008_keys():
         assert (got[0].float() - ref).abs().max() <= 4e-3 + 2e-2 * float(ref.abs().max()), f"random query {i}"
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", [(8, 2, 128, 16, 0), (3, 3, 64, 8, 0), (6, 2, 96, 16, 300), (32, 1, 32, 4, 0),
+                                                        (4, 4, 160, 16, 130), (16, 2, 256, 32, 0)])
+def test_attention_float32_decoding_requests(n_heads, n_kv, hd, ps, window):
+    """Single tokens in 32-bit: a wave of the matrix-core split takes a chunk of 128 keys for all heads of a kv head (1,
+    3, 4, 8 and 32 of them here).  Lengths at and around the chunks' edges, with and without a window whose edge cuts
+    a chunk; each query matches one key strongly, at the first and last key it may see and at the chunks' edges, so
+    the output must be that key's value; and random queries agree with the plain formula to 32-bit rounding."""
+    lens = [1, 127, 128, 129, 256, 257, 700, 1500]
+    case = PagedCase(torch.float32, lens, n_heads, n_kv, hd, ps, seed=31)
+    G = n_heads // n_kv
+    g = torch.Generator().manual_seed(4)
+    for shift in range(3):
+        qs, fars = [], []
+        for r, n in enumerate(lens):
+            lo = max(0, n - window) if window else 0
+            seen = sorted({e for e in (lo, lo + 1, n - 1, 127, 128, 255, 256, n - 2, (lo + n) // 2) if lo <= e < n})
+            far = seen[(r + shift * 2) % len(seen)]
+            fars.append(far)
+            qs.append((case.k[r][far].repeat_interleave(G, dim=0) * 8.0).unsqueeze(0))
+        got = case.run(qs, [[n - 1] for n in lens], window=window, n_single=len(lens), single_keys=sum(lens))
+        for r in range(len(lens)):
+            want = case.v[r][fars[r]].repeat_interleave(G, dim=0)
+            ref = case.reference(r, qs[r], [lens[r] - 1], window=window)[0].float()
+            if lens[r] > 1:
+                assert (ref - want).abs().max() < 0.05, "the case itself"
+            assert (got[r] - ref).abs().max() <= 1e-4, f"request of length {lens[r]}, key {fars[r]}"
+    qs = [torch.randn((1, n_heads, hd), generator=g) for _ in lens]
+    got = case.run(qs, [[n - 1] for n in lens], window=window, n_single=len(lens), single_keys=sum(lens))
+    for r in range(len(lens)):
+        ref = case.reference(r, qs[r], [lens[r] - 1], window=window)[0]
+        err = (got[r].double() - ref).abs()
+        assert (err <= out_tol(ref, torch.float32, 2e-6)).all(), f"request of length {lens[r]}: {float(err.max())}"
+
+
+@pytest.mark.parametrize("M,N,K", [(3, 48, 64), (8, 4096, 4096), (16, 6144, 2048), (5, 130, 96), (9, 28672, 256), (12, 16400, 128),
+                                   (16, 2048, 8192), (7, 5000, 1024), (4, 100, 32)])
+def test_gemm_float32_few_rows_on_the_matrix_cores(M, N, K):
+    """3 to 16 rows in 32-bit: the product on v_mfma_f32_16x16x4_f32 against float64, every epilogue, rows with a
+    stride, weights whose last feature tile is cut by N, and against the walk that takes the same product when the
+    matrix cores are switched off (both true 32-bit: they differ by the order of their sums only)."""
+    a_full = rnd((M, K + 24), torch.float32, 3)
+    a = a_full[:, :K]
+    w = rnd((N, K), torch.float32, 4, 0.1)
+    acc = a.double().cpu() @ w.double().cpu().T
+    k = kernels()
+    for epi in (EPI_STORE, EPI_STORE_F32, EPI_ACCUM_F32, EPI_SWIGLU):
+        outs = []
+        for mfma in (True, False):
+            k.allow_mfma = mfma
+            try:
+                if epi == EPI_ACCUM_F32:
+                    out = rnd((M, N), torch.float32, 5)
+                    ref = out.double().cpu() + acc
+                elif epi == EPI_SWIGLU:
+                    out = torch.zeros((M, N // 2), dtype=torch.float32, device=DEV)
+                    ref = plain_silu(acc[:, 0::2]) * acc[:, 1::2]
+                else:
+                    out = torch.zeros((M, N), dtype=torch.float32, device=DEV)
+                    ref = acc
+                k.gemm(a, w, out, epi)
+            finally:
+                k.allow_mfma = True
+            err = (out.double().cpu() - ref).abs()
+            floor = 2e-6 * math.sqrt(K)
+            if epi == EPI_SWIGLU:
+                floor *= 1 + 0.1 * math.sqrt(K)      # a sum's rounding error is multiplied by the other factor, of size 0.1 sqrt(K)
+            assert (err <= out_tol(ref, torch.float32, floor)).all(), (epi, mfma, float(err.max()))
+            outs.append(out.cpu())
+        assert ((outs[0] - outs[1]).abs().double() <= 2 * out_tol(ref, torch.float32, floor)).all()
+
+
 def test_attention_chunk_rule_and_its_scratch():
     """The keys per wave that the split takes: a power of two from 64 to 1024 whatever the host says about the
     keys; never under what the scratch is sized by (the answer for one key); and the same results whichever chunk
