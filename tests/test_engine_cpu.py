@@ -154,3 +154,38 @@ def test_cancel_while_a_step_is_in_flight(engine_a):
     assert len(got[a]) == 1
     core = eng.cache.core
     assert core.pages_free() == 24 and core.slots_in_use() == 0 and not core.in_flight()
+
+
+@pytest.mark.parametrize("when", ["before the scheduler is told", "after the scheduler is told"])
+@pytest.mark.parametrize("at_step", [1, 3, 6])
+def test_an_interrupt_while_a_step_lands_leaves_engine_and_scheduler_agreeing(engine_a, when, at_step):
+    """generate() is interrupted inside the landing of a step, once before the scheduler has taken the step's
+    samples and once right after, with another step already started ahead.  The interrupt itself comes out (not an
+    error about a step nobody knows), nothing is left held, and the engine generates the same tokens afterwards."""
+    eng, tensors = engine_a
+    assert eng.overlap
+    core = eng.cache.core
+    real, calls = core.commit, [0]
+
+    def commit(sampled):
+        calls[0] += 1
+        if calls[0] == at_step and when.startswith("before"):
+            raise KeyboardInterrupt
+        finished = real(sampled)
+        if calls[0] == at_step:
+            raise KeyboardInterrupt
+        return finished
+
+    prompts = [[5, 6, 7], [9, 1], [3, 3, 3, 3, 8, 2, 1]]
+    core.commit = commit
+    try:
+        with pytest.raises(KeyboardInterrupt):
+            eng.generate(prompts, max_new_tokens=6)
+    finally:
+        core.commit = real
+    assert calls[0] >= at_step
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0
+    assert not core.in_flight() and not eng.has_unfinished() and core.idle()
+    got = eng.generate(prompts, max_new_tokens=6)
+    assert got == [plain_generate(TINY_A, tensors, p, 6) for p in prompts]
+    assert core.pages_free() == core.pages_total() and core.slots_in_use() == 0 and not core.in_flight()
