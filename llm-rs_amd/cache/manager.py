@@ -99,18 +99,35 @@ class CacheManager:
 
     @staticmethod
     def pages_that_fit(needs: Sequence[Tuple[object, Optional[int]]], dtype: torch.dtype, page_size: int, free_bytes: int,
-                       fraction: float, max_requests: int, max_seq_len: int) -> List[int]:
+                       fraction: float, max_requests: int, max_seq_len: int, max_step_tokens: int = 0) -> List[int]:
         """Pages for each group such that all of them take `fraction` of `free_bytes` less what the per-request
-        needs take, and no more than `max_requests` requests of `max_seq_len` tokens could ever fill
-        (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM)."""
+        needs take (src/kv_pool.rs:26-35 sizes its pool the same way, from RAM).  No group gets more than
+        `max_requests` requests could ever hold: `max_seq_len` tokens each, or, in a group with a window, the
+        window and the `max_step_tokens` tokens of a step's portion; what such a group does not need goes to the
+        others."""
         group_needs, layers_in_group, _, per_request = _group_runs(needs)
         if not group_needs:
             return []
         fixed = sum(cache_kind(needs[i][0]).bytes_per_request(needs[i][0]) for i in per_request) * max_requests
-        per_token = sum(n * cache_kind(need).bytes_per_token(need, dtype) for need, n in zip(group_needs, layers_in_group))
-        tokens = int(max(free_bytes - fixed, 0) * fraction) // max(per_token, 1)
-        tokens = min(tokens, max_requests * max_seq_len)
-        return [max(tokens // page_size, 1)] * len(group_needs)
+        budget = int(max(free_bytes - fixed, 0) * fraction)
+        step = min(max_step_tokens or max_seq_len, max_seq_len)
+        caps, costs = [], []
+        for need, n_layers in zip(group_needs, layers_in_group):
+            kind = cache_kind(need)
+            held = max_seq_len
+            if kind.window(need) > 0:
+                # a page's worth more than the span: the span starts anywhere in a page
+                held = min(held, kind.window(need) + step + page_size)
+            caps.append(max_requests * -(-held // page_size))
+            costs.append(n_layers * kind.bytes_per_token(need, dtype) * page_size)
+        lo, hi = 1, max(caps)          # the most pages P with sum(cost * min(cap, P)) within the budget, at least one
+        while lo < hi:
+            mid = (lo + hi + 1) // 2
+            if sum(c * min(cap, mid) for c, cap in zip(costs, caps)) <= budget:
+                lo = mid
+            else:
+                hi = mid - 1
+        return [min(cap, lo) for cap in caps]
 
     def bytes_per_token(self) -> int:
         return sum(g.bytes_per_token() for g in self.groups)

@@ -93,7 +93,7 @@ class Engine:
         self.max_seq_len = min(max_seq_len or spec.max_positions, spec.max_positions)
         needs = self.model.cache_needs()
         if num_pages is None:
-            num_pages = self._pages_from_memory(needs, page_size, kv_memory_fraction, max_requests)
+            num_pages = self._pages_from_memory(needs, page_size, kv_memory_fraction, max_requests, max_chunk or max_batch_tokens)
         self.cache = CacheManager(needs, self.dtype, self.device, page_size, num_pages, max_requests,
                                   token_budget=max_batch_tokens, max_chunk=max_chunk, max_positions=self.max_seq_len)
         self.runner = StepRunner(self.model, self.cache, self.device)
@@ -151,7 +151,7 @@ class Engine:
         """The model's tensors on the host, by file name and in the file's layout (`Model.weights`)."""
         return self.model.weights()
 
-    def _pages_from_memory(self, needs, page_size, fraction, max_requests):
+    def _pages_from_memory(self, needs, page_size, fraction, max_requests, max_step_tokens):
         """Pages that fit `fraction` of the memory still free after the weights and after what every request
         slot gets of fixed size; what a token and a slot cost is the cache kinds' to say."""
         if self.device.type != "cuda":
@@ -159,7 +159,8 @@ class Engine:
                 raise ValueError("num_pages must be given when the engine is not on a GPU")
             return []
         free, _ = torch.cuda.mem_get_info(self.device)
-        return CacheManager.pages_that_fit(needs, self.dtype, page_size, free, fraction, max_requests, self.max_seq_len)
+        return CacheManager.pages_that_fit(needs, self.dtype, page_size, free, fraction, max_requests, self.max_seq_len,
+                                           max_step_tokens)
 
     # -- manual stepping (trace replay, tests) -----------------------------------
     def open_request(self) -> int:

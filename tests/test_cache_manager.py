@@ -160,3 +160,38 @@ def test_batch_words():
         core.build_batch([a], [3], [2], [1, 2], [], words)       # position 4 was never ensured
     with pytest.raises(CoreError, match="words"):
         core.build_batch([a], [0], [3], [1, 2, 3], [], np.zeros(4, dtype=np.int32))
+
+
+def test_pool_sizes_from_memory_give_a_window_only_what_it_can_hold():
+    """Two groups, one with a window: the windowed one is given what `max_requests` requests can hold at once (the
+    window, a step's portion, and a page for where the span starts), the other the rest, and the most any request
+    ever holds in the windowed group (measured on the host core, portion after portion) stays within its share."""
+    import torch
+    from llm_rs_amd.cache import CacheManager, PagedKV
+    full, windowed = PagedKV(2, 32), PagedKV(2, 32, window=40)
+    needs = [(full, None), (windowed, None), (full, None), (windowed, 1)]        # the last run reads run 1's cache
+    page, requests, seq, step = 16, 4, 4096, 48
+    per_page = lambda layers: layers * 2 * (32 + 32) * 2 * page
+    budget = 3_000_000
+    got = CacheManager.pages_that_fit(needs, torch.bfloat16, page, 2 * budget, 0.5, requests, seq, step)
+    assert got[1] == requests * -(-(40 + step + page) // page) == 28
+    assert got[0] == (budget - got[1] * per_page(1)) // per_page(2)
+    assert got[0] * per_page(2) + got[1] * per_page(1) <= budget < (got[0] + 1) * per_page(2) + got[1] * per_page(1)
+    # with memory to spare nobody gets more than the requests can fill; with next to none, one page each
+    assert CacheManager.pages_that_fit(needs, torch.bfloat16, page, 1 << 40, 0.9, requests, seq, step) == [requests * seq // page, 28]
+    assert CacheManager.pages_that_fit(needs, torch.bfloat16, page, 1000, 0.9, requests, seq, step) == [1, 1]
+    # without the step's size a portion may be a whole sequence: no less than the other group then
+    assert CacheManager.pages_that_fit(needs, torch.bfloat16, page, 1 << 40, 0.9, requests, seq) == [requests * seq // page] * 2
+    core = HostCore([(page, got[0], 0), (page, got[1], 40)], requests, step * requests, step, seq)
+    slots = [core.acquire_slot() for _ in range(requests)]
+    rng = random.Random(3)
+    at = [0] * requests
+    for _ in range(200):
+        for s in slots:
+            n = rng.randint(1, step)
+            assert core.ensure(s, at[s], n), "the windowed group ran out although sized for the worst case"
+            at[s] += n
+            assert core.pages_held(s, 1) <= got[1] // requests
+        if max(at) + step > got[0] // requests * page:
+            break
+    check_invariants(core, slots)
