@@ -349,7 +349,7 @@ def run_long(args) -> dict:
         points[key] = round(batch / s, 1)
         fractions[key] = round((weight_bytes + batch * (ctx + warmup + steps // 2) * per_token) / s / PEAK_HBM, 4)
         print(f"[bench] {key}: {s * 1e3:.3f} ms/step, {fractions[key] * 100:.1f}% of the HBM roofline (with filling the caches: "
-              f"{time.time() - t0:.0f} s)", file=sys.stderr, flush=True)
+              f"{time.time() - t0:.1f} s)", file=sys.stderr, flush=True)
     args.steps, args.warmup = steps, warmup
     return long_line(args, b.config.num_hidden_layers, points, fractions, first_s)
 

@@ -71,6 +71,7 @@ __device__ __forceinline__ float other_half(float x) {
 // Keys outside [lo, pos] are masked; that pass is skipped (edge false, the same in all lanes)
 // for tiles that lie wholly inside every column's range.
 #define SOFTMAX_SLACK 8.0f
+#define ATTN_WIDE_FROM_KEYS 32768        // tiles of eight waves from this bound on the step's lengths
 __device__ __forceinline__ bool softmax_tile(f32x16& S, float& m, float& l, int t0, int pos, int lo,
                                              int h, float c, float& alpha, bool edge) {
     if (edge) {
@@ -273,8 +274,8 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const bf16* __restrict_
 // (swz: kk for 256-byte rows and longer, kk >> 1 for 128-byte rows): the 16 lanes of an operand
 // read want one chunk of 16 different keys and then hit 16 different bank groups.  Values are
 // [HD][16] per page and are read in lane order; they need no swizzle.
-template <int HD>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attn_tiles_lds_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
+template <int HD, int WAVES = 4>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attn_tiles_lds_kernel(const bf16* __restrict__ q, bf16* __restrict__ out,
                                                              const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                                                              const int* __restrict__ block_table,
                                                              const int* __restrict__ positions,
@@ -285,7 +286,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     constexpr int ROW_BYTES = HD * 2;
     constexpr int PAGE_BYTES = 16 * ROW_BYTES;      // a page of one kv head: keys [16][HD], values [HD][16]
     constexpr int TILE_BYTES = 2 * PAGE_BYTES;      // a tile's keys, or its values: two pages
-    constexpr int HALF = PAGE_BYTES / 2048;         // load instructions of a wave for its half page
+    static_assert(WAVES == 4 || WAVES == 8, "four waves, or eight for long caches");
+    constexpr int SHARE = PAGE_BYTES / (WAVES / 2); // bytes of a page that one wave brings: two pages, WAVES / 2 waves each
+    static_assert(SHARE >= 1024 && SHARE % 1024 == 0, "a load instruction of a wave brings 1 KB");
+    constexpr int HALF = SHARE / 1024;              // load instructions of a wave for its share of a page
     constexpr int SWZ_SHIFT = ROW_BYTES >= 256 ? 0 : 1;
     constexpr int R = (8 * TILE_BYTES <= 65536) ? 4 : 2;   // tiles in each of the two rings (keys, values)
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * R * TILE_BYTES];
@@ -297,18 +301,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     // from the last to the first: the longest start first, they decide when the grid ends.  All
     // blocks of the first two rounds (a round: as many blocks as the device holds at once in one
     // layer, `round_blocks`) are resident together, the second round beside the first on the same
-    // units, so the second round runs in the opposite order and puts the shortest beside the longest.
-    int n_btiles = count_tiles(q_starts, n_entries, 4 * tpt, skip_single);      // (every wave for itself: the same figures)
+    // units, so the second round runs in the opposite order and puts the shortest beside the longest
+    // (`round_blocks` 0, for blocks that have a unit to themselves: from the last to the first throughout).
+    int n_btiles = count_tiles(q_starts, n_entries, WAVES * tpt, skip_single);      // (every wave for itself: the same figures)
     int g = blockIdx.x / a.n_kv_heads;
     if (g >= n_btiles) return;                       // the grid is sized for the most tiles the tokens could make
     int gr = round_blocks / a.n_kv_heads;
     if (g >= gr && g < 2 * gr) g = gr + (min(2 * gr, n_btiles) - 1 - g);
-    int btile = n_btiles - 1 - g;                    // 4 * tpt tokens of one entry
+    int btile = n_btiles - 1 - g;                    // WAVES * tpt tokens of one entry
     int e = 0, rem = 0;
-    if (!locate_tile(q_starts, n_entries, 4 * tpt, skip_single, btile, e, rem)) return;
+    if (!locate_tile(q_starts, n_entries, WAVES * tpt, skip_single, btile, e, rem)) return;
     int e_end = q_starts[e + 1];
-    int btok0 = q_starts[e] + rem * 4 * tpt;
-    int btok_last = min(btok0 + 4 * tpt, e_end) - 1;
+    int btok0 = q_starts[e] + rem * WAVES * tpt;
+    int btok_last = min(btok0 + WAVES * tpt, e_end) - 1;
     // this wave's tokens (it may have none, at the end of an entry: it still helps to load)
     int tok0 = btok0 + wave * tpt;
     int ntok = max(0, min(tpt, e_end - tok0));
@@ -340,18 +345,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 128 ?
     float m = -INFINITY, l = 0.0f;
     float scale_log2e = a.scale * 1.44269504088896341f;
 
-    // ---- loads.  A tile's keys are two pages and so are its values; each wave brings half a page
-    // of both (page wave & 1, half wave >> 1).  What a lane fetches for its place in the page's
+    // ---- loads.  A tile's keys are two pages and so are its values; each wave brings its share of a
+    // page of both (page wave & 1, share wave >> 1: half a page with four waves, a quarter with eight).  What a lane fetches for its place in the page's
     // LDS image does not change from tile to tile:
     unsigned goff_k[HALF], goff_v[HALF];
 #pragma unroll
     for (int i = 0; i < HALF; ++i) {
-        int off = (wave >> 1) * (PAGE_BYTES / 2) + i * 1024 + lane * 16;
+        int off = (wave >> 1) * SHARE + i * 1024 + lane * 16;
         int krow = off / ROW_BYTES, slot = (off % ROW_BYTES) / 16;
         goff_k[i] = krow * ROW_BYTES + ((slot ^ ((krow >> SWZ_SHIFT) & (CHUNKS - 1) & 15)) * 16);   // keys: the chunk that belongs in this slot
         goff_v[i] = off;
     }
-    unsigned lds_part = (wave & 1) * PAGE_BYTES + (wave >> 1) * (PAGE_BYTES / 2);   // this wave's part of a tile's image
+    unsigned lds_part = (wave & 1) * PAGE_BYTES + (wave >> 1) * SHARE;   // this wave's part of a tile's image
     const unsigned char* k_base = (const unsigned char*)(kc + (size_t)kvh * (16 * HD));
     const unsigned char* v_base = (const unsigned char*)(vc + (size_t)kvh * (16 * HD));
     size_t page_stride = (size_t)a.n_kv_heads * (16 * HD) * sizeof(bf16);
@@ -1061,9 +1066,23 @@ static int launch(hipStream_t stream, const bf16* q, bf16* out, const bf16* kc, 
     }
     if (!only_single) {
         if constexpr (HD == 64 || HD == 128 || HD == 256) {
-            int btiles = a.n_tokens / (4 * tpt) + n_entries;
-            attn_tiles_lds_kernel<HD><<<btiles * a.n_kv_heads, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
-                                                                                 n_entries, a, G, tpt, split, llmrs_compute_units());
+            // Over long caches blocks of eight waves, one to a unit: every tile of keys and values comes in for
+            // twice the columns (a portion of 2048 tokens of the 8B shape over 32,768 / 65,536 / 131,072 keys:
+            // 856 -> 893, 877 -> 934, 883 -> 947 TFLOP/s; over 8,192 keys 4 % slower, over 2,048 a quarter: the
+            // blocks' lengths then differ too much for one block to a unit).
+            bool wide = false;
+            if constexpr (HD == 128) wide = max_seq_len >= ATTN_WIDE_FROM_KEYS;     // (head size 256 has no registers for two waves a SIMD)
+            if (wide) {
+                if constexpr (HD == 128) {
+                    int btiles = a.n_tokens / (8 * tpt) + n_entries;
+                    attn_tiles_lds_kernel<HD, 8><<<btiles * a.n_kv_heads, 512, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
+                                                                                        n_entries, a, G, tpt, split, 0);
+                }
+            } else {
+                int btiles = a.n_tokens / (4 * tpt) + n_entries;
+                attn_tiles_lds_kernel<HD><<<btiles * a.n_kv_heads, 256, 0, stream>>>(q, out, kc, vc, table, positions, q_starts,
+                                                                                     n_entries, a, G, tpt, split, llmrs_compute_units());
+            }
         } else {
             int tiles = a.n_tokens / tpt + n_entries;
             int blocks = ((tiles + 3) / 4) * a.n_kv_heads;

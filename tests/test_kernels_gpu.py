@@ -382,6 +382,50 @@ def test_attention_at_131008_keys():
         assert (got[0].float() - ref).abs().max() <= 4e-3 + 2e-2 * float(ref.abs().max()), f"random query {i}"
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,window", [(8, 2, 128, 0), (6, 2, 128, 20000), (16, 2, 128, 0)])
+def test_attention_prompt_portions_over_long_caches(n_heads, n_kv, hd, window):
+    """Prompt portions against caches of 33,000 and 40,000 keys in bfloat16: from 32,768 keys on the tiles' blocks
+    have eight waves at head size 128 (with 4, 3 and 8 heads to a kv head here: 64, 80 and 32 tokens a block), and a column's sums
+    must be the four-wave blocks' bit for bit.  Portions that end inside a block and one that is a single block's
+    worth; every query of the first request matches one key strongly (the first and last it may see, the edges of
+    pages and of the 32-key tiles, its own position), so its output must be that key's value; random queries agree
+    with the plain formula; and the same portions under a bound below 32,768 keys (the four-wave blocks) give the
+    same bits."""
+    lens = [33000, 40000, 50]
+    case = PagedCase(torch.bfloat16, lens, n_heads, n_kv, hd, 16, seed=41)
+    G = n_heads // n_kv
+    g = torch.Generator().manual_seed(6)
+    counts = [150, 64, 7]
+    q_pos = [list(range(n - c, n)) for n, c in zip(lens, counts)]
+    qs = [torch.randn((c, n_heads, hd), generator=g).to(torch.bfloat16) for c in counts]
+    fars = []
+    for i, p in enumerate(q_pos[0]):
+        lo = max(0, p + 1 - window) if window else 0
+        far = (lo, lo + 1, p, p - 1, 31, 32, 16383, 16384, 32767, 32768, (lo + p) // 2, lo + 15, lo + 16)[i % 13]
+        far = min(max(far, lo), p)
+        fars.append(far)
+        qs[0][i] = (case.k[0][far].float().repeat_interleave(G, dim=0) * 8.0).to(torch.bfloat16)
+    got = case.run(qs, q_pos, window=window, n_single=0)
+    at = 0
+    for r, p in enumerate(q_pos):
+        rows = got[at:at + len(p)].float()
+        at += len(p)
+        pick = range(0, len(p), 2) if r == 0 else (0, len(p) // 2, len(p) - 1)      # (every kind of far key: 2 and 13 share no factor)
+        for i in pick:
+            ref = case.reference(r, qs[r][i:i + 1], [p[i]], window=window)[0].float()
+            if r == 0:
+                want = case.v[0][fars[i]].float().repeat_interleave(G, dim=0)
+                assert (ref - want).abs().max() < 0.05, "the case itself: softmax must be peaked on the far key"
+            assert (rows[i] - ref).abs().max() <= 4e-3 + 2e-2 * float(ref.abs().max()), (r, i)
+    # a request of 40,000 keys under a bound of 32,000 would be a caller's mistake, so the four-wave blocks are
+    # asked for through the two requests that such a bound fits: the first, cut to 32,000 keys, and the third
+    short = [list(range(32000 - 150, 32000)), [], q_pos[2]]
+    qs_short = [qs[0], qs[1][:0], qs[2]]
+    four = case.run(qs_short, short, window=window, n_single=0, bound=32000)
+    eight = case.run(qs_short, short, window=window, n_single=0, bound=32768)
+    assert torch.equal(four, eight), "a column's sums do not depend on how many waves share its keys"
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", [(8, 2, 128, 16, 0), (3, 3, 64, 8, 0), (6, 2, 96, 16, 300), (32, 1, 32, 4, 0),
                                                         (4, 4, 160, 16, 130), (16, 2, 256, 32, 0)])
 def test_attention_float32_decoding_requests(n_heads, n_kv, hd, ps, window):
