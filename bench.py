@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long]
+    python bench.py --gpus 1 --steps K --warmup W [--workload decode8b|serve1b|mixed70b|sizes|sizes1b|prompts|long|widths|portions]
 
 The default run (`decode8b`) is the Llama-3.1-8B shape with random bfloat16 weights: 8
 requests, each with 2,048 tokens of context in the cache, decode K steps through the
@@ -31,6 +31,8 @@ The other workloads print one line of the same form each:
             were timed on (hidden 1536 to 6144, odd intermediates), at 1, 8, 64, 256 and 2048 rows: GB/s of weights or
             TFLOP/s for each, so that a width that falls into a poor choice shows; value = the worst share of the best
             share seen at the same number of rows.
+  portions  the attention of one request's prompt portion of 2,048 tokens alone (8B shape's heads), over caches of
+            2,048 (the whole prompt: causal) to 131,072 keys: TFLOP/s for each; value = the one over 65,536 keys.
 With LLM_PERF set in the environment every kernel call is timed by itself and a table
 by kernel goes to stderr (the reference's switch, src/backend/metal/mod.rs:235,321-400).
 """
@@ -61,7 +63,7 @@ LLAMA_8B = _llama(32, 4096, 32, 8, 128, 14336, 8.0, False)
 LLAMA_1B = _llama(16, 2048, 32, 8, 64, 8192, 32.0, True)
 LLAMA_70B = _llama(80, 8192, 64, 8, 128, 28672, 8.0, False)
 SHAPES = {"Llama-3.1-8B shape": LLAMA_8B, "Llama-3.2-1B shape": LLAMA_1B, "Llama-3.1-70B shape": LLAMA_70B}
-WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths")
+WORKLOADS = ("decode8b", "serve1b", "mixed70b", "sizes", "sizes1b", "prompts", "long", "widths", "portions")
 
 
 def flat_config(model: str, layers_run: int, global_batch: int, seq_len: int, page_size: int, **more) -> dict:
@@ -485,6 +487,56 @@ def run_widths(args) -> dict:
     return line
 
 
+def run_portions(args) -> dict:
+    """The attention kernel for entries with several tokens, by itself: a portion of 2,048 tokens of one request whose
+    cache holds `keys` keys (the portion's own among them), heads and head size of the 8B shape, pages in order."""
+    import torch
+    from llm_rs_amd.kernels import kernels
+    k, dev = kernels(), "cuda:0"
+    H, KV, HD, PS, T = LLAMA_8B["num_attention_heads"], LLAMA_8B["num_key_value_heads"], LLAMA_8B["head_dim"], 16, 2048
+    points, fractions, first_s = {}, {}, 0.0
+    for keys in (2048, 8192, 16384, 32768, 65536, 131072):
+        pages = keys // PS
+        kc = torch.randn(pages * KV * PS * HD, device=dev).to(torch.bfloat16)
+        vc = torch.randn(pages * KV * PS * HD, device=dev).to(torch.bfloat16)
+        q = torch.randn(T, H * HD, device=dev).to(torch.bfloat16)
+        out = torch.empty_like(q)
+        table = torch.arange(pages, dtype=torch.int32, device=dev).reshape(1, pages)
+        entry = torch.zeros(T, dtype=torch.int32, device=dev)
+        positions = torch.arange(keys - T, keys, dtype=torch.int32, device=dev)
+        q_starts = torch.tensor([0, T], dtype=torch.int32, device=dev)
+        seq_lens = torch.tensor([keys], dtype=torch.int32, device=dev)
+
+        def call():
+            k.attention(q, out, kc, vc, table, entry, positions, q_starts, seq_lens, H, KV, HD, PS, pages, 0, HD ** -0.5, None, keys, 0)
+
+        for _ in range(2 if points else 20):            # (the first calls of the process also see the clocks rise)
+            call()
+        torch.cuda.synchronize()
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            call()
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / reps
+        flops = 4.0 * H * HD * (T * keys - T * (T - 1) / 2)           # two products, each query over the keys it may see
+        if keys == 65536:
+            first_s = sec
+        points[f"attention_{keys}"] = round(flops / sec / 1e12, 1)
+        fractions[f"attention_{keys}"] = round(flops / sec / PEAK_FLOPS["bfloat16"], 4)
+        print(f"[bench] portion of {T} tokens over {keys} keys: {sec * 1e6:9.1f} us  {flops / sec / 1e12:6.0f} TFLOP/s", file=sys.stderr, flush=True)
+        del kc, vc
+    first = "attention_65536"
+    line = base_line("TFLOP/s of the attention of a 2,048-token prompt portion alone (8B shape's heads) over caches of 2,048 to 131,072 keys; "
+                     "value: over 65,536", points[first], reps, 2, first_s, "bfloat16",
+                     {"model": "Llama-3.1-8B shape (attention only)", "global_batch": 1, "seq_len": 65536, "parallelism": "single GPU",
+                      "num_attention_heads": H, "num_key_value_heads": KV, "head_dim": HD, "page_size": PS, "portion_tokens": T})
+    line["unit"] = "TFLOP/s"
+    line["points"] = points
+    line["peak_frac"] = fractions
+    return line
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -510,7 +562,7 @@ def main() -> int:
     args.steps = args.steps if args.steps is not None else (8 if heavy else 64)
     args.warmup = args.warmup if args.warmup is not None else (2 if heavy else 8)
     line = {"decode8b": run_decode8b, "serve1b": run_serve1b, "mixed70b": run_mixed70b, "sizes": run_sizes, "sizes1b": run_sizes,
-            "prompts": run_prompts, "long": run_long, "widths": run_widths}[args.workload](args)
+            "prompts": run_prompts, "long": run_long, "widths": run_widths, "portions": run_portions}[args.workload](args)
     from llm_rs_amd.kernels import kernels
     if kernels().times is not None:         # LLM_PERF: what was still to be shown of the per-kernel table
         kernels().times.dump()
